@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Headline benchmark: prefill dispatch + combine on one MI355X.
+
+A step is one pass of the hot path over one synthetic batch at the prefill shape
+(T=4096, H=7168, 256 experts, top-8 with Zipf(1.2) popularity, seed 0):
+  layout (counts / prefix / stable permutation, with the host read-back of R that a fresh dispatch
+  needs) -> FP8 e4m3 dispatch with the per-128 quantiser fused into the expand-permute ->
+  combine of BF16 gradients N(0,1) [R,H] (the backward of dispatch).
+`value` is the algorithmic HBM bytes of dispatch + combine per second of wall time of that step.
+Prints ONE JSON line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(tokens, hidden, topk, rows):
+    """Bytes each kernel must move (no padding, no re-reads)."""
+    idx = tokens * topk * 8
+    dispatch = tokens * hidden * 2 + tokens * topk * 4 + rows * hidden + rows * (hidden // 128) * 4 + rows * 4
+    combine = rows * hidden * 2 + tokens * topk * 4 + tokens * hidden * 2
+    layout = idx + 2 * tokens * topk * 4
+    return dict(layout=layout, dispatch=dispatch, combine=combine)
+
+
+def time_kernel(fn, iters, torch):
+    """Average device time of `fn` in microseconds, HIP events on the stream the kernels run on."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1000.0 / iters
+
+
+def cpu_baseline(x, idx, w, grads, cfg, nbytes):
+    """The reference CPU path (torch CPU, all host threads) on the same inputs."""
+    import torch
+
+    from oracle import baseline
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    tokens = min(cfg["tokens"], 1024)  # bounded sample: the first 1024 tokens of the same batch
+    xs, ids, ws = x[:tokens], idx[:tokens], w[:tokens]
+
+    def step():
+        counts, psum, r2row, r2route = baseline.layout(ids, cfg["experts"])
+        baseline.dispatch_fp8(xs, ws, r2route, cfg["topk"])
+        baseline.combine(grads[: r2route.numel()], r2row)
+        return r2route.numel()
+
+    rows = step()
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter_ns()
+        step()
+        times.append((time.perf_counter_ns() - t0) / 1e9)
+    mean = sum(times) / len(times)
+    sample_bytes = algorithmic_bytes(tokens, cfg["hidden"], cfg["topk"], rows)
+    moved = sample_bytes["dispatch"] + sample_bytes["combine"]
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return dict(
+        value=moved / mean / 1e9,
+        unit="GB/s",
+        cores=cores,
+        kind="port",
+        sample=f"first {tokens} tokens of the same batch ({rows} rows), 1 warm-up + 5 timed passes, "
+        f"mean {mean * 1e3:.1f} ms per pass, torch CPU {torch.get_num_threads()} threads, {model}",
+    )
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--kernel-iters", type=int, default=50)
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share; --gpus must be 1 (no multi-GPU path in this build)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from deepep_amd import ops
+    from oracle import cases
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    x, idx, w, cfg = cases.make_inputs("C3", seed=0)
+    tokens, hidden, topk, experts = cfg["tokens"], cfg["hidden"], cfg["topk"], cfg["experts"]
+    rows_expected = tokens * topk
+    grads = torch.randn(rows_expected, hidden, generator=torch.Generator().manual_seed(1)).bfloat16()
+    xd, idxd, wd, gd = x.to(dev), idx.to(dev), w.to(dev), grads.to(dev)
+    ws = ops.Workspace(max(ops.layout_workspace_bytes(tokens, topk, experts), 1 << 20))
+
+    def step():
+        lay = ops.layout(ws, idxd, experts)
+        rows = int(lay["num_rows"].item())  # the read-back a fresh dispatch needs to size its outputs
+        recv = ops.dispatch_quant_fp8(xd, wd, lay["route_to_row"], lay["row_to_route"], rows)
+        out = ops.combine(gd[:rows], lay["route_to_row"])
+        return rows, recv, out
+
+    for _ in range(args.warmup):
+        rows, _, _ = step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        rows, _, _ = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    nbytes = algorithmic_bytes(tokens, hidden, topk, rows)
+    moved = nbytes["dispatch"] + nbytes["combine"]
+
+    # Per-kernel device time (HIP events on the launch stream), same inputs.
+    lay = ops.layout(ws, idxd, experts)
+    r2row, r2route = lay["route_to_row"], lay["row_to_route"]
+    grows = gd[:rows]
+    out_buf = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    it = args.kernel_iters
+    recv_w = ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows)[2]
+    us = dict(
+        layout=time_kernel(lambda: ops.layout(ws, idxd, experts), it, torch),
+        dispatch_fp8_quant=time_kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), it, torch),
+        dispatch_bf16=time_kernel(lambda: ops.dispatch_copy(xd, None, wd, r2row, r2route, rows), it, torch),
+        combine=time_kernel(lambda: ops.combine(grows, r2row, out=out_buf), it, torch),
+        combine_weighted=time_kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), it, torch),
+    )
+    bf16_dispatch_bytes = tokens * hidden * 2 + tokens * topk * 4 + rows * hidden * 2 + rows * 4
+    kernels = {
+        "layout": dict(us=us["layout"], bytes=nbytes["layout"]),
+        "dispatch_fp8_quant": dict(us=us["dispatch_fp8_quant"], bytes=nbytes["dispatch"]),
+        "dispatch_bf16": dict(us=us["dispatch_bf16"], bytes=bf16_dispatch_bytes),
+        "combine": dict(us=us["combine"], bytes=nbytes["combine"]),
+        "combine_weighted": dict(us=us["combine_weighted"], bytes=nbytes["combine"] + rows * 4),
+    }
+    for entry in kernels.values():
+        entry["GBps"] = entry["bytes"] / entry["us"] / 1e3
+        entry["frac_of_8TBps"] = entry["GBps"] / HBM_PEAK_GBS
+
+    dominant = kernels["combine"]
+    result = {
+        "metric": "dispatch+combine HBM GB/s (T=4096,H=7168,k=8)",
+        "value": moved / (ms_per_step * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "prefill: T=4096, H=7168, 256 experts, top-8 Zipf(1.2), seed 0; step = layout (+R read-back) "
+            "+ FP8 e4m3 dispatch with fused per-128 quant + BF16 combine of N(0,1) grads [R,H]",
+            "tokens": tokens,
+            "hidden": hidden,
+            "topk": topk,
+            "experts": experts,
+            "rows": rows,
+            "bytes_per_step": moved,
+        },
+        "roofline": {
+            "kernel": "combine_kernel<false>",
+            "bound": "hbm",
+            "achieved": dominant["GBps"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": dominant["GBps"] / HBM_PEAK_GBS,
+            "traffic": None,
+        },
+        "kernels": kernels,
+        "dispatch_plus_combine_us": us["dispatch_fp8_quant"] + us["combine"],
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(x, idx, w, grads, cfg, nbytes)
+    ws.destroy()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,113 @@
+// Combine: every token gathers its expert rows and reduces them in fp32, in slot order, with an
+// optional per-row weight, then rounds once to BF16.  A token (column part) is owned by exactly one
+// workgroup, so there are no atomics and the summation order is fixed.
+//
+// Operation order follows the reference's aggregate kernel
+// (csrc/direct/kernels/aggregate/aggregate_impl.h:166-226): acc = +0; per valid slot
+// tmp = float(y); tmp = tmp * w; acc = acc + tmp (separate multiply and add); final cast RNE.
+// Unweighted form: tests/elastic/test_combine.py:504-515; weighted form:
+// tests/elastic/test_ep_low_latency.py:449-463; weight-return channel: docs/elastic.md:71.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+namespace dpep {
+namespace {
+
+constexpr int kMaxThreads = 256;
+constexpr int kBatch = 8;  // rows fetched per thread before the dependent adds start
+
+template <bool kWeighted>
+__global__ __launch_bounds__(kMaxThreads) void combine_kernel(
+    const u32x4* __restrict__ y, const float* __restrict__ row_weights, const int* __restrict__ route_to_row,
+    int num_topk, int vec_per_row, int vec_per_part, int parts, u32x4* __restrict__ out,
+    const float* __restrict__ return_in, float* __restrict__ return_out)
+{
+    __shared__ int rows[DPEP_MAX_TOPK + kBatch];
+    __shared__ float wts[DPEP_MAX_TOPK + kBatch];
+    const int token = blockIdx.x / parts, part = blockIdx.x % parts;
+    if (threadIdx.x < DPEP_MAX_TOPK + kBatch) {
+        int row = -1;
+        if (threadIdx.x < num_topk) row = route_to_row[static_cast<size_t>(token) * num_topk + threadIdx.x];
+        rows[threadIdx.x] = row;
+        if (kWeighted) wts[threadIdx.x] = row >= 0 ? row_weights[row] : 0.0f;
+        if (part == 0 && return_out != nullptr && threadIdx.x < num_topk)
+            return_out[static_cast<size_t>(token) * num_topk + threadIdx.x] = row >= 0 ? return_in[row] : 0.0f;
+    }
+    __syncthreads();
+    const int v_begin = part * vec_per_part;
+    const int v_end = min(v_begin + vec_per_part, vec_per_row);
+    for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x) {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+        for (int s0 = 0; s0 < num_topk; s0 += kBatch) {
+            u32x4 val[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) {
+                const int row = rows[s0 + j];
+                if (row >= 0) val[j] = load16_nt(y + static_cast<size_t>(row) * vec_per_row + v);
+            }
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) {
+                if (rows[s0 + j] < 0) continue;
+                const float w = kWeighted ? wts[s0 + j] : 1.0f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float lo = bf16_to_f32(val[j][i] & 0xffffu);
+                    float hi = bf16_to_f32(val[j][i] >> 16);
+                    if (kWeighted) {
+                        lo = __fmul_rn(lo, w);
+                        hi = __fmul_rn(hi, w);
+                    }
+                    acc[2 * i] = __fadd_rn(acc[2 * i], lo);
+                    acc[2 * i + 1] = __fadd_rn(acc[2 * i + 1], hi);
+                }
+            }
+        }
+        u32x4 packed;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16(acc[2 * i]) | (f32_to_bf16(acc[2 * i + 1]) << 16);
+        store16_nt(out + static_cast<size_t>(token) * vec_per_row + v, packed);
+    }
+}
+
+}  // namespace
+}  // namespace dpep
+
+extern "C" {
+
+int dpep_combine(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
+                 int num_rows, int hidden, void* out, const float* return_in, float* return_out, void* stream)
+{
+    using namespace dpep;
+    DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "combine: bad T=%d K=%d", num_tokens,
+                 num_topk);
+    DPEP_REQUIRE(num_rows >= 0 && static_cast<long long>(num_rows) <= static_cast<long long>(num_tokens) * num_topk,
+                 "combine: num_rows=%d outside [0, T*K]", num_rows);
+    DPEP_REQUIRE(hidden > 0 && hidden % 8 == 0, "combine: hidden=%d must be a positive multiple of 8", hidden);
+    DPEP_REQUIRE((return_in == nullptr) == (return_out == nullptr), "combine: return_in and return_out go together");
+    if (num_tokens == 0) return DPEP_OK;
+    DPEP_REQUIRE(route_to_row != nullptr && out != nullptr && aligned16(out), "combine: NULL or misaligned buffer");
+    DPEP_REQUIRE(num_rows == 0 || (y != nullptr && aligned16(y)), "combine: y must be 16-byte aligned");
+    const int vec = hidden / 8;
+    int parts = 1;
+    while (num_tokens * parts < 2048 && vec / (parts * 2) >= 64 && parts < 16) parts *= 2;
+    const int per_part = (vec + parts - 1) / parts;
+    parts = (vec + per_part - 1) / per_part;
+    int threads = (per_part + 63) / 64 * 64;
+    if (threads > kMaxThreads) threads = kMaxThreads;
+    if (threads < 64) threads = 64;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (row_weights != nullptr)
+        hipLaunchKernelGGL(combine_kernel<true>, dim3(num_tokens * parts), dim3(threads), 0, s,
+                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, per_part, parts,
+                           static_cast<u32x4*>(out), return_in, return_out);
+    else
+        hipLaunchKernelGGL(combine_kernel<false>, dim3(num_tokens * parts), dim3(threads), 0, s,
+                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, per_part, parts,
+                           static_cast<u32x4*>(out), return_in, return_out);
+    return launch_status("combine");
+}
+
+}  // extern "C"

@@ -1,0 +1,296 @@
+// Expand-permute payload dispatch: out[row(t,s)] = x[t] for every route that owns a row, optionally
+// fused with the per-128-element FP8 e4m3fn block quantiser.  HBM-bound: 16-byte coalesced loads,
+// non-temporal 16-byte stores, each input row read once and written to its K destinations.
+//
+// Observable contract: tests/elastic/test_dispatch.py:1391-1416 (payload, scales and weights arrive
+// bit-exactly in row order), tests/clos/common.py:276-279; quantiser deep_ep/utils/math.py:45-61.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+namespace dpep {
+namespace {
+
+constexpr int kMaxThreads = 256;
+
+// ---- token-major copy: one workgroup per (token, column part); read once, write K times -----------
+__global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
+    const u32x4* __restrict__ x, const float* __restrict__ scales, const float* __restrict__ weights,
+    const int* __restrict__ route_to_row, int num_topk, int vec_per_row, int vec_per_part, int parts, int scale_cols,
+    u32x4* __restrict__ out, float* __restrict__ out_scales, float* __restrict__ out_weights)
+{
+    __shared__ int rows[DPEP_MAX_TOPK];
+    __shared__ int any_valid;
+    const int token = blockIdx.x / parts, part = blockIdx.x % parts;
+    if (threadIdx.x == 0) any_valid = 0;
+    __syncthreads();
+    if (threadIdx.x < num_topk) {
+        const int row = route_to_row[static_cast<size_t>(token) * num_topk + threadIdx.x];
+        rows[threadIdx.x] = row;
+        if (row >= 0) any_valid = 1;
+    }
+    __syncthreads();
+    if (!any_valid) return;
+    const int v_begin = part * vec_per_part;
+    const int v_end = min(v_begin + vec_per_part, vec_per_row);
+    const u32x4* src = x + static_cast<size_t>(token) * vec_per_row;
+    for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x) {
+        const u32x4 value = load16_nt(src + v);
+        for (int s = 0; s < num_topk; ++s) {
+            const int row = rows[s];
+            if (row >= 0) store16_nt(out + static_cast<size_t>(row) * vec_per_row + v, value);
+        }
+    }
+    if (part == 0) {
+        if (scales != nullptr) {
+            for (int c = threadIdx.x; c < scale_cols; c += blockDim.x) {
+                const float value = scales[static_cast<size_t>(token) * scale_cols + c];
+                for (int s = 0; s < num_topk; ++s) {
+                    const int row = rows[s];
+                    if (row >= 0) out_scales[static_cast<size_t>(row) * scale_cols + c] = value;
+                }
+            }
+        }
+        if (weights != nullptr && threadIdx.x < num_topk && rows[threadIdx.x] >= 0)
+            out_weights[rows[threadIdx.x]] = weights[static_cast<size_t>(token) * num_topk + threadIdx.x];
+    }
+}
+
+// ---- row-major copy: one workgroup per (output row, column part); for sparse receive shares -------
+__global__ __launch_bounds__(kMaxThreads) void dispatch_copy_row_kernel(
+    const u32x4* __restrict__ x, const float* __restrict__ scales, const float* __restrict__ weights,
+    const int* __restrict__ row_to_route, int num_topk, int vec_per_row, int vec_per_part, int parts, int scale_cols,
+    u32x4* __restrict__ out, float* __restrict__ out_scales, float* __restrict__ out_weights)
+{
+    const int row = blockIdx.x / parts, part = blockIdx.x % parts;
+    const int route = row_to_route[row];
+    const int token = route / num_topk;
+    const int v_begin = part * vec_per_part;
+    const int v_end = min(v_begin + vec_per_part, vec_per_row);
+    const u32x4* src = x + static_cast<size_t>(token) * vec_per_row;
+    u32x4* dst = out + static_cast<size_t>(row) * vec_per_row;
+    for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x) store16_nt(dst + v, load16(src + v));
+    if (part == 0) {
+        if (scales != nullptr)
+            for (int c = threadIdx.x; c < scale_cols; c += blockDim.x)
+                out_scales[static_cast<size_t>(row) * scale_cols + c] = scales[static_cast<size_t>(token) * scale_cols + c];
+        if (weights != nullptr && threadIdx.x == 0) out_weights[row] = weights[route];
+    }
+}
+
+// ---- per-128 FP8 quantiser ------------------------------------------------------------------------
+// One lane owns 16 consecutive BF16 values (two 16-byte loads), so 8 adjacent lanes own one
+// 128-element block.  amax is reduced over those 8 lanes with DPP-free xor shuffles inside the wave.
+struct Quant16 {
+    u32x4 codes;  // 16 e4m3fn bytes
+    float scale;  // amax / 448
+};
+
+__device__ __forceinline__ float max8(float v)
+{
+    v = fmaxf(v, __shfl_xor(v, 1));
+    v = fmaxf(v, __shfl_xor(v, 2));
+    v = fmaxf(v, __shfl_xor(v, 4));
+    return v;
+}
+
+// fp32 -> e4m3fn byte pair, round-to-nearest-even, on the gfx950 converter (OCP FP8).
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d)
+{
+    int packed = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    packed = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, packed, true);
+    return static_cast<uint32_t>(packed);
+}
+
+__device__ __forceinline__ Quant16 quantize16(u32x4 lo, u32x4 hi)
+{
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = bf16_to_f32(lo[i] & 0xffffu);
+        v[2 * i + 1] = bf16_to_f32(lo[i] >> 16);
+        v[8 + 2 * i] = bf16_to_f32(hi[i] & 0xffffu);
+        v[8 + 2 * i + 1] = bf16_to_f32(hi[i] >> 16);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    amax = fmaxf(max8(amax), 1e-4f);
+    // The reference writes 448.0 / amax, which torch evaluates as reciprocal(amax) * 448:
+    // two correctly rounded fp32 operations, reproduced here.
+    const float inv = __fmul_rn(__fdiv_rn(1.0f, amax), 448.0f);
+    Quant16 q;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        q.codes[i] = pack4_e4m3(__fmul_rn(v[4 * i], inv), __fmul_rn(v[4 * i + 1], inv), __fmul_rn(v[4 * i + 2], inv),
+                                __fmul_rn(v[4 * i + 3], inv));
+    q.scale = __fdiv_rn(amax, 448.0f);
+    return q;
+}
+
+// token-major: one workgroup per (token, column part); units = 16-element groups per row (H/16).
+__global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
+    const u32x4* __restrict__ x, const float* __restrict__ weights, const int* __restrict__ route_to_row, int num_topk,
+    int units_per_row, int units_per_part, int parts, u32x4* __restrict__ out, float* __restrict__ out_scales,
+    float* __restrict__ out_weights)
+{
+    __shared__ int rows[DPEP_MAX_TOPK];
+    __shared__ int any_valid;
+    const int token = blockIdx.x / parts, part = blockIdx.x % parts;
+    if (threadIdx.x == 0) any_valid = 0;
+    __syncthreads();
+    if (threadIdx.x < num_topk) {
+        const int row = route_to_row[static_cast<size_t>(token) * num_topk + threadIdx.x];
+        rows[threadIdx.x] = row;
+        if (row >= 0) any_valid = 1;
+    }
+    __syncthreads();
+    if (!any_valid) return;
+    const int u_begin = part * units_per_part;
+    const int u_end = min(u_begin + units_per_part, units_per_row);
+    const int scale_cols = units_per_row / 8;
+    const u32x4* src = x + static_cast<size_t>(token) * units_per_row * 2;
+    // units_per_part is a multiple of 8 and blockDim of 64, so the 8 lanes of a block stay together.
+    for (int u = u_begin + threadIdx.x; u < u_end; u += blockDim.x) {
+        const Quant16 q = quantize16(load16_nt(src + 2 * u), load16_nt(src + 2 * u + 1));
+        for (int s = 0; s < num_topk; ++s) {
+            const int row = rows[s];
+            if (row < 0) continue;
+            store16_nt(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
+            if ((u & 7) == 0) out_scales[static_cast<size_t>(row) * scale_cols + (u >> 3)] = q.scale;
+        }
+    }
+    if (part == 0 && weights != nullptr && threadIdx.x < num_topk && rows[threadIdx.x] >= 0)
+        out_weights[rows[threadIdx.x]] = weights[static_cast<size_t>(token) * num_topk + threadIdx.x];
+}
+
+// row-major: one workgroup per (output row, column part); row_to_route == nullptr means identity
+// (row == token), which is the stand-alone quantiser.
+__global__ __launch_bounds__(kMaxThreads) void dispatch_quant_row_kernel(
+    const u32x4* __restrict__ x, const float* __restrict__ weights, const int* __restrict__ row_to_route, int num_topk,
+    int units_per_row, int units_per_part, int parts, u32x4* __restrict__ out, float* __restrict__ out_scales,
+    float* __restrict__ out_weights)
+{
+    const int row = blockIdx.x / parts, part = blockIdx.x % parts;
+    const int route = row_to_route != nullptr ? row_to_route[row] : row;
+    const int token = row_to_route != nullptr ? route / num_topk : row;
+    const int u_begin = part * units_per_part;
+    const int u_end = min(u_begin + units_per_part, units_per_row);
+    const int scale_cols = units_per_row / 8;
+    const u32x4* src = x + static_cast<size_t>(token) * units_per_row * 2;
+    for (int u = u_begin + threadIdx.x; u < u_end; u += blockDim.x) {
+        const Quant16 q = quantize16(load16(src + 2 * u), load16(src + 2 * u + 1));
+        store16_nt(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
+        if ((u & 7) == 0) out_scales[static_cast<size_t>(row) * scale_cols + (u >> 3)] = q.scale;
+    }
+    if (part == 0 && weights != nullptr && threadIdx.x == 0) out_weights[row] = weights[route];
+}
+
+// Split a row of `units` work items over `parts` workgroups so that a launch of `rows` rows has
+// enough workgroups to fill 256 CUs; each part is a multiple of `granule` units.
+struct Split {
+    int parts, per_part, threads;
+};
+
+Split choose_split(int rows, int units, int granule)
+{
+    Split s;
+    const int target_blocks = 2048;
+    int parts = 1;
+    while (rows * parts < target_blocks && units / (parts * 2) >= 64 && parts < 16) parts *= 2;
+    int per_part = (units + parts - 1) / parts;
+    per_part = (per_part + granule - 1) / granule * granule;
+    s.parts = (units + per_part - 1) / per_part;
+    s.per_part = per_part;
+    int threads = (per_part + 63) / 64 * 64;
+    s.threads = threads > kMaxThreads ? kMaxThreads : threads;
+    return s;
+}
+
+int check_common(const char* what, int num_tokens, int num_topk, int num_rows, const int32_t* route_to_row,
+                 const int32_t* row_to_route)
+{
+    DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "%s: bad T=%d K=%d", what, num_tokens,
+                 num_topk);
+    DPEP_REQUIRE(num_rows >= 0 && static_cast<long long>(num_rows) <= static_cast<long long>(num_tokens) * num_topk,
+                 "%s: num_rows=%d outside [0, T*K]", what, num_rows);
+    DPEP_REQUIRE(num_rows == 0 || (route_to_row != nullptr && row_to_route != nullptr), "%s: NULL routing maps", what);
+    return DPEP_OK;
+}
+
+}  // namespace
+}  // namespace dpep
+
+extern "C" {
+
+int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_weights, const int32_t* route_to_row,
+                       const int32_t* row_to_route, int num_tokens, int num_topk, int num_rows, int row_bytes,
+                       int scale_cols, void* out, float* out_scales, float* out_weights, void* stream)
+{
+    using namespace dpep;
+    if (int rc = check_common("dispatch_copy", num_tokens, num_topk, num_rows, route_to_row, row_to_route)) return rc;
+    DPEP_REQUIRE(row_bytes > 0 && row_bytes % 16 == 0, "dispatch_copy: row_bytes=%d must be a positive multiple of 16",
+                 row_bytes);
+    DPEP_REQUIRE((scales == nullptr) == (out_scales == nullptr), "dispatch_copy: scales and out_scales go together");
+    DPEP_REQUIRE(scales == nullptr || scale_cols > 0, "dispatch_copy: scale_cols must be positive with scales");
+    DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "dispatch_copy: weights and out_weights go together");
+    if (num_rows == 0) return DPEP_OK;
+    DPEP_REQUIRE(x != nullptr && out != nullptr && aligned16(x) && aligned16(out), "dispatch_copy: x/out must be 16-byte aligned");
+    const int vec = row_bytes / 16;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (num_rows > num_tokens) {
+        const Split sp = choose_split(num_tokens, vec, 1);
+        hipLaunchKernelGGL(dispatch_copy_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
+                           static_cast<const u32x4*>(x), scales, topk_weights, route_to_row, num_topk, vec, sp.per_part,
+                           sp.parts, scale_cols, static_cast<u32x4*>(out), out_scales, out_weights);
+        return launch_status("dispatch_copy_token");
+    }
+    const Split sp = choose_split(num_rows, vec, 1);
+    hipLaunchKernelGGL(dispatch_copy_row_kernel, dim3(num_rows * sp.parts), dim3(sp.threads), 0, s,
+                       static_cast<const u32x4*>(x), scales, topk_weights, row_to_route, num_topk, vec, sp.per_part,
+                       sp.parts, scale_cols, static_cast<u32x4*>(out), out_scales, out_weights);
+    return launch_status("dispatch_copy_row");
+}
+
+int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int32_t* route_to_row,
+                            const int32_t* row_to_route, int num_tokens, int num_topk, int num_rows, int hidden,
+                            void* out, float* out_scales, float* out_weights, void* stream)
+{
+    using namespace dpep;
+    if (int rc = check_common("dispatch_quant_fp8", num_tokens, num_topk, num_rows, route_to_row, row_to_route)) return rc;
+    DPEP_REQUIRE(hidden > 0 && hidden % 128 == 0, "dispatch_quant_fp8: hidden=%d must be a positive multiple of 128", hidden);
+    DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "dispatch_quant_fp8: weights and out_weights go together");
+    if (num_rows == 0) return DPEP_OK;
+    DPEP_REQUIRE(x && out && out_scales && aligned16(x) && aligned16(out), "dispatch_quant_fp8: x/out must be 16-byte aligned");
+    const int units = hidden / 16;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (num_rows > num_tokens) {
+        const Split sp = choose_split(num_tokens, units, 8);
+        hipLaunchKernelGGL(dispatch_quant_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
+                           static_cast<const u32x4*>(x), topk_weights, route_to_row, num_topk, units, sp.per_part,
+                           sp.parts, static_cast<u32x4*>(out), out_scales, out_weights);
+        return launch_status("dispatch_quant_token");
+    }
+    const Split sp = choose_split(num_rows, units, 8);
+    hipLaunchKernelGGL(dispatch_quant_row_kernel, dim3(num_rows * sp.parts), dim3(sp.threads), 0, s,
+                       static_cast<const u32x4*>(x), topk_weights, row_to_route, num_topk, units, sp.per_part, sp.parts,
+                       static_cast<u32x4*>(out), out_scales, out_weights);
+    return launch_status("dispatch_quant_row");
+}
+
+int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float* out_scales, void* stream)
+{
+    using namespace dpep;
+    DPEP_REQUIRE(num_tokens >= 0, "cast_to_fp8: bad T=%d", num_tokens);
+    DPEP_REQUIRE(hidden > 0 && hidden % 128 == 0, "cast_to_fp8: hidden=%d must be a positive multiple of 128", hidden);
+    if (num_tokens == 0) return DPEP_OK;
+    DPEP_REQUIRE(x && out && out_scales && aligned16(x) && aligned16(out), "cast_to_fp8: x/out must be 16-byte aligned");
+    const int units = hidden / 16;
+    const Split sp = choose_split(num_tokens, units, 8);
+    hipLaunchKernelGGL(dispatch_quant_row_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), nullptr, nullptr, 1, units,
+                       sp.per_part, sp.parts, static_cast<u32x4*>(out), out_scales, nullptr);
+    return launch_status("cast_to_fp8");
+}
+
+}  // extern "C"

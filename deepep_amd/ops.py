@@ -1,0 +1,218 @@
+"""Tensor-level entry points over the C-ABI (the counterpart of ``deep_ep._C`` in the reference,
+csrc/bindings/module.cpp:17-95).
+
+Like the reference's ``pointer()`` helper (csrc/ops/dispatch.cpp:36-49) every tensor is re-validated
+here — device, dtype, contiguity, exact shape — before its address crosses the boundary.  Outputs
+are allocated by the caller's framework (torch), never by the native side.  All calls enqueue on
+torch's current stream and return without synchronising.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require(name, t, dtype, shape=None, device=None):
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"{name} must be a tensor")
+    if t.device.type != "cuda":
+        raise ValueError(f"{name} must live on the GPU (got {t.device})")
+    if device is not None and t.device != device:
+        raise ValueError(f"{name} is on {t.device}, expected {device}")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype} (got {t.dtype})")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)} (got {tuple(t.shape)})")
+    return t
+
+
+class Workspace:
+    """Owner of the native HBM workspace."""
+
+    def __init__(self, num_bytes: int, device: Optional[torch.device] = None):
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        self._lib = _lib.load()
+        handle = ctypes.c_void_p()
+        with torch.cuda.device(self.device):
+            _lib.check(self._lib.dpep_workspace_create(int(num_bytes), ctypes.byref(handle)), "workspace_create")
+        self._handle = handle
+        self.num_bytes = int(num_bytes)
+
+    @property
+    def handle(self):
+        if self._handle is None:
+            raise RuntimeError("workspace was destroyed")
+        return self._handle
+
+    @property
+    def closed(self) -> bool:
+        return self._handle is None
+
+    def destroy(self) -> None:
+        if self._handle is not None:
+            handle, self._handle = self._handle, None
+            with torch.cuda.device(self.device):
+                torch.cuda.synchronize(self.device)
+                _lib.check(self._lib.dpep_workspace_destroy(handle), "workspace_destroy")
+
+
+def layout_workspace_bytes(num_tokens: int, num_topk: int, num_local: int) -> int:
+    return int(_lib.load().dpep_layout_workspace_bytes(num_tokens, num_topk, num_local))
+
+
+def layout(ws: Workspace, topk_idx: torch.Tensor, num_experts: int, expert_begin: int = 0, num_local: Optional[int] = None):
+    """Routing layout on the device.  Returns device tensors; no host synchronisation.
+
+    dict(counts[L], psum[L], offsets[L+1], route_to_row[T,K], row_to_route[T*K] (first R valid), num_rows[1]).
+    """
+    lib = _lib.load()
+    _require("topk_idx", topk_idx, torch.int64, device=ws.device)
+    if topk_idx.ndim != 2:
+        raise ValueError("topk_idx must be [T, K]")
+    tokens, topk = topk_idx.shape
+    num_local = num_experts - expert_begin if num_local is None else num_local
+    dev = topk_idx.device
+    meta = torch.empty(3 * num_local + 2, dtype=torch.int32, device=dev)
+    counts, psum = meta[:num_local], meta[num_local : 2 * num_local]
+    offsets, num_rows = meta[2 * num_local : 3 * num_local + 1], meta[3 * num_local + 1 :]
+    route_to_row = torch.empty((tokens, topk), dtype=torch.int32, device=dev)
+    row_to_route = torch.empty((tokens * topk,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        status = lib.dpep_layout(
+            ws.handle, _ptr(topk_idx), tokens, topk, num_experts, expert_begin, num_local, _ptr(counts), _ptr(psum),
+            _ptr(offsets), _ptr(route_to_row), _ptr(row_to_route), _ptr(num_rows), _stream(dev),
+        )
+    _lib.check(status, "layout")
+    return dict(counts=counts, psum=psum, offsets=offsets, route_to_row=route_to_row, row_to_route=row_to_route,
+                num_rows=num_rows, meta=meta)
+
+
+def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows: int):
+    """out[row] = x[token(row)] (+ scale rows, + per-row weights).  x is BF16 [T,H] or FP8 [T,H]."""
+    lib = _lib.load()
+    if not isinstance(x, torch.Tensor) or x.dtype not in (torch.bfloat16, torch.float8_e4m3fn, torch.float16):
+        raise ValueError("x must be a BF16, FP16 or FP8 E4M3FN tensor")
+    _require("x", x, x.dtype)
+    if x.ndim != 2:
+        raise ValueError("x must be [T, H]")
+    dev = x.device
+    tokens, hidden = x.shape
+    _require("route_to_row", route_to_row, torch.int32, device=dev)
+    topk = route_to_row.shape[1]
+    _require("route_to_row", route_to_row, torch.int32, (tokens, topk), dev)
+    _require("row_to_route", row_to_route, torch.int32, device=dev)
+    row_bytes = hidden * x.element_size()
+    if row_bytes % 16:
+        raise ValueError("hidden row size must be a multiple of 16 bytes")
+    scale_cols = 0
+    out_scales = None
+    if scales is not None:
+        _require("scales", scales, torch.float32, device=dev)
+        if scales.ndim != 2 or scales.shape[0] != tokens:
+            raise ValueError("scales must be [T, C]")
+        scale_cols = scales.shape[1]
+        out_scales = torch.empty((num_rows, scale_cols), dtype=torch.float32, device=dev)
+    out_weights = None
+    if topk_weights is not None:
+        _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)
+        out_weights = torch.empty((num_rows,), dtype=torch.float32, device=dev)
+    out = torch.empty((num_rows, hidden), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        status = lib.dpep_dispatch_copy(
+            _ptr(x), _ptr(scales), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, num_rows,
+            row_bytes, scale_cols, _ptr(out), _ptr(out_scales), _ptr(out_weights), _stream(dev),
+        )
+    _lib.check(status, "dispatch_copy")
+    return out, out_scales, out_weights
+
+
+def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: int):
+    """Fused per-128 FP8 quantisation + expand-permute of BF16 x [T,H]."""
+    lib = _lib.load()
+    _require("x", x, torch.bfloat16)
+    if x.ndim != 2:
+        raise ValueError("x must be [T, H]")
+    dev = x.device
+    tokens, hidden = x.shape
+    if hidden % 128:
+        raise ValueError("hidden must be a multiple of 128 for FP8 dispatch")
+    _require("route_to_row", route_to_row, torch.int32, device=dev)
+    topk = route_to_row.shape[1]
+    _require("route_to_row", route_to_row, torch.int32, (tokens, topk), dev)
+    _require("row_to_route", row_to_route, torch.int32, device=dev)
+    out_weights = None
+    if topk_weights is not None:
+        _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)
+        out_weights = torch.empty((num_rows,), dtype=torch.float32, device=dev)
+    out = torch.empty((num_rows, hidden), dtype=torch.float8_e4m3fn, device=dev)
+    out_scales = torch.empty((num_rows, hidden // 128), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        status = lib.dpep_dispatch_quant_fp8(
+            _ptr(x), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, num_rows, hidden,
+            _ptr(out), _ptr(out_scales), _ptr(out_weights), _stream(dev),
+        )
+    _lib.check(status, "dispatch_quant_fp8")
+    return out, out_scales, out_weights
+
+
+def cast_to_fp8(x):
+    """per_token_cast_to_fp8 on the device: BF16 [T,H] -> (FP8 [T,H], FP32 [T,H/128])."""
+    lib = _lib.load()
+    _require("x", x, torch.bfloat16)
+    if x.ndim != 2 or x.shape[1] % 128:
+        raise ValueError("x must be [T, H] with H a multiple of 128")
+    tokens, hidden = x.shape
+    out = torch.empty((tokens, hidden), dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty((tokens, hidden // 128), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        status = lib.dpep_cast_to_fp8(_ptr(x), tokens, hidden, _ptr(out), _ptr(scales), _stream(x.device))
+    _lib.check(status, "cast_to_fp8")
+    return out, scales
+
+
+def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
+    """out[t] = bf16( sum_s fp32(y[row(t,s)]) (* row_weights[row]) ); optional weight-return channel."""
+    lib = _lib.load()
+    _require("y", y, torch.bfloat16)
+    if y.ndim != 2:
+        raise ValueError("y must be [R, H]")
+    dev = y.device
+    rows, hidden = y.shape
+    if hidden % 8:
+        raise ValueError("hidden must be a multiple of 8")
+    _require("route_to_row", route_to_row, torch.int32, device=dev)
+    if route_to_row.ndim != 2:
+        raise ValueError("route_to_row must be [T, K]")
+    tokens, topk = route_to_row.shape
+    if row_weights is not None:
+        _require("row_weights", row_weights, torch.float32, (rows,), dev)
+    returned = None
+    if return_values is not None:
+        _require("return_values", return_values, torch.float32, (rows,), dev)
+        returned = torch.empty((tokens, topk), dtype=torch.float32, device=dev)
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    else:
+        _require("out", out, torch.bfloat16, (tokens, hidden), dev)
+    with torch.cuda.device(dev):
+        status = lib.dpep_combine(
+            _ptr(y), _ptr(row_weights), _ptr(route_to_row), tokens, topk, rows, hidden, _ptr(out),
+            _ptr(return_values), _ptr(returned), _stream(dev),
+        )
+    _lib.check(status, "combine")
+    return out, returned

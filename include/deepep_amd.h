@@ -1,0 +1,127 @@
+/*
+ * deepep_amd — C ABI of the MI355X (gfx950) dispatch / combine / W4A8-MoE hot path.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a negative DPEP_E* code otherwise, and never throws;
+ *     dpep_last_error() returns a thread-local message for the last failure on this thread;
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); every call only
+ *     enqueues work on that stream and returns without synchronising;
+ *   - output buffers are allocated by the caller; the library owns only the workspace;
+ *   - one call at a time per workspace (the host layer keeps the reference's per-buffer lock).
+ *
+ * Each entry point cites the reference interface it replaces (paths relative to the reference
+ * checkout).
+ */
+#ifndef DEEPEP_AMD_H
+#define DEEPEP_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DPEP_OK 0
+#define DPEP_EINVAL (-1)  /* bad argument (maps to ValueError, like std::invalid_argument in csrc/ops) */
+#define DPEP_ERUNTIME (-2) /* HIP failure (maps to RuntimeError, like std::runtime_error in csrc/ops) */
+
+#define DPEP_MAX_TOPK 32
+#define DPEP_MAX_LOCAL_EXPERTS 1024
+
+const char* dpep_last_error(void);
+int dpep_version(void);
+
+/* Workspace: one hipMalloc'd HBM block standing in for the reference's symmetric SHMEM workspace
+ * (csrc/runtime/session.cpp:40-140, Runtime(...) in csrc/bindings/module.cpp:54-71).  Holds the
+ * layout scratch (per-chunk histograms) and the MegaMoE intermediates of one EP rank's share. */
+int dpep_workspace_create(size_t bytes, void** ws);
+int dpep_workspace_destroy(void* ws);
+int dpep_workspace_capacity(void* ws, size_t* bytes);
+/* Scratch bytes dpep_layout needs for T*K routes and L local experts
+ * (notify_layout() workspace_bytes, csrc/ops/notify.cpp:98-110). */
+size_t dpep_layout_workspace_bytes(int num_tokens, int num_topk, int num_local_experts);
+
+/* Routing layout: validity, per-expert counts, prefix sums and the stable permutation.
+ * Replaces notify() (csrc/ops/notify.cpp:112-190 -> notify_full_kernel, csrc/kernels/notify/notify.cpp:2026)
+ * and the count/prefix half of expand() (csrc/direct/ops/expand.cpp:52-219).
+ *   topk_idx      int64 [T,K]; a route is valid for this rank iff 0 <= e < num_experts and
+ *                 expert_begin <= e < expert_begin + num_local
+ *   counts        int32 [L]    rows per local expert (expert_totals slice / actual_expert_counts)
+ *   psum          int32 [L]    inclusive prefix (psum_num_recv_tokens_per_expert)
+ *   offsets       int32 [L+1]  exclusive prefix with leading 0 (expert_offsets)
+ *   route_to_row  int32 [T*K]  row of route (t,s), -1 if it produces no row (recv_to_expanded_idx)
+ *   row_to_route  int32 [T*K]  first R entries valid: flat route id t*K+s of each row (weight_return_meta)
+ *   num_rows      int32 [1]    R */
+int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk, int num_experts,
+                int expert_begin, int num_local, int32_t* counts, int32_t* psum, int32_t* offsets,
+                int32_t* route_to_row, int32_t* row_to_route, int32_t* num_rows, void* stream);
+
+/* Expand-permute payload dispatch: out[row(t,s)] = x[t] for every route with a row.
+ * Replaces dispatch() (csrc/ops/dispatch.cpp:82-211 -> dispatch_kernel, csrc/kernels/dispatch/dispatch.cpp:628)
+ * and the scatter half of expand() (csrc/direct/kernels/expand/expand.cpp:334-520).
+ *   row_bytes     bytes per payload row (BF16: 2H, FP8: H); must be a multiple of 16
+ *   scales        optional fp32 [T, scale_cols] side rows moved with the payload (FP8 per-128 scales)
+ *   topk_weights  optional fp32 [T,K]; out_weights[row] = topk_weights[t,s]
+ *   num_rows      R (host value read back from dpep_layout) */
+int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_weights,
+                       const int32_t* route_to_row, const int32_t* row_to_route, int num_tokens,
+                       int num_topk, int num_rows, int row_bytes, int scale_cols, void* out,
+                       float* out_scales, float* out_weights, void* stream);
+
+/* Fused per-128-element FP8 e4m3fn quantisation + expand-permute: the reference's caller-side
+ * per_token_cast_to_fp8 (deep_ep/utils/math.py:45-61) followed by the FP8 dispatch above, in one pass.
+ *   x             bf16 [T,H], H % 128 == 0
+ *   out           fp8  [R,H]; out_scales fp32 [R, H/128] */
+int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int32_t* route_to_row,
+                            const int32_t* row_to_route, int num_tokens, int num_topk, int num_rows,
+                            int hidden, void* out, float* out_scales, float* out_weights, void* stream);
+
+/* Stand-alone per-128 quantiser (deep_ep/utils/math.py:45-61): x bf16 [T,H] -> fp8 [T,H], fp32 [T,H/128]. */
+int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float* out_scales, void* stream);
+
+/* Combine: out[t] = bf16_rne( sum over slots in order, skipping -1, of fp32(y[row]) (* w[row]) ).
+ * Replaces combine() (csrc/ops/combine.cpp:198-326 -> combine_kernel, csrc/kernels/combine/combine.cpp:2965)
+ * with row_weights == NULL, and aggregate() / the low-latency combine
+ * (csrc/direct/ops/aggregate.cpp:44-143, csrc/direct/kernels/aggregate/aggregate_impl.h:166-226,
+ * csrc/kernels/combine/low_latency.cpp:41) with row_weights != NULL.
+ *   y             bf16 [R,H], H % 8 == 0
+ *   row_weights   optional fp32 [R]: multiply each row before the add (separate mul and add)
+ *   return_in     optional fp32 [R]: weight-return channel; return_out[t,s] = return_in[row], 0 without a row
+ *   out           bf16 [T,H];  return_out fp32 [T,K] */
+int dpep_combine(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens,
+                 int num_topk, int num_rows, int hidden, void* out, const float* return_in,
+                 float* return_out, void* stream);
+
+/* MXFP8 activation quantiser, block 32 (quantize_input, experiments/megamoe/python/
+ * deep_ep_experimental/megamoe/reference.py:44-54; device ComputeMxScale/QuantizeMxFp8Data).
+ *   x bf16 [B,H], H % 32 == 0 -> codes e4m3 [B,H], scales e8m0 [B,H/32] */
+int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* scales, void* stream);
+
+/* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480). */
+size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, int intermediate, int num_local);
+
+/* One-off weight re-layout (transform_weights_for_mega_moe, experiments/megamoe/python/.../api.py:311-379):
+ * raw packed FP4 [L,N,K/2] + e8m0 [L,N,K/32]  ->  the tile order the GEMM kernel streams.
+ * Byte shuffle only; out buffers have the same sizes as the inputs. */
+int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scales, int num_local, int n,
+                                 int k, uint8_t* out_packed, uint8_t* out_scales, void* stream);
+
+/* Fused W4A8 MoE forward for one rank's local experts (Plan::forward, experiments/megamoe/csrc/forward.cpp:340-478
+ * -> mega_moe_kernel_do, kernel_launch.hpp:8-13):
+ * layout -> gather rows -> GMM1 (MXFP8 x MXFP4) -> bf16 -> SwiGLU -> MXFP8 requant -> GMM2 -> bf16 ->
+ * route-weighted fp32 reduce per token -> bf16.
+ *   x_codes e4m3 [B,H], x_scales e8m0 [B,H/32], topk_idx int32 [B,K] (distinct, in [0,E)), topk_weights fp32 [B,K]
+ *   w1/s1: prepared GMM1 weights [L,2I,H/2] / [L,2I,H/32]; w2/s2: prepared GMM2 weights [L,H,I/2] / [L,H,I/32]
+ *   y bf16 [B,H]; expert_token_nums int32 [L] */
+int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales, const int32_t* topk_idx,
+                         const float* topk_weights, const uint8_t* w1, const uint8_t* s1, const uint8_t* w2,
+                         const uint8_t* s2, int num_tokens, int hidden, int intermediate, int num_topk,
+                         int num_experts, int expert_begin, int num_local, void* y, int32_t* expert_token_nums,
+                         void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,254 @@
+"""GPU parity: HIP layout / dispatch / quantise / combine through the C-ABI vs the CPU oracle.
+
+Bit-exact for layout, indices, payloads, scales and weights; combine bit-exact against the oracle's
+slot-ordered fp32 sum (and therefore within 1 BF16 ulp of the fp64 sum, checked in the CPU suite).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cases
+from oracle import combine as ocombine
+from oracle import layout as olayout
+from oracle import quant as oquant
+from tests.gpu_util import bf16_bits, bits_to_bf16, f32_bits, fp8_bits, i32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from deepep_amd import ops as module
+
+    return module
+
+
+@pytest.fixture(scope="module")
+def ws(ops):
+    workspace = ops.Workspace(64 << 20)
+    yield workspace
+    workspace.destroy()
+
+
+def _check_layout(ops, ws, idx_np, experts, begin=0, local=None):
+    idx = torch.from_numpy(np.ascontiguousarray(idx_np, dtype=np.int64)).cuda()
+    got = ops.layout(ws, idx, experts, begin, local)
+    want = olayout.layout(idx_np, experts, begin, local)
+    rows = int(got["num_rows"].item())
+    assert rows == want["num_rows"]
+    for key in ("counts", "psum", "offsets", "route_to_row"):
+        np.testing.assert_array_equal(i32(got[key]), want[key], err_msg=key)
+    np.testing.assert_array_equal(i32(got["row_to_route"][:rows]), want["row_to_route"])
+    return got, want, rows
+
+
+LAYOUT_SHAPES = [
+    # tokens, topk, experts, begin, local
+    (1, 1, 1, 0, 1),
+    (3, 2, 4, 0, 4),
+    (37, 5, 12, 0, 12),
+    (128, 4, 16, 0, 16),
+    (128, 8, 256, 0, 256),
+    (257, 8, 256, 32, 64),
+    (1000, 16, 1024, 0, 1024),
+    (4096, 8, 256, 0, 256),
+    (16384, 8, 384, 0, 6),
+    (16384, 8, 384, 378, 6),
+    (5000, 6, 7, 2, 3),
+]
+
+
+@pytest.mark.parametrize("tokens,topk,experts,begin,local", LAYOUT_SHAPES)
+def test_layout_matches_oracle(ops, ws, tokens, topk, experts, begin, local):
+    rng = np.random.default_rng(tokens * 31 + topk)
+    idx = rng.integers(-1, experts + 1, size=(tokens, topk))  # includes -1 and == E (both invalid)
+    _check_layout(ops, ws, idx, experts, begin, local)
+
+
+def test_layout_skew_duplicates_and_masks(ops, ws):
+    idx = np.zeros((2048, 8), dtype=np.int64)  # every slot hits expert 0: duplicates count separately
+    _check_layout(ops, ws, idx, 256)
+    idx = np.full((300, 8), -1, dtype=np.int64)  # all masked
+    got, _, rows = _check_layout(ops, ws, idx, 256)
+    assert rows == 0
+    _check_layout(ops, ws, np.zeros((0, 8), dtype=np.int64), 256)  # zero tokens
+
+
+def test_layout_reference_matrix_routes(ops, ws):
+    # deterministic generator of the reference's golden matrix (tests/utils/cases.py:150-157), EP8 case
+    routes = cases.matrix_routes(2, 256, 8, [4096, 4095])  # first two source ranks of ep8_token_volume
+    idx = np.asarray([row for rank in routes for row in rank], dtype=np.int64)
+    for rank in (0, 3):
+        _check_layout(ops, ws, idx, 256, rank * 32, 32)
+
+
+@pytest.mark.parametrize("name,tokens", [("C1", None), ("C2", None), ("C3", 512), ("C4", 2048)])
+@pytest.mark.parametrize("with_weights", [True, False])
+def test_dispatch_bf16_bit_exact(ops, ws, name, tokens, with_weights):
+    x, idx, w, cfg = cases.make_inputs(name, tokens=tokens)
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    xd = x.cuda()
+    wd = w.cuda() if with_weights else None
+    out, out_scales, out_w = ops.dispatch_copy(xd, None, wd, got["route_to_row"], got["row_to_route"], rows)
+    assert out_scales is None
+    np.testing.assert_array_equal(bf16_bits(out), olayout.expand_rows(bf16_bits(x), want["row_to_route"], cfg["topk"]))
+    if with_weights:
+        np.testing.assert_array_equal(f32_bits(out_w), olayout.expand_weights(w.numpy(), want["row_to_route"]).view(np.uint32))
+    else:
+        assert out_w is None
+
+
+@pytest.mark.parametrize("hidden", [16, 48, 128, 1024, 7168])
+def test_dispatch_bf16_widths_and_reference_payload(ops, ws, hidden):
+    # reference fixture values: ((src*13 + t*7 + c*3 + g*11) % 127 - 63) / 16 are BF16-exact
+    tokens, topk, experts = 70, 6, 24
+    values, _ = cases.dispatch_payload_values(2, tokens, 1, max(hidden, 128))
+    x = torch.from_numpy(values[:, :hidden].copy()).bfloat16()
+    idx = np.asarray(cases.matrix_routes(1, experts, topk, [tokens])[0])
+    got, want, rows = _check_layout(ops, ws, idx, experts)
+    w = torch.from_numpy(cases.dispatch_weights(2, tokens, topk, 1))
+    out, _, out_w = ops.dispatch_copy(x.cuda(), None, w.cuda(), got["route_to_row"], got["row_to_route"], rows)
+    np.testing.assert_array_equal(bf16_bits(out), olayout.expand_rows(bf16_bits(x), want["row_to_route"], topk))
+    np.testing.assert_array_equal(out_w.cpu().numpy(), olayout.expand_weights(w.numpy(), want["row_to_route"]))
+
+
+@pytest.mark.parametrize("name,tokens", [("C1", None), ("C3", 300), ("C4", 4096)])
+def test_dispatch_fp8_prequantized_copy(ops, ws, name, tokens):
+    # reference semantic: FP8 payload + FP32 scales move unchanged (docs/elastic.md:61)
+    x, idx, w, cfg = cases.make_inputs(name, tokens=tokens)
+    q, s = oquant.cast_to_fp8_torch(x)
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    out, out_s, out_w = ops.dispatch_copy(q.cuda(), s.cuda(), w.cuda(), got["route_to_row"], got["row_to_route"], rows)
+    np.testing.assert_array_equal(fp8_bits(out), olayout.expand_rows(fp8_bits(q), want["row_to_route"], cfg["topk"]))
+    np.testing.assert_array_equal(f32_bits(out_s), olayout.expand_rows(f32_bits(s), want["row_to_route"], cfg["topk"]))
+    np.testing.assert_array_equal(f32_bits(out_w), olayout.expand_weights(w.numpy(), want["row_to_route"]).view(np.uint32))
+
+
+@pytest.mark.parametrize("scale", [1.0, 1e-3, 300.0, 1e-5, 3e4, 2.0**-20])
+def test_cast_to_fp8_bit_exact_random(ops, scale):
+    gen = torch.Generator().manual_seed(int(scale * 1000) % 97)
+    x = (torch.randn(96, 7168, generator=gen) * scale).bfloat16()
+    x[0, :128] = 0
+    q, s = ops.cast_to_fp8(x.cuda())
+    q_ref, s_ref = oquant.cast_to_fp8_torch(x)
+    np.testing.assert_array_equal(fp8_bits(q), fp8_bits(q_ref))
+    np.testing.assert_array_equal(f32_bits(s), f32_bits(s_ref))
+
+
+def test_cast_to_fp8_every_bf16_magnitude(ops):
+    # every finite positive BF16 pattern as a block maximum with a spread of smaller entries: exercises
+    # the reciprocal, the product rounding and every e4m3 code including subnormals.
+    mags = np.arange(0x0001, 0x7F80, dtype=np.uint16)
+    block = np.zeros((mags.size, 128), dtype=np.uint16)
+    block[:, 0] = mags
+    for j in range(1, 128):
+        block[:, j] = np.maximum(mags.astype(np.int32) - 3 * j - (j % 5) * 128, 0).astype(np.uint16) | (0x8000 if j % 2 else 0)
+    q, s = ops.cast_to_fp8(bits_to_bf16(block))
+    q_ref, s_ref = oquant.cast_to_fp8_int(block)
+    np.testing.assert_array_equal(fp8_bits(q), q_ref)
+    np.testing.assert_array_equal(f32_bits(s), s_ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("name,tokens", [("C1", None), ("C2", None), ("C3", 700), ("C4", 4096)])
+def test_dispatch_quant_fp8_fused_equals_quantize_then_copy(ops, ws, name, tokens):
+    x, idx, w, cfg = cases.make_inputs(name, tokens=tokens)
+    q_ref, s_ref = oquant.cast_to_fp8_torch(x)
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    out, out_s, out_w = ops.dispatch_quant_fp8(x.cuda(), w.cuda(), got["route_to_row"], got["row_to_route"], rows)
+    np.testing.assert_array_equal(fp8_bits(out), olayout.expand_rows(fp8_bits(q_ref), want["row_to_route"], cfg["topk"]))
+    np.testing.assert_array_equal(f32_bits(out_s), olayout.expand_rows(f32_bits(s_ref), want["row_to_route"], cfg["topk"]))
+    np.testing.assert_array_equal(f32_bits(out_w), olayout.expand_weights(w.numpy(), want["row_to_route"]).view(np.uint32))
+
+
+@pytest.mark.parametrize("name,tokens", [("C1", None), ("C2", None), ("C3", 600), ("C4", 4096)])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_combine_matches_oracle(ops, ws, name, tokens, weighted):
+    x, idx, w, cfg = cases.make_inputs(name, tokens=tokens)
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    gen = torch.Generator().manual_seed(5)
+    y = torch.randn(rows, cfg["hidden"], generator=gen).bfloat16()
+    w_rows = torch.from_numpy(olayout.expand_weights(w.numpy(), want["row_to_route"]))
+    ret = torch.rand(rows, generator=gen)
+    out, returned = ops.combine(y.cuda(), got["route_to_row"], w_rows.cuda() if weighted else None, ret.cuda())
+    ref = ocombine.combine(bf16_bits(y), want["route_to_row"], w_rows.numpy() if weighted else None)
+    np.testing.assert_array_equal(bf16_bits(out), ref)
+    np.testing.assert_array_equal(f32_bits(returned), ocombine.return_weights(ret.numpy(), want["route_to_row"]).view(np.uint32))
+
+
+def test_combine_reference_bounded_integer_fixture(ops, ws):
+    # tests/elastic/test_combine.py:496-515: exact sums base*count + sum((e%3-1)+(s%3-1))
+    tokens, hidden, experts, topk, generation = 333, 7168, 64, 8, 2
+    idx = np.asarray(cases.matrix_routes(1, experts, topk, [tokens])[0])
+    idx[7, :] = -1
+    got, want, rows = _check_layout(ops, ws, idx, experts)
+    base = cases.combine_payload_values(0, tokens, generation, hidden)
+    route = want["row_to_route"]
+    e, s = idx.reshape(-1)[route], route % topk
+    y = torch.from_numpy(olayout.expand_rows(base, route, topk) + ((e % 3 - 1) + (s % 3 - 1))[:, None].astype(np.float32)).bfloat16()
+    out, _ = ops.combine(y.cuda(), got["route_to_row"])
+    expected = cases.combine_expected_values(idx.tolist(), experts, 0, generation, hidden)
+    np.testing.assert_array_equal(out.float().cpu().numpy(), expected)
+
+
+def test_combine_order_and_unfused_arithmetic(ops):
+    big = 2.0**24
+    y = torch.tensor([[big] * 8, [1.0] * 8, [-big] * 8]).bfloat16().cuda()
+    r2r = torch.tensor([[0, 1, 2], [0, 2, 1]], dtype=torch.int32).cuda()
+    out, _ = ops.combine(y, r2r)
+    assert out.float().cpu()[:, 0].tolist() == [0.0, 1.0]
+    a, w, c = np.float32(1.0 + 2.0**-7), np.float32(1.0 + 2.0**-23), np.float32(-1.0)
+    y = torch.tensor([[float(a)] * 8, [float(c)] * 8]).bfloat16().cuda()
+    out, _ = ops.combine(y, torch.tensor([[0, 1]], dtype=torch.int32).cuda(), torch.tensor([float(w), 1.0]).cuda())
+    unfused = np.float32(np.float32(a * w) + c)
+    assert out.float().cpu()[0, 0].item() == torch.tensor(float(unfused)).bfloat16().float().item()
+
+
+def test_roundtrip_identity_multiplicity(ops, ws):
+    # dispatch then unweighted combine of the untouched rows gives x * (number of valid slots), exactly
+    # when x is small-integer valued (tests/test_reference.py:88-97).
+    tokens, hidden, experts, topk = 500, 256, 32, 8
+    rng = np.random.default_rng(1)
+    idx = rng.integers(-1, experts, size=(tokens, topk))
+    x = torch.from_numpy(rng.integers(-8, 9, size=(tokens, hidden)).astype(np.float32)).bfloat16()
+    got, want, rows = _check_layout(ops, ws, idx, experts)
+    out, _, _ = ops.dispatch_copy(x.cuda(), None, None, got["route_to_row"], got["row_to_route"], rows)
+    back, _ = ops.combine(out, got["route_to_row"])
+    count = (idx >= 0).sum(axis=1, keepdims=True).astype(np.float32)
+    np.testing.assert_array_equal(back.float().cpu().numpy(), x.float().numpy() * count)
+
+
+def test_full_size_prefill_properties(ops, ws):
+    # BASELINE prefill shape (T=4096, H=7168, E=256, K=8, Zipf): checks that do not need the oracle to
+    # materialise 470 MB: row checksums of the FP8 payload against the token checksums, and the combine
+    # of the dispatched BF16 rows against count * x on integer-valued input.
+    x, idx, w, cfg = cases.make_inputs("C3")
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"])
+    assert rows == 4096 * 8
+    xd = x.cuda()
+    q, s = ops.cast_to_fp8(xd)
+    out, out_s, out_w = ops.dispatch_quant_fp8(xd, w.cuda(), got["route_to_row"], got["row_to_route"], rows)
+    token_of_row = (got["row_to_route"][:rows] // cfg["topk"]).long()
+    assert torch.equal(out.view(torch.uint8), q.view(torch.uint8)[token_of_row])
+    assert torch.equal(out_s.view(torch.int32), s.view(torch.int32)[token_of_row])
+    assert torch.equal(out_w.view(torch.int32), w.cuda().view(-1).view(torch.int32)[got["row_to_route"][:rows].long()])
+    xi = torch.randint(-8, 9, x.shape, generator=torch.Generator().manual_seed(1)).bfloat16().cuda()
+    rows_bf16, _, _ = ops.dispatch_copy(xi, None, None, got["route_to_row"], got["row_to_route"], rows)
+    back, _ = ops.combine(rows_bf16, got["route_to_row"])
+    assert torch.equal(back.float(), xi.float() * 8)
+
+
+def test_argument_errors(ops, ws):
+    idx = torch.zeros((4, 2), dtype=torch.int64).cuda()
+    with pytest.raises(ValueError):
+        ops.layout(ws, idx, 4, 3, 2)  # local range past E
+    with pytest.raises(ValueError):
+        ops.layout(ws, idx.int(), 4)  # wrong dtype
+    lay = ops.layout(ws, idx, 4)
+    x = torch.zeros((4, 24), dtype=torch.bfloat16).cuda()
+    with pytest.raises(ValueError):
+        ops.dispatch_copy(x[:, :20].contiguous(), None, None, lay["route_to_row"], lay["row_to_route"], 8)  # 40-byte rows
+    with pytest.raises(ValueError):
+        ops.dispatch_quant_fp8(x, None, lay["route_to_row"], lay["row_to_route"], 8)  # H % 128
+    with pytest.raises(ValueError):
+        ops.combine(torch.zeros((8, 12), dtype=torch.bfloat16).cuda(), lay["route_to_row"])  # H % 8
