@@ -5,19 +5,23 @@
 // tests/elastic/test_dispatch.py:538-548): rows are ordered (local expert, token, slot); every valid
 // slot gets its own row (duplicates included); invalid ids produce no row.
 //
-// Decomposition: the flat route stream is cut into chunks of kChunk routes, one wavefront each.
-//   count  : each wave histograms its chunk              -> hist[chunk][expert]
-//   scan   : one workgroup turns hist into exclusive bases (over chunks, then over experts)
-//   assign : each wave replays its chunk in order; the rank of a route among equal experts inside a
-//            64-route step comes from ballot/popcount, the carry between steps lives in LDS.
+// Decomposition: the flat route stream is cut into chunks, one wavefront each, four per workgroup.
+//   count  : each wave histograms its chunk                    -> hist[chunk][expert]   (<= 64 KiB, L2-resident)
+//   assign : each workgroup sums the histogram columns (all chunks -> expert totals and their exclusive
+//            scan; chunks before each of its waves -> that wave's base), then every wave replays its
+//            chunk in order.  The rank of a route among equal experts inside a 64-route step comes from
+//            ballot/popcount, the carry between steps lives in LDS.  There is no separate scan launch.
 #include "common.h"
 
 namespace dpep {
 namespace {
 
-constexpr int kChunk = 256;        // routes per wavefront
-constexpr int kWavesPerBlock = 4;  // wavefronts per workgroup in count/assign
-constexpr int kScanThreads = 1024;
+constexpr int kWaves = 4;             // wavefronts (= chunks) per workgroup
+constexpr int kThreads = kWaves * kWave;
+constexpr int kHistInts = 16384;      // chunks * padded experts never exceeds this
+constexpr int kMinChunk = 256;        // routes per wavefront, lower bound (multiple of 64)
+constexpr int kPrefetch = 8;          // 64-route steps whose ids are fetched before the ordered replay
+constexpr int kColumnBatch = 16;      // histogram loads in flight per thread
 
 __device__ __forceinline__ uint64_t lanes_below()
 {
@@ -37,10 +41,10 @@ __device__ __forceinline__ uint64_t match_expert(int e, bool valid, int nbits)
 }
 
 template <typename IdxT>
-__device__ __forceinline__ int local_expert(const IdxT* __restrict__ idx, int route, int n_routes, int num_experts,
+__device__ __forceinline__ int local_expert(const IdxT* __restrict__ idx, int route, int end, int num_experts,
                                             int expert_begin, int num_local)
 {
-    if (route >= n_routes) return -1;
+    if (route >= end) return -1;
     const long long e = static_cast<long long>(idx[route]);
     if (e < 0 || e >= num_experts) return -1;
     const long long local = e - expert_begin;
@@ -48,111 +52,201 @@ __device__ __forceinline__ int local_expert(const IdxT* __restrict__ idx, int ro
 }
 
 template <typename IdxT>
-__global__ __launch_bounds__(kWavesPerBlock* kWave) void layout_count_kernel(
-    const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int nbits,
-    int num_chunks, int* __restrict__ hist)
+__global__ __launch_bounds__(kThreads) void layout_count_kernel(const IdxT* __restrict__ idx, int n_routes,
+                                                                int num_experts, int expert_begin, int num_local,
+                                                                int nbits, int chunk, int num_chunks,
+                                                                int* __restrict__ hist)
 {
     extern __shared__ int lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int chunk = blockIdx.x * kWavesPerBlock + wave;
+    const int g = blockIdx.x * kWaves + wave;
+    if (g >= num_chunks) return;
     int* mine = lds + wave * num_local;
     for (int e = lane; e < num_local; e += kWave) mine[e] = 0;
     __builtin_amdgcn_wave_barrier();
-    if (chunk >= num_chunks) return;
-    const int begin = chunk * kChunk;
-    for (int step = 0; step < kChunk; step += kWave) {
-        const int e = local_expert(idx, begin + step + lane, n_routes, num_experts, expert_begin, num_local);
-        const uint64_t mask = match_expert(e, e >= 0, nbits);
-        if (e >= 0 && (mask & lanes_below()) == 0) mine[e] += __popcll(mask);
-        __builtin_amdgcn_wave_barrier();
+    const int begin = g * chunk;
+    const int end = min(begin + chunk, n_routes);
+    for (int base = begin; base < end; base += kPrefetch * kWave) {
+        int experts[kPrefetch];
+#pragma unroll
+        for (int i = 0; i < kPrefetch; ++i)
+            experts[i] = local_expert(idx, base + i * kWave + lane, end, num_experts, expert_begin, num_local);
+#pragma unroll
+        for (int i = 0; i < kPrefetch; ++i) {
+            const int e = experts[i];
+            const uint64_t mask = match_expert(e, e >= 0, nbits);
+            if (e >= 0 && (mask & lanes_below()) == 0) mine[e] += __popcll(mask);
+            __builtin_amdgcn_wave_barrier();
+        }
     }
-    int* out = hist + static_cast<size_t>(chunk) * num_local;
+    int* out = hist + static_cast<size_t>(g) * num_local;
     for (int e = lane; e < num_local; e += kWave) out[e] = mine[e];
 }
 
-// hist[chunk][e] (counts) -> exclusive base of chunk `chunk` for expert e, including the expert's
-// own offset; also emits counts / psum / offsets / num_rows.
-__global__ __launch_bounds__(kScanThreads) void layout_scan_kernel(int* __restrict__ hist, int num_chunks,
-                                                                   int num_local, int ex, int* __restrict__ counts,
-                                                                   int* __restrict__ psum, int* __restrict__ offsets,
-                                                                   int* __restrict__ num_rows)
+// Column sums of hist for one expert over the chunks {first, first+stride, ...}: the total, and for
+// each wave w of this workgroup the part that lies in chunks before chunk0 + w.
+struct ColumnSums {
+    int total;
+    int before[kWaves];
+};
+
+__device__ __forceinline__ ColumnSums column_sums(const int* __restrict__ hist, int num_local, int e, int first,
+                                                  int stride, int num_chunks, int chunk0)
 {
-    __shared__ int partial[kScanThreads];
-    __shared__ int scan_a[DPEP_MAX_LOCAL_EXPERTS];
-    __shared__ int scan_b[DPEP_MAX_LOCAL_EXPERTS];
-    const int tid = threadIdx.x;
-    const int parts = kScanThreads / ex;
-    const int p = tid / ex, e = tid % ex;
-    const int per_part = (num_chunks + parts - 1) / parts;
-    const int g0 = min(p * per_part, num_chunks), g1 = min(g0 + per_part, num_chunks);
-    int sum = 0;
-    if (e < num_local)
-        for (int g = g0; g < g1; ++g) sum += hist[static_cast<size_t>(g) * num_local + e];
-    partial[tid] = sum;
-    __syncthreads();
-    int before = 0;
-    for (int q = 0; q < p; ++q) before += partial[q * ex + e];
-    if (p == parts - 1 && e < num_local) scan_a[e] = before + sum;  // total rows of expert e
-    __syncthreads();
-    // Inclusive Hillis-Steele scan over experts (num_local <= 1024 == blockDim).
-    int* src = scan_a;
-    int* dst = scan_b;
-    for (int stride = 1; stride < num_local; stride <<= 1) {
-        if (tid < num_local) dst[tid] = src[tid] + (tid >= stride ? src[tid - stride] : 0);
+    ColumnSums sums;
+    sums.total = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sums.before[w] = 0;
+    for (int c0 = first; c0 < num_chunks; c0 += kColumnBatch * stride) {
+        int v[kColumnBatch];
+#pragma unroll
+        for (int j = 0; j < kColumnBatch; ++j) {
+            const int c = c0 + j * stride;
+            v[j] = c < num_chunks ? hist[static_cast<size_t>(c) * num_local + e] : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < kColumnBatch; ++j) {
+            const int c = c0 + j * stride;
+            sums.total += v[j];
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) sums.before[w] += c < chunk0 + w ? v[j] : 0;
+        }
+    }
+    return sums;
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(kThreads) void layout_assign_kernel(
+    const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int padded_local,
+    int nbits, int chunk, int num_chunks, const int* __restrict__ hist, int* __restrict__ counts,
+    int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows, int* __restrict__ route_to_row,
+    int* __restrict__ row_to_route)
+{
+    // totals[e]: rows of expert e (later its exclusive offset); running[w][e]: next row of expert e for wave w.
+    __shared__ int totals[DPEP_MAX_LOCAL_EXPERTS];
+    __shared__ int running[kWaves][DPEP_MAX_LOCAL_EXPERTS];
+    __shared__ int partial[kThreads * (kWaves + 1)];
+    __shared__ int wave_sums[kWaves];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int chunk0 = blockIdx.x * kWaves;
+
+    if (padded_local >= kThreads) {
+        for (int e = tid; e < num_local; e += kThreads) {
+            const ColumnSums sums = column_sums(hist, num_local, e, 0, 1, num_chunks, chunk0);
+            totals[e] = sums.total;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) running[w][e] = sums.before[w];
+        }
+    } else {
+        // Few experts: split the chunks over `parts` thread groups (at most 16), then reduce through LDS.
+        int parts = kThreads / padded_local;
+        if (parts > 16) parts = 16;
+        const int p = tid / padded_local, e = tid % padded_local;
+        const bool active = p < parts && e < num_local;
+        if (active) {
+            const ColumnSums sums = column_sums(hist, num_local, e, p, parts, num_chunks, chunk0);
+            partial[tid * (kWaves + 1)] = sums.total;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) partial[tid * (kWaves + 1) + 1 + w] = sums.before[w];
+        }
         __syncthreads();
-        int* t = src;
-        src = dst;
-        dst = t;
+        if (tid < num_local) {
+            int total = 0, before[kWaves] = {0, 0, 0, 0};
+            for (int q = 0; q < parts; ++q) {
+                const int* src = partial + (q * padded_local + tid) * (kWaves + 1);
+                total += src[0];
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) before[w] += src[1 + w];
+            }
+            totals[tid] = total;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) running[w][tid] = before[w];
+        }
     }
-    if (tid < num_local) {
-        const int incl = src[tid];
-        const int total = incl - (tid > 0 ? src[tid - 1] : 0);
-        counts[tid] = total;
-        psum[tid] = incl;
-        offsets[tid + 1] = incl;
-        if (tid == 0) offsets[0] = 0;
-        if (tid == num_local - 1) num_rows[0] = incl;
+    __syncthreads();
+
+    // Exclusive scan of totals over experts: four consecutive experts per thread, then a workgroup scan.
+    int mine[4], local_sum = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = tid * 4 + j;
+        mine[j] = e < num_local ? totals[e] : 0;
+        local_sum += mine[j];
     }
-    if (e < num_local) {
-        int running = before + (e > 0 ? src[e - 1] : 0);
-        for (int g = g0; g < g1; ++g) {
-            const size_t at = static_cast<size_t>(g) * num_local + e;
-            const int v = hist[at];
-            hist[at] = running;
-            running += v;
+    int incl = local_sum;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) wave_sums[wave] = incl;
+    __syncthreads();
+    int offset = incl - local_sum;
+    for (int w = 0; w < wave; ++w) offset += wave_sums[w];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = tid * 4 + j;
+        if (e < num_local) {
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) running[w][e] += offset;
+            if (blockIdx.x == 0) {
+                counts[e] = mine[j];
+                psum[e] = offset + mine[j];
+                offsets[e + 1] = offset + mine[j];
+            }
+        }
+        offset += mine[j];
+    }
+    if (blockIdx.x == 0 && tid == kThreads - 1) {
+        offsets[0] = 0;
+        num_rows[0] = offset;
+    }
+    __syncthreads();
+
+    const int g = chunk0 + wave;
+    if (g >= num_chunks) return;
+    int* next_row = running[wave];
+    const int begin = g * chunk;
+    const int end = min(begin + chunk, n_routes);
+    for (int base = begin; base < end; base += kPrefetch * kWave) {
+        int experts[kPrefetch];
+#pragma unroll
+        for (int i = 0; i < kPrefetch; ++i)
+            experts[i] = local_expert(idx, base + i * kWave + lane, end, num_experts, expert_begin, num_local);
+#pragma unroll
+        for (int i = 0; i < kPrefetch; ++i) {
+            const int route = base + i * kWave + lane;
+            const int e = experts[i];
+            const uint64_t mask = match_expert(e, e >= 0, nbits);
+            const int ahead = __popcll(mask & lanes_below());
+            int row = -1;
+            if (e >= 0) row = next_row[e] + ahead;
+            __builtin_amdgcn_wave_barrier();
+            if (e >= 0 && ahead == 0) next_row[e] = row + __popcll(mask);
+            __builtin_amdgcn_wave_barrier();
+            if (route < end) {
+                route_to_row[route] = row;
+                if (row >= 0) row_to_route[row] = route;
+            }
         }
     }
 }
 
-template <typename IdxT>
-__global__ __launch_bounds__(kWavesPerBlock* kWave) void layout_assign_kernel(
-    const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int nbits,
-    int num_chunks, const int* __restrict__ base, int* __restrict__ route_to_row, int* __restrict__ row_to_route)
+int padded_experts(int num_local)
 {
-    extern __shared__ int lds[];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int chunk = blockIdx.x * kWavesPerBlock + wave;
-    if (chunk >= num_chunks) return;
-    int* running = lds + wave * num_local;
-    const int* mine = base + static_cast<size_t>(chunk) * num_local;
-    for (int e = lane; e < num_local; e += kWave) running[e] = mine[e];
-    __builtin_amdgcn_wave_barrier();
-    const int begin = chunk * kChunk;
-    for (int step = 0; step < kChunk; step += kWave) {
-        const int route = begin + step + lane;
-        const int e = local_expert(idx, route, n_routes, num_experts, expert_begin, num_local);
-        const uint64_t mask = match_expert(e, e >= 0, nbits);
-        const int ahead = __popcll(mask & lanes_below());
-        int row = -1;
-        if (e >= 0) row = running[e] + ahead;
-        __builtin_amdgcn_wave_barrier();
-        if (e >= 0 && ahead == 0) running[e] = row + __popcll(mask);
-        __builtin_amdgcn_wave_barrier();
-        if (route < n_routes) {
-            route_to_row[route] = row;
-            if (row >= 0) row_to_route[row] = route;
-        }
-    }
+    int padded = 1;
+    while (padded < num_local) padded <<= 1;
+    return padded;
+}
+
+// Chunk length: as many chunks as the histogram budget allows (16..256), at least kMinChunk routes each.
+int chunk_routes(int n_routes, int padded_local)
+{
+    int max_chunks = kHistInts / padded_local;
+    max_chunks = max_chunks > 256 ? 256 : (max_chunks < 16 ? 16 : max_chunks);
+    int chunk = (n_routes + max_chunks - 1) / max_chunks;
+    chunk = (chunk + kWave - 1) / kWave * kWave;
+    return chunk < kMinChunk ? kMinChunk : chunk;
 }
 
 template <typename IdxT>
@@ -173,29 +267,24 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
     DPEP_REQUIRE(n_routes == 0 || (idx && route_to_row && row_to_route), "layout: NULL routing buffer");
     const size_t need = dpep_layout_workspace_bytes(num_tokens, num_topk, num_local);
     DPEP_REQUIRE(need <= w->bytes, "layout: workspace too small (%zu needed, %zu available)", need, w->bytes);
-    const int num_chunks = (n_routes + kChunk - 1) / kChunk;
+    const int padded = padded_experts(num_local);
+    const int chunk = chunk_routes(n_routes, padded);
+    const int num_chunks = (n_routes + chunk - 1) / chunk;
     int nbits = 0;
     while ((1 << nbits) < num_local) ++nbits;
-    int ex = 1;
-    while (ex < num_local) ex <<= 1;
     int* hist = static_cast<int*>(w->base);
-    const int blocks = (num_chunks + kWavesPerBlock - 1) / kWavesPerBlock;
-    const size_t lds = static_cast<size_t>(kWavesPerBlock) * num_local * sizeof(int);
+    const int blocks = (num_chunks + kWaves - 1) / kWaves;
     if (blocks > 0) {
-        hipLaunchKernelGGL(layout_count_kernel<IdxT>, dim3(blocks), dim3(kWavesPerBlock * kWave), lds, stream, idx,
-                           n_routes, num_experts, expert_begin, num_local, nbits, num_chunks, hist);
+        hipLaunchKernelGGL(layout_count_kernel<IdxT>, dim3(blocks), dim3(kThreads),
+                           static_cast<size_t>(kWaves) * num_local * sizeof(int), stream, idx, n_routes, num_experts,
+                           expert_begin, num_local, nbits, chunk, num_chunks, hist);
         if (int rc = launch_status("layout_count")) return rc;
     }
-    hipLaunchKernelGGL(layout_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, hist, num_chunks, num_local, ex,
-                       counts, psum, offsets, num_rows);
-    if (int rc = launch_status("layout_scan")) return rc;
-    if (blocks > 0) {
-        hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks), dim3(kWavesPerBlock * kWave), lds, stream, idx,
-                           n_routes, num_experts, expert_begin, num_local, nbits, num_chunks, hist, route_to_row,
-                           row_to_route);
-        if (int rc = launch_status("layout_assign")) return rc;
-    }
-    return DPEP_OK;
+    // With no routes one workgroup still publishes the all-zero counts and prefix sums.
+    hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks > 0 ? blocks : 1), dim3(kThreads), 0, stream, idx,
+                       n_routes, num_experts, expert_begin, num_local, padded, nbits, chunk, num_chunks, hist, counts,
+                       psum, offsets, num_rows, route_to_row, row_to_route);
+    return launch_status("layout_assign");
 }
 
 }  // namespace
@@ -216,10 +305,7 @@ extern "C" {
 size_t dpep_layout_workspace_bytes(int num_tokens, int num_topk, int num_local_experts)
 {
     if (num_tokens < 0 || num_topk < 1 || num_local_experts < 1) return 0;
-    const size_t routes = static_cast<size_t>(num_tokens) * num_topk;
-    const size_t chunks = (routes + dpep::kChunk - 1) / dpep::kChunk;
-    const size_t bytes = (chunks > 0 ? chunks : 1) * num_local_experts * sizeof(int);
-    return (bytes + 255) / 256 * 256;
+    return static_cast<size_t>(dpep::kHistInts) * sizeof(int);
 }
 
 int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk, int num_experts, int expert_begin,
