@@ -1,0 +1,646 @@
+"""``ElasticBuffer`` / ``EPHandle`` with the reference's V2 interface, on one MI355X.
+
+Mirrors deep_ep/backends/mesh_clos/elastic.py (EPHandle :88-173, ElasticBuffer.__init__ :178-269,
+dispatch :648-1008, combine :1010-1283, _notify :1285-1531): same argument names, defaults, return
+tuples and exception types.  What is different, deliberately:
+
+  * one process, one GPU: ``world_size`` defaults to 1 (the reference rejects < 2).  Passing
+    ``rank``/``world_size`` makes the buffer act as ONE rank's share of an EP job: it owns experts
+    ``[rank*E/P, (rank+1)*E/P)`` and ``x`` / ``topk_idx`` are the flattened token stream of all source
+    ranks, so rows come out in the reference's (local expert, source rank, token, slot) order;
+  * the routing metadata is the plain pair route_to_row / row_to_route instead of SHMEM peer
+    tables; payload rows are written straight into torch-allocated outputs;
+  * ``use_fp8_dispatch=True`` with a BF16 ``x`` quantises per 128 elements inside the dispatch
+    kernel and returns ``(fp8, scales)`` (the reference moves pre-quantised tuples only — which this
+    class also accepts).
+"""
+
+from __future__ import annotations
+
+import threading
+import warnings
+from typing import Optional, Tuple, Union
+
+import torch
+
+from .compat import accept_aliases
+from .event import EventHandle, EventOverlap, gpu_api
+
+WORLD_SIZES = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
+MAX_TOKENS = 16384
+MAX_HIDDEN = 7168
+MAX_TOPK = 16
+MAX_EXPERTS = 1024
+MIN_WORKSPACE_BYTES = 2 << 20
+# Routing tensors whose (data_ptr, version) are pinned at dispatch and re-checked by every later
+# cached dispatch and combine.
+_ROUTING = ("topk_idx", "route_to_row", "weight_return_meta", "expert_totals", "psum_num_recv_tokens_per_expert")
+
+
+def _integer(name, value, lower, upper):
+    if type(value) is not int or not lower <= value <= upper:
+        raise ValueError(f"{name} must be an integer in [{lower}, {upper}]")
+
+
+def _validate_hidden(hidden, fp8=False):
+    _integer("hidden", hidden, 1, MAX_HIDDEN)
+    alignment = 128 if fp8 else 16
+    if hidden % alignment:
+        raise ValueError(f"hidden must be a multiple of {alignment}")
+
+
+def _load_native():
+    from . import ops
+
+    ops._lib.load()  # raises if libdeepep_amd.so is not built: there is no fallback path
+    return ops
+
+
+class EPHandle:
+    """Routing plan produced by a fresh dispatch; reused by cached dispatch and by combine."""
+
+    @accept_aliases(num_compute_units="num_sms")
+    def __init__(
+        self,
+        do_expand: bool,
+        num_experts: int,
+        expert_alignment: int,
+        num_max_tokens_per_rank: int,
+        num_sms: int,
+        topk_idx: torch.Tensor,
+        num_recv_tokens: int,
+        num_expanded_tokens: int,
+        num_recv_tokens_per_expert_list: list,
+        psum_num_recv_tokens_per_scaleup_rank: torch.Tensor,
+        psum_num_recv_tokens_per_expert: torch.Tensor,
+        num_unaligned_recv_tokens_per_expert: torch.Tensor,
+        recv_src_metadata: torch.Tensor,
+        dst_buffer_slot_idx: torch.Tensor,
+        token_metadata_at_forward: Optional[torch.Tensor],
+        channel_linked_list: Optional[torch.Tensor],
+        is_low_latency: bool = False,
+    ):
+        self.do_expand = do_expand
+        self.num_experts = num_experts
+        self.expert_alignment = expert_alignment
+        self.num_max_tokens_per_rank = num_max_tokens_per_rank
+        self.num_compute_units = num_sms
+        self.topk_idx = topk_idx
+        self.num_recv_tokens = num_recv_tokens
+        self.num_expanded_tokens = num_expanded_tokens
+        self.num_recv_tokens_per_expert_list = num_recv_tokens_per_expert_list
+        self.psum_num_recv_tokens_per_scaleup_rank = psum_num_recv_tokens_per_scaleup_rank
+        self.psum_num_recv_tokens_per_expert = psum_num_recv_tokens_per_expert
+        self.num_unaligned_recv_tokens_per_expert = num_unaligned_recv_tokens_per_expert
+        self.recv_src_metadata = recv_src_metadata
+        self.dst_buffer_slot_idx = dst_buffer_slot_idx
+        self.token_metadata_at_forward = token_metadata_at_forward
+        self.channel_linked_list = channel_linked_list
+        self.is_low_latency = is_low_latency
+        # Single-GPU routing metadata.
+        self.route_to_row = None          # int32 [T,K]: row of each route, -1 without a row
+        self.weight_return_meta = None    # int32 [R]: flat route id (src*T+t)*K+s of each row
+        self.expert_totals = None         # int32 [L]: rows per local expert
+        self.expert_offsets = None        # int32 [L+1]: exclusive prefix
+        self.source_weights = None        # fp32 [R]: saved route weights (low-latency style handles)
+        self.rank = None
+        self.world_size = None
+        self.num_tokens = None
+        self.num_topk = None
+        self.hidden = None
+        self.metadata_only = True
+        self.metadata_version = 7
+        self._buffer_token = None
+        self._routing_versions = {}
+
+    @property
+    def num_sms(self):
+        return self.num_compute_units
+
+    @num_sms.setter
+    def num_sms(self, value):
+        self.num_compute_units = value
+
+
+class _Runtime:
+    """Process-local owner of the HBM workspace and the communication stream (the single-GPU
+    counterpart of deep_ep/_runtime.py:67-308 without SHMEM bootstrap)."""
+
+    def __init__(self, native, num_bytes, rank, world_size, combine_only):
+        self.native = native
+        self.device = gpu_api().current_device()
+        self.torch_device = torch.device("cuda", self.device)
+        self.rank, self.world_size = rank, world_size
+        self.combine_only = combine_only
+        self.capacity = num_bytes
+        self.notify_lock = threading.RLock()
+        self.notify_failed = False
+        self.notify_inflight = None
+        self.workspace = native.Workspace(num_bytes, self.torch_device)
+        self.stream = gpu_api().Stream(device=self.torch_device)
+        self.closed = False
+
+    def ensure_alive(self):
+        if self.closed:
+            raise RuntimeError("ElasticBuffer was destroyed")
+
+    def close(self):
+        if not self.closed:
+            self.stream.synchronize()
+            self.workspace.destroy()
+            self.closed = True
+            self.notify_inflight = None
+
+
+def _resolve_world(group, rank, world_size):
+    if group is not None:
+        if rank is not None or world_size is not None:
+            raise ValueError("Pass either group or rank/world_size, not both")
+        import torch.distributed as dist
+
+        if not isinstance(group, dist.ProcessGroup):
+            raise TypeError("group must be an initialized torch.distributed ProcessGroup")
+        if dist.get_world_size(group) != 1:
+            raise NotImplementedError(
+                "This build runs one rank per process on one GPU without inter-GPU transport: "
+                "use a single-rank group, or rank=/world_size= to compute one rank's share"
+            )
+        return 0, 1
+    if world_size is None and rank is None:
+        return 0, 1
+    _integer("world_size", world_size, 1, 512)
+    if world_size not in WORLD_SIZES:
+        raise ValueError("Runtime supports EP1/2/4/8/16/32/64/128/256/512")
+    _integer("rank", rank, 0, world_size - 1)
+    return rank, world_size
+
+
+class ElasticBuffer:
+    """Dispatch / combine for one EP rank on one GPU; see the module docstring for the deviations."""
+
+    @accept_aliases(num_device_timeout_secs="num_gpu_timeout_secs")
+    def __init__(
+        self,
+        group=None,
+        num_bytes: Optional[int] = None,
+        num_cpu_bytes: int = 0,
+        num_max_tokens_per_rank: int = 0,
+        hidden: int = 0,
+        num_topk: int = 0,
+        use_fp8_dispatch: bool = False,
+        deterministic: bool = False,
+        allow_hybrid_mode: bool = True,
+        allow_multiple_reduction: bool = True,
+        prefer_overlap_with_compute: bool = True,
+        sl_idx: int = 3,
+        num_allocated_qps: int = 0,
+        num_cpu_timeout_secs: int = 300,
+        num_gpu_timeout_secs: int = 100,
+        explicitly_destroy: bool = False,
+        *,
+        rank: Optional[int] = None,
+        world_size: Optional[int] = None,
+        bootstrap: str = "default",
+        combine_only: bool = False,
+        use_1g_huge_pages: bool = True,
+        debug_collectives: bool = False,
+        machine_type: str = "auto",
+        rootinfo_path: Optional[str] = None,
+    ):
+        native = _load_native()
+        if (
+            num_cpu_bytes != 0
+            or deterministic is not False
+            or allow_hybrid_mode is not True
+            or allow_multiple_reduction is not True
+            or prefer_overlap_with_compute is not True
+            or sl_idx != 3
+            or type(num_allocated_qps) is not int
+            or num_allocated_qps not in (0, 6)
+            or num_gpu_timeout_secs != 100
+        ):
+            raise NotImplementedError("ElasticBuffer supports default options and num_allocated_qps=0/6")
+        if type(use_fp8_dispatch) is not bool:
+            raise TypeError("use_fp8_dispatch must be bool")
+        if explicitly_destroy is not True:
+            raise NotImplementedError("Runtime currently requires explicitly_destroy=True")
+        if type(combine_only) is not bool or type(debug_collectives) is not bool:
+            raise TypeError("combine_only and debug_collectives must be bool")
+        _integer("num_max_tokens_per_rank", num_max_tokens_per_rank, 0, MAX_TOKENS)
+        _integer("num_topk", num_topk, 0, MAX_TOPK)
+        _integer("hidden", hidden, 0, MAX_HIDDEN)
+        if hidden:
+            _validate_hidden(hidden, use_fp8_dispatch)
+        resolved_rank, resolved_world = _resolve_world(group, rank, world_size)
+        if num_bytes is None:
+            if not num_max_tokens_per_rank or not num_topk or not hidden:
+                raise NotImplementedError("Pass num_bytes or provide token/topk bounds and hidden")
+            num_bytes = self.get_buffer_size_hint(
+                group, num_max_tokens_per_rank, hidden, num_topk, use_fp8_dispatch, world_size=world_size
+            )
+        _integer("num_bytes", num_bytes, MIN_WORKSPACE_BYTES, (1 << 63) - 1)
+        self.num_max_tokens_per_rank = num_max_tokens_per_rank
+        self.hidden = hidden
+        self.num_topk = num_topk
+        self.use_fp8_dispatch = use_fp8_dispatch
+        self.machine_type = "mi355x"
+        self._handle_token = object()
+        self._runtime = _Runtime(native, num_bytes, resolved_rank, resolved_world, combine_only)
+
+    def __del__(self):
+        runtime = getattr(self, "_runtime", None)
+        if runtime is not None and not runtime.closed:
+            warnings.warn("ElasticBuffer was not destroyed explicitly; call destroy()", ResourceWarning)
+
+    def _live_runtime(self) -> _Runtime:
+        runtime = getattr(self, "_runtime", None)
+        if runtime is None:
+            raise RuntimeError("ElasticBuffer is not initialised")
+        return runtime
+
+    def destroy(self) -> None:
+        """Release the workspace; repeating a successful destroy is safe."""
+        self._live_runtime().close()
+
+    @staticmethod
+    def get_buffer_size_hint(
+        group,
+        num_max_tokens_per_rank: int,
+        hidden: int,
+        num_topk: int = 0,
+        use_fp8_dispatch: bool = False,
+        allow_hybrid_mode: bool = True,
+        allow_multiple_reduction: bool = True,
+        *,
+        world_size: Optional[int] = None,
+        machine_type: str = "auto",
+        rootinfo_path: Optional[str] = None,
+    ) -> int:
+        """Workspace bytes for the given bounds.
+
+        Payload rows go straight into the returned tensors, so the workspace only holds the layout
+        scratch; the hint is that scratch rounded up to the 2 MiB minimum.
+        """
+        native = _load_native()
+        _validate_hidden(hidden, use_fp8_dispatch)
+        if allow_hybrid_mode is not True or allow_multiple_reduction is not True:
+            raise NotImplementedError("Dispatch sizing supports only default algorithm options")
+        _integer("num_max_tokens_per_rank", num_max_tokens_per_rank, 1, MAX_TOKENS)
+        _integer("num_topk", num_topk, 0, MAX_TOPK)
+        world = 1 if world_size is None else world_size
+        if world not in WORLD_SIZES:
+            raise ValueError("Runtime supports EP1/2/4/8/16/32/64/128/256/512")
+        scratch = native.layout_workspace_bytes(world * num_max_tokens_per_rank, max(num_topk, 1), MAX_EXPERTS)
+        return max(MIN_WORKSPACE_BYTES, (scratch + (2 << 20) - 1) // (2 << 20) * (2 << 20))
+
+    def barrier(self, use_comm_stream: bool = True, with_cpu_sync: bool = False, sequential: bool = True) -> None:
+        """Host-synchronous barrier: with one rank it drains the communication stream."""
+        if type(use_comm_stream) is not bool or with_cpu_sync is not True or sequential is not True:
+            raise NotImplementedError("Only the host-synchronous sequential barrier is implemented")
+        runtime = self._live_runtime()
+        runtime.ensure_alive()
+        runtime.stream.synchronize()
+
+    @staticmethod
+    def capture() -> EventHandle:
+        """Record an event on the current stream."""
+        return EventHandle()
+
+    def get_comm_stream(self) -> torch.cuda.Stream:
+        runtime = self._live_runtime()
+        runtime.ensure_alive()
+        return runtime.stream
+
+    def get_physical_domain_size(self) -> Tuple[int, int]:
+        raise NotImplementedError("ElasticBuffer.get_physical_domain_size is declared but not implemented")
+
+    def get_logical_domain_size(self) -> Tuple[int, int]:
+        raise NotImplementedError("ElasticBuffer.get_logical_domain_size is declared but not implemented")
+
+    @accept_aliases(
+        scaleout_gbs="rdma_gbs",
+        scaleup_gbs="nvlink_gbs",
+        compute_read_gbs="sm_read_gbs",
+        compute_write_gbs="sm_write_gbs",
+        compute_unit_read_gbs="sm_read_gbs",
+        compute_unit_write_gbs="sm_write_gbs",
+    )
+    def get_theoretical_num_sms(
+        self,
+        num_experts: int,
+        num_topk: int,
+        num_scaleout_topk: int = 0,
+        rdma_gbs: float = 0,
+        nvlink_gbs: float = 0,
+        sm_read_gbs: float = 200,
+        sm_write_gbs: float = 50,
+    ) -> int:
+        raise NotImplementedError("ElasticBuffer.get_theoretical_num_sms is declared but not implemented")
+
+    get_theoretical_num_compute_units = get_theoretical_num_sms
+
+    @accept_aliases(num_compute_units="num_sms")
+    def get_theoretical_num_qps(self, num_sms: int) -> int:
+        raise NotImplementedError("ElasticBuffer.get_theoretical_num_qps is declared but not implemented")
+
+    # ------------------------------------------------------------------------------------------
+    def _check_tensor(self, value, dtype, shape=None):
+        runtime = self._runtime
+        return (
+            isinstance(value, torch.Tensor)
+            and value.dtype == dtype
+            and value.device == runtime.torch_device
+            and value.is_contiguous()
+            and not value.requires_grad
+            and (shape is None or tuple(value.shape) == tuple(shape))
+        )
+
+    def _check_versions(self, handle):
+        for name, version in handle._routing_versions.items():
+            tensor = getattr(handle, name)
+            if torch.is_inference(tensor) or (tensor.data_ptr(), tensor._version) != version:
+                raise ValueError(f"Cached routing was modified: {name}")
+
+    @accept_aliases(num_compute_units="num_sms", use_aligned_col_major_sf="use_tma_aligned_col_major_sf")
+    def dispatch(
+        self,
+        x: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]],
+        topk_idx: Optional[torch.Tensor] = None,
+        topk_weights: Optional[torch.Tensor] = None,
+        cumulative_local_expert_recv_stats: Optional[torch.Tensor] = None,
+        num_experts: Optional[int] = None,
+        num_max_tokens_per_rank: Optional[int] = None,
+        expert_alignment: Optional[int] = None,
+        num_sms: int = 0,
+        num_qps: int = 0,
+        previous_event: Optional[EventHandle] = None,
+        previous_event_before_epilogue: Optional[EventHandle] = None,
+        async_with_compute_stream: bool = False,
+        allocate_on_comm_stream: bool = False,
+        handle: Optional[EPHandle] = None,
+        do_handle_copy: bool = True,
+        do_cpu_sync: Optional[bool] = None,
+        do_expand: Optional[bool] = None,
+        do_zero_padding: bool = False,
+        use_tma_aligned_col_major_sf: bool = False,
+    ):
+        """Return ``(expanded_x | (expanded_x, scales), None, expanded_weights | None, handle, event)``.
+
+        Rows are ordered (local expert, source rank, token, top-k slot); one row per valid slot;
+        ids < 0 or >= num_experts produce no row; weights are moved, never applied.
+        A fresh call computes the layout and reads the per-expert counts back to the host (one
+        synchronisation); ``handle=`` reuses a previous plan with a new payload.
+        """
+        runtime = self._live_runtime()
+        runtime.ensure_alive()
+        native = runtime.native
+        if runtime.combine_only:
+            raise ValueError("Dispatch requires combine_only=False when constructing ElasticBuffer")
+        if isinstance(handle, EPHandle) and handle.is_low_latency:
+            raise NotImplementedError("Cached dispatch is not supported for LL handles")
+        with runtime.notify_lock:
+            if runtime.notify_failed:
+                raise RuntimeError("A previous communication launch failed; restart the distributed job")
+            for name, value in (
+                ("async_with_compute_stream", async_with_compute_stream),
+                ("allocate_on_comm_stream", allocate_on_comm_stream),
+                ("do_handle_copy", do_handle_copy),
+                ("do_zero_padding", do_zero_padding),
+                ("use_aligned_col_major_sf", use_tma_aligned_col_major_sf),
+            ):
+                if type(value) is not bool:
+                    raise TypeError(f"{name} must be bool")
+            if do_expand is not None and do_expand is not True:
+                raise NotImplementedError("Dispatch supports only the expanded expert layout")
+            if do_cpu_sync is not None and type(do_cpu_sync) is not bool:
+                raise TypeError("do_cpu_sync must be bool or None")
+            if handle is None and do_cpu_sync is False:
+                raise NotImplementedError("Fresh notify requires do_cpu_sync=None/True")
+            if expert_alignment is not None and (type(expert_alignment) is not int or expert_alignment != 1):
+                raise NotImplementedError("Dispatch supports expert_alignment=1")
+            if (
+                cumulative_local_expert_recv_stats is not None
+                or previous_event_before_epilogue is not None
+                or allocate_on_comm_stream
+                or do_zero_padding
+                or use_tma_aligned_col_major_sf
+            ):
+                raise NotImplementedError(
+                    "Stats, epilogue events, padding and alternate allocation/scale layouts are unavailable"
+                )
+            if previous_event is not None and (
+                not isinstance(previous_event, EventHandle) or previous_event._device != runtime.device
+            ):
+                raise ValueError("previous_event must belong to the buffer GPU")
+            fp8_input = isinstance(x, tuple)
+            if fp8_input and len(x) != 2:
+                raise ValueError("FP8 input must be (hidden, scales)")
+            hidden, scales = x if fp8_input else (x, None)
+            if not self._check_tensor(hidden, torch.float8_e4m3fn if fp8_input else torch.bfloat16) or hidden.ndim != 2:
+                raise ValueError(
+                    "x must be contiguous BF16, or (FP8 E4M3FN, FP32 scales), on the buffer GPU without grad"
+                )
+            tokens, width = hidden.shape
+            fuse_quant = self.use_fp8_dispatch and not fp8_input
+            fp8 = fp8_input or fuse_quant
+            _validate_hidden(width, fp8)
+            if self.hidden and width != self.hidden:
+                raise ValueError("hidden differs from buffer configuration")
+            if fp8_input and not self._check_tensor(scales, torch.float32, (tokens, width // 128)):
+                raise ValueError("FP8 scales must be contiguous FP32 [T,H/128] on the buffer GPU without grad")
+            if type(num_sms) is not int or num_sms not in (0, 64 if fp8 else 32):
+                raise ValueError("num_compute_units must be 0/32 for BF16 or 0/64 for FP8")
+            if type(num_qps) is not int or num_qps not in (0, 2):
+                raise ValueError("Primary dispatch uses two QPs per peer; num_qps=0/2")
+            world = runtime.world_size
+            if handle is not None:
+                if (
+                    not isinstance(handle, EPHandle)
+                    or handle._buffer_token is not self._handle_token
+                    or handle.metadata_only
+                    or handle.metadata_version != 7
+                ):
+                    raise ValueError("Cached handle must come from this buffer's successful payload dispatch")
+                if topk_idx is not None:
+                    raise ValueError("Cached dispatch inherits routing; omit topk_idx")
+                if num_experts is not None and num_experts != handle.num_experts:
+                    raise ValueError("num_experts differs from cached routing")
+                self._check_versions(handle)
+                num_experts, topk = handle.num_experts, handle.num_topk
+                if tokens != handle.num_tokens:
+                    raise ValueError("Cached dispatch requires the original token count")
+                if width != handle.hidden:
+                    raise ValueError("Cached dispatch requires the original hidden size")
+            else:
+                if not self._check_tensor(topk_idx, torch.int64) or topk_idx.ndim != 2 or topk_idx.shape[0] != tokens:
+                    raise ValueError("topk_idx must be contiguous int64 [T,K] on the buffer GPU")
+                if not do_handle_copy and torch.is_inference(topk_idx):
+                    raise ValueError("Inference routing tensors require do_handle_copy=True")
+                topk = topk_idx.shape[1]
+            _integer("tokens", tokens, 1, MAX_TOKENS * world)
+            _integer("topk", topk, 1, MAX_TOPK)
+            _integer("experts", num_experts, world, MAX_EXPERTS)
+            if num_experts % world:
+                raise ValueError("num_experts must be divisible by EP")
+            bound = self.num_max_tokens_per_rank
+            per_rank = -(-tokens // world)
+            capacity = (bound or per_rank) if num_max_tokens_per_rank is None else num_max_tokens_per_rank
+            _integer("num_max_tokens_per_rank", capacity, per_rank, MAX_TOKENS)
+            if bound and capacity > bound:
+                raise ValueError("Input/capacity exceeds the buffer token bound")
+            if self.num_topk and self.num_topk != topk:
+                raise ValueError("topk differs from buffer configuration")
+            if topk_weights is not None and not self._check_tensor(topk_weights, torch.float32, (tokens, topk)):
+                raise ValueError("topk_weights must be contiguous FP32 [T,K] on the buffer GPU without grad")
+
+            # ---- launch: everything from here runs on the communication stream --------------
+            try:
+                if previous_event is not None:
+                    previous_event.current_stream_wait()
+                producer = EventHandle()
+                with gpu_api().stream(runtime.stream):
+                    producer.current_stream_wait()
+                    if handle is None:
+                        handle = self._notify(hidden, topk_idx, num_experts, capacity, do_handle_copy)
+                    rows = handle.num_expanded_tokens
+                    row_to_route = handle._row_to_route_full
+                    if fuse_quant:
+                        out, out_scales, out_weights = native.dispatch_quant_fp8(
+                            hidden, topk_weights, handle.route_to_row, row_to_route, rows
+                        )
+                    else:
+                        out, out_scales, out_weights = native.dispatch_copy(
+                            hidden, scales, topk_weights, handle.route_to_row, row_to_route, rows
+                        )
+                    retained = (hidden, scales, topk_weights, out, out_scales, out_weights, handle.topk_idx) + tuple(
+                        getattr(handle, name) for name in _ROUTING
+                    )
+                    handle.metadata_only = False
+                    handle.num_compute_units = 64 if fp8 else 32
+                    handle._routing_versions = {
+                        name: (getattr(handle, name).data_ptr(), getattr(handle, name)._version) for name in _ROUTING
+                    }
+                    event = EventOverlap._from_resources(EventHandle(), retained)
+                if not async_with_compute_stream:
+                    event.current_stream_wait(release_handle=True)
+                runtime.notify_inflight = None
+                return (out, out_scales) if fp8 else out, None, out_weights, handle, event
+            except Exception:
+                runtime.notify_failed = True
+                raise
+
+    def _notify(self, hidden, topk_idx, num_experts, capacity, do_handle_copy) -> EPHandle:
+        """Routing layout + the one host read-back (counts, prefix, R) that sizes the outputs."""
+        runtime = self._runtime
+        native = runtime.native
+        tokens, width = hidden.shape
+        topk = topk_idx.shape[1]
+        local = num_experts // runtime.world_size
+        begin = runtime.rank * local
+        # Persistent routing keeps version counters even when the caller runs in inference mode.
+        with torch.inference_mode(False), torch.no_grad():
+            indices = topk_idx.clone() if do_handle_copy else topk_idx
+            plan = native.layout(runtime.workspace, indices, num_experts, begin, local)
+            summary = plan["meta"].cpu().tolist()  # counts | psum | offsets | R
+        counts = summary[:local]
+        rows = summary[3 * local + 1]
+        handle = EPHandle(
+            True, num_experts, 1, capacity, 64, indices, None, rows, counts, None, plan["psum"], plan["counts"], None,
+            None, None, None,
+        )
+        handle.route_to_row = plan["route_to_row"]
+        handle._row_to_route_full = plan["row_to_route"]
+        with torch.inference_mode(False), torch.no_grad():
+            handle.weight_return_meta = plan["row_to_route"][:rows]
+        handle.expert_totals = plan["counts"]
+        handle.expert_offsets = plan["offsets"]
+        handle.rank, handle.world_size = runtime.rank, runtime.world_size
+        handle.num_tokens, handle.num_topk, handle.hidden = tokens, topk, width
+        handle._buffer_token = self._handle_token
+        return handle
+
+    @accept_aliases(num_compute_units="num_sms")
+    def combine(
+        self,
+        x: torch.Tensor,
+        handle: EPHandle,
+        topk_weights: Optional[torch.Tensor] = None,
+        bias=None,
+        num_sms: int = 0,
+        num_qps: int = 0,
+        previous_event: EventHandle = None,
+        previous_event_before_epilogue: Optional[EventHandle] = None,
+        async_with_compute_stream: bool = False,
+        allocate_on_comm_stream: bool = False,
+    ):
+        """Return ``(out[T,H] bf16, out_weights[T,K] | None, event)``.
+
+        High-throughput handles: unweighted fp32 sum of each token's expert rows in slot order, one
+        rounding to BF16; ``topk_weights[R]`` travel on the separate return channel and come back as
+        ``[T,K]`` with 0 in slots without a row.  Low-latency style handles (``is_low_latency``):
+        the saved ``handle.source_weights`` multiply each row before the sum.
+        """
+        runtime = self._live_runtime()
+        runtime.ensure_alive()
+        native = runtime.native
+        with runtime.notify_lock:
+            if runtime.notify_failed:
+                raise RuntimeError("A previous communication launch failed; restart the distributed job")
+            if type(async_with_compute_stream) is not bool or type(allocate_on_comm_stream) is not bool:
+                raise TypeError("Stream options must be bool")
+            if bias is not None:
+                raise NotImplementedError("Combine currently supports bias=None")
+            if previous_event_before_epilogue is not None or allocate_on_comm_stream:
+                raise NotImplementedError("Epilogue events and allocate_on_comm_stream are unavailable")
+            if type(num_sms) is not int or num_sms not in (0, 64):
+                raise ValueError("Combine uses 64 compute units; num_compute_units=0/64")
+            if type(num_qps) is not int or num_qps not in (0, 2):
+                raise ValueError("Combine uses two QPs per cross sender; num_qps=0/2")
+            if previous_event is not None and (
+                not isinstance(previous_event, EventHandle) or previous_event._device != runtime.device
+            ):
+                raise ValueError("previous_event must belong to the buffer GPU")
+            if (
+                not isinstance(handle, EPHandle)
+                or handle._buffer_token is not self._handle_token
+                or handle.metadata_only
+                or handle.metadata_version != 7
+            ):
+                raise ValueError("Combine needs this buffer's successful expanded payload dispatch handle")
+            if not handle.do_expand or handle.expert_alignment != 1:
+                raise ValueError("Combine supports expanded layout without padding")
+            if handle.rank != runtime.rank or handle.world_size != runtime.world_size:
+                raise ValueError("Handle topology differs from the buffer")
+            self._check_versions(handle)
+            rows = handle.num_expanded_tokens
+            if not self._check_tensor(x, torch.bfloat16, (rows, handle.hidden)):
+                raise ValueError(
+                    "x must be contiguous BF16 [num_expanded_tokens,H] matching the handle on the buffer GPU without grad"
+                )
+            if topk_weights is not None and not self._check_tensor(topk_weights, torch.float32, (rows,)):
+                raise ValueError(
+                    "topk_weights must be contiguous FP32 [num_expanded_tokens] on the buffer GPU without grad"
+                )
+            weighted = handle.is_low_latency
+            if weighted and handle.source_weights is None:
+                raise ValueError("Low-latency handle carries no saved route weights")
+            try:
+                if previous_event is not None:
+                    previous_event.current_stream_wait()
+                producer = EventHandle()
+                with gpu_api().stream(runtime.stream):
+                    producer.current_stream_wait()
+                    output, output_weights = native.combine(
+                        x, handle.route_to_row, handle.source_weights if weighted else None, topk_weights
+                    )
+                    retained = (x, topk_weights, output, output_weights, handle.topk_idx) + tuple(
+                        getattr(handle, name) for name in _ROUTING
+                    )
+                    event = EventOverlap._from_resources(EventHandle(), retained)
+                if not async_with_compute_stream:
+                    event.current_stream_wait(release_handle=True)
+                runtime.notify_inflight = None
+                return output, output_weights, event
+            except Exception:
+                runtime.notify_failed = True
+                raise

@@ -1,0 +1,34 @@
+"""Tensor helpers with the reference's names (deep_ep/utils/math.py:45-79)."""
+
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+
+from . import ops
+
+
+def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Quantise each group of 128 values to E4M3 with FP32 scales, on the GPU (HIP kernel).
+
+    Bit-identical to the reference's torch expression on CPU.  ``x`` must be a contiguous BF16
+    [T, H] GPU tensor with H a multiple of 128 (the reference zero-pads other widths)."""
+    if x.dim() != 2:
+        raise AssertionError("x must be a 2D tensor")
+    return ops.cast_to_fp8(x)
+
+
+def per_token_cast_back(x_fp8: torch.Tensor, x_scales: torch.Tensor) -> torch.Tensor:
+    """bf16(fp32(q) * scale); int32 scales are four packed e8m0 bytes of which the low one is used."""
+    if x_fp8.numel() == 0:
+        return x_fp8.to(torch.bfloat16)
+    if x_fp8.dim() != 2:
+        raise AssertionError("x_fp8 must be a 2D tensor")
+    tokens, hidden = x_fp8.shape
+    if hidden % 128:
+        raise ValueError("hidden must be a multiple of 128")
+    if x_scales.dtype == torch.int:
+        x_scales = (x_scales.view(dtype=torch.uint8).to(torch.int) << 23).view(dtype=torch.float)
+    values = x_fp8.to(torch.float32).view(tokens, -1, 128)
+    return (values * x_scales.view(tokens, -1, 1)).view(tokens, hidden).to(torch.bfloat16)
