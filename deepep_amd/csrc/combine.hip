@@ -17,7 +17,8 @@ namespace {
 constexpr int kMaxThreads = 256;
 constexpr int kBatch = 8;  // rows fetched per thread before the dependent adds start
 
-template <bool kWeighted>
+// kWeights: 0 = plain sum, 1 = weight per expert row (w[row]), 2 = weight per route (w[t*K + s]).
+template <int kWeights>
 __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ row_weights, const int* __restrict__ route_to_row,
     int num_topk, int vec_per_row, int vec_per_part, int parts, u32x4* __restrict__ out,
@@ -30,7 +31,9 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
         int row = -1;
         if (threadIdx.x < num_topk) row = route_to_row[static_cast<size_t>(token) * num_topk + threadIdx.x];
         rows[threadIdx.x] = row;
-        if (kWeighted) wts[threadIdx.x] = row >= 0 ? row_weights[row] : 0.0f;
+        if (kWeights == 1) wts[threadIdx.x] = row >= 0 ? row_weights[row] : 0.0f;
+        if (kWeights == 2)
+            wts[threadIdx.x] = row >= 0 ? row_weights[static_cast<size_t>(token) * num_topk + threadIdx.x] : 0.0f;
         if (part == 0 && return_out != nullptr && threadIdx.x < num_topk)
             return_out[static_cast<size_t>(token) * num_topk + threadIdx.x] = row >= 0 ? return_in[row] : 0.0f;
     }
@@ -51,12 +54,12 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
 #pragma unroll
             for (int j = 0; j < kBatch; ++j) {
                 if (rows[s0 + j] < 0) continue;
-                const float w = kWeighted ? wts[s0 + j] : 1.0f;
+                const float w = kWeights != 0 ? wts[s0 + j] : 1.0f;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float lo = bf16_to_f32(val[j][i] & 0xffffu);
                     float hi = bf16_to_f32(val[j][i] >> 16);
-                    if (kWeighted) {
+                    if (kWeights != 0) {
                         lo = __fmul_rn(lo, w);
                         hi = __fmul_rn(hi, w);
                     }
@@ -72,7 +75,36 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     }
 }
 
+struct CombineGrid {
+    int parts, per_part, threads;
+};
+
+CombineGrid combine_grid(int num_tokens, int vec)
+{
+    CombineGrid g;
+    int parts = 1;
+    while (num_tokens * parts < 2048 && vec / (parts * 2) >= 64 && parts < 16) parts *= 2;
+    g.per_part = (vec + parts - 1) / parts;
+    g.parts = (vec + g.per_part - 1) / g.per_part;
+    int threads = (g.per_part + 63) / 64 * 64;
+    g.threads = threads > kMaxThreads ? kMaxThreads : (threads < 64 ? 64 : threads);
+    return g;
+}
+
 }  // namespace
+
+// Route-weighted reduce used by the MegaMoE forward: out[t] = bf16( sum_s w[t,s] * float(y[row(t,s)]) ).
+int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
+                   int hidden, void* out, hipStream_t stream)
+{
+    const int vec = hidden / 8;
+    const CombineGrid g = combine_grid(num_tokens, vec);
+    hipLaunchKernelGGL(combine_kernel<2>, dim3(num_tokens * g.parts), dim3(g.threads), 0, stream,
+                       static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk, vec, g.per_part, g.parts,
+                       static_cast<u32x4*>(out), nullptr, nullptr);
+    return launch_status("combine_routes");
+}
+
 }  // namespace dpep
 
 extern "C" {
@@ -91,21 +123,15 @@ int dpep_combine(const void* y, const float* row_weights, const int32_t* route_t
     DPEP_REQUIRE(route_to_row != nullptr && out != nullptr && aligned16(out), "combine: NULL or misaligned buffer");
     DPEP_REQUIRE(num_rows == 0 || (y != nullptr && aligned16(y)), "combine: y must be 16-byte aligned");
     const int vec = hidden / 8;
-    int parts = 1;
-    while (num_tokens * parts < 2048 && vec / (parts * 2) >= 64 && parts < 16) parts *= 2;
-    const int per_part = (vec + parts - 1) / parts;
-    parts = (vec + per_part - 1) / per_part;
-    int threads = (per_part + 63) / 64 * 64;
-    if (threads > kMaxThreads) threads = kMaxThreads;
-    if (threads < 64) threads = 64;
+    const CombineGrid g = combine_grid(num_tokens, vec);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (row_weights != nullptr)
-        hipLaunchKernelGGL(combine_kernel<true>, dim3(num_tokens * parts), dim3(threads), 0, s,
-                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, per_part, parts,
+        hipLaunchKernelGGL(combine_kernel<1>, dim3(num_tokens * g.parts), dim3(g.threads), 0, s,
+                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, g.per_part, g.parts,
                            static_cast<u32x4*>(out), return_in, return_out);
     else
-        hipLaunchKernelGGL(combine_kernel<false>, dim3(num_tokens * parts), dim3(threads), 0, s,
-                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, per_part, parts,
+        hipLaunchKernelGGL(combine_kernel<0>, dim3(num_tokens * g.parts), dim3(g.threads), 0, s,
+                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, g.per_part, g.parts,
                            static_cast<u32x4*>(out), return_in, return_out);
     return launch_status("combine");
 }

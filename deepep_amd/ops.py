@@ -216,3 +216,76 @@ def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
         )
     _lib.check(status, "combine")
     return out, returned
+
+
+# ---------------------------------------------------------------------------------------------
+# MegaMoE (W4A8) entry points
+# ---------------------------------------------------------------------------------------------
+def mx_quant(x):
+    """MXFP8 activation quantiser: BF16 [B,H] -> (e4m3 codes [B,H] as float8_e4m3fn, e8m0 bytes [B,H/32] uint8)."""
+    lib = _lib.load()
+    _require("x", x, torch.bfloat16)
+    if x.ndim != 2 or x.shape[1] % 32:
+        raise ValueError("x must be [B, H] with H a multiple of 32")
+    rows, hidden = x.shape
+    codes = torch.empty((rows, hidden), dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty((rows, hidden // 32), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        status = lib.dpep_mx_quant(_ptr(x), rows, hidden, _ptr(codes), _ptr(scales), _stream(x.device))
+    _lib.check(status, "mx_quant")
+    return codes, scales
+
+
+def megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local) -> int:
+    return int(_lib.load().dpep_megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local))
+
+
+def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
+    """Raw packed FP4 uint8 [L,N,K/2] + e8m0 uint8 [L,N,K/32] -> the kernel's streaming order (same sizes)."""
+    lib = _lib.load()
+    _require("w_packed", w_packed, torch.uint8)
+    if w_packed.ndim != 3:
+        raise ValueError("w_packed must be [L, N, K/2]")
+    experts, n, half_k = w_packed.shape
+    k = half_k * 2
+    _require("w_scales", w_scales.reshape(experts, n, -1), torch.uint8, (experts, n, k // 32), w_packed.device)
+    out_w = torch.empty_like(w_packed)
+    out_s = torch.empty((experts, n, k // 32), dtype=torch.uint8, device=w_packed.device)
+    with torch.cuda.device(w_packed.device):
+        status = lib.dpep_megamoe_prepare_weights(
+            _ptr(w_packed), _ptr(w_scales), experts, n, k, int(bool(gate_up)), _ptr(out_w), _ptr(out_s),
+            _stream(w_packed.device),
+        )
+    _lib.check(status, "megamoe_prepare_weights")
+    return out_w, out_s
+
+
+def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s2, num_experts, expert_begin,
+                    num_local, y, expert_token_nums):
+    """Fused W4A8 forward of one rank's local experts; writes y [B,H] BF16 and expert_token_nums [L] int32."""
+    lib = _lib.load()
+    dev = ws.device
+    _require("x_codes", x_codes, torch.float8_e4m3fn, device=dev)
+    tokens, hidden = x_codes.shape
+    _require("x_scales", x_scales, torch.uint8, (tokens, hidden // 32), dev)
+    _require("topk_idx", topk_idx, torch.int32, device=dev)
+    topk = topk_idx.shape[1]
+    _require("topk_idx", topk_idx, torch.int32, (tokens, topk), dev)
+    _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)
+    _require("w1", w1, torch.uint8, device=dev)
+    if w1.ndim != 3 or w1.shape[0] != num_local or w1.shape[2] * 2 != hidden or w1.shape[1] % 2:
+        raise ValueError("w1 must be prepared [L, 2I, H/2]")
+    intermediate = w1.shape[1] // 2
+    _require("s1", s1, torch.uint8, (num_local, 2 * intermediate, hidden // 32), dev)
+    _require("w2", w2, torch.uint8, (num_local, hidden, intermediate // 2), dev)
+    _require("s2", s2, torch.uint8, (num_local, hidden, intermediate // 32), dev)
+    _require("y", y, torch.bfloat16, (tokens, hidden), dev)
+    _require("expert_token_nums", expert_token_nums, torch.int32, (num_local,), dev)
+    with torch.cuda.device(dev):
+        status = lib.dpep_megamoe_forward(
+            ws.handle, _ptr(x_codes), _ptr(x_scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(w1), _ptr(s1), _ptr(w2),
+            _ptr(s2), tokens, hidden, intermediate, topk, num_experts, expert_begin, num_local, _ptr(y),
+            _ptr(expert_token_nums), _stream(dev),
+        )
+    _lib.check(status, "megamoe_forward")
+    return y, expert_token_nums

@@ -104,9 +104,11 @@ size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, in
 
 /* One-off weight re-layout (transform_weights_for_mega_moe, experiments/megamoe/python/.../api.py:311-379):
  * raw packed FP4 [L,N,K/2] + e8m0 [L,N,K/32]  ->  the tile order the GEMM kernel streams.
- * Byte shuffle only; out buffers have the same sizes as the inputs. */
+ * Byte shuffle only; out buffers have the same sizes as the inputs.  gate_up != 0 (first GEMM, N = 2I,
+ * gate rows then up rows) interleaves gate and up in groups of 32 output columns so SwiGLU is lane-local
+ * (the counterpart of _interleave_gate_up_128, api.py:285-293). */
 int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scales, int num_local, int n,
-                                 int k, uint8_t* out_packed, uint8_t* out_scales, void* stream);
+                                 int k, int gate_up, uint8_t* out_packed, uint8_t* out_scales, void* stream);
 
 /* Fused W4A8 MoE forward for one rank's local experts (Plan::forward, experiments/megamoe/csrc/forward.cpp:340-478
  * -> mega_moe_kernel_do, kernel_launch.hpp:8-13):

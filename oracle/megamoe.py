@@ -98,14 +98,18 @@ def quantize_weight_mxfp4(w):
     amax = np.abs(blocks).max(axis=-1)
     biased = (np.maximum(amax, np.float32(2.0**-125)).astype(np.float32).view(np.uint32) >> np.uint32(23)).astype(np.int32)
     byte = np.clip(biased - 2, 0, 254)
-    scaled = (blocks.astype(np.float64) * np.exp2(127.0 - byte)[..., None]).astype(np.float32)
+    scaled = blocks * np.exp2(127.0 - byte).astype(np.float32)[..., None]
     mag = np.minimum(np.abs(scaled), np.float32(6.0))
-    grid = E2M1[:8]
-    upper = np.searchsorted(grid, mag).clip(0, 7)
-    lower = np.maximum(upper - 1, 0)
-    d_lo, d_hi = mag - grid[lower], grid[upper] - mag
-    take_low = (d_lo < d_hi) | ((d_lo == d_hi) & (lower % 2 == 0))
-    nibble = np.where(take_low, lower, upper).astype(np.uint8) | (np.signbit(scaled).astype(np.uint8) << 3)
+    # nearest e2m1 magnitude, ties to the even code: count the rounding boundaries passed
+    # (0.25 -> 0, 0.75 -> 1.0, 1.25 -> 1.0, 1.75 -> 2.0, 2.5 -> 2.0, 3.5 -> 4.0, 5.0 -> 4.0).
+    code = (mag > 0.25).astype(np.uint8)
+    code += mag >= 0.75
+    code += mag > 1.25
+    code += mag >= 1.75
+    code += mag > 2.5
+    code += mag >= 3.5
+    code += mag > 5.0
+    nibble = code | (np.signbit(scaled).astype(np.uint8) << 3)
     nibble = nibble.reshape(*w.shape[:-1], k)
     packed = (nibble[..., 0::2] | (nibble[..., 1::2] << 4)).astype(np.uint8)
     return packed, byte.astype(np.uint8).reshape(*w.shape[:-1], k // 64, 2)

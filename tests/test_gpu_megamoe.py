@@ -1,0 +1,114 @@
+"""GPU parity of the W4A8 path: MX quantiser bit-exact; fused forward within 2e-2 relative Frobenius error
+of the fp32 dequantised oracle (oracle/megamoe.py, restating the reference's NumPy oracle)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import megamoe as mm
+from tests.gpu_util import bf16_bits, fp8_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from deepep_amd import ops as module
+
+    return module
+
+
+@pytest.mark.parametrize("scale", [1.0, 1e-3, 500.0, 1e-30, 1e30])
+def test_mx_quant_bit_exact(ops, scale):
+    gen = torch.Generator().manual_seed(3)
+    x = (torch.randn(77, 1024, generator=gen) * scale).bfloat16()
+    x[0, :32] = 0
+    x[1, :32] = 448.0
+    x[2, 5] = 3.0e38
+    codes, scales = ops.mx_quant(x.cuda())
+    ref_codes, ref_scales = mm.mx_quantize(x.float().numpy())
+    np.testing.assert_array_equal(scales.cpu().numpy(), ref_scales)
+    np.testing.assert_array_equal(fp8_bits(codes), ref_codes)
+
+
+def test_mx_quant_reference_anchors(ops):
+    # experiments/megamoe/tests/test_reference.py:37-45
+    x = torch.full((2, 64), 0.5)
+    x[:, 32:] = 4.0
+    codes, scales = ops.mx_quant(x.bfloat16().cuda())
+    assert scales.cpu().tolist() == [[118, 121], [118, 121]]
+    np.testing.assert_array_equal(mm.mx_dequantize(fp8_bits(codes), scales.cpu().numpy()), x.numpy())
+    codes, scales = ops.mx_quant(torch.zeros(1, 32, dtype=torch.bfloat16).cuda())
+    assert not fp8_bits(codes).any() and not scales.cpu().numpy().any()
+
+
+def _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=0):
+    rng = np.random.default_rng(seed)
+    x = (rng.normal(size=(tokens, hidden))).astype(np.float32)
+    x_codes, x_scales = mm.mx_quantize(x)
+    w1 = (rng.normal(size=(local, 2 * inter, hidden)) * 0.02).astype(np.float32)
+    w2 = (rng.normal(size=(local, hidden, inter)) * 0.02).astype(np.float32)
+    p1, s1 = mm.quantize_weight_mxfp4(w1)
+    p2, s2 = mm.quantize_weight_mxfp4(w2)
+    idx = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int32)
+    weights = rng.random((tokens, topk)).astype(np.float32)
+    weights /= weights.sum(axis=1, keepdims=True)
+    return x_codes, x_scales, (p1, s1), (p2, s2), idx, weights
+
+
+def _oracle(x_codes, x_scales, l1, l2, idx, weights, begin):
+    xq = mm.mx_dequantize(x_codes, x_scales)
+    d1 = mm.unpack_weight(*l1)
+    d2 = mm.unpack_weight(*l2)
+    return mm.round_bf16(mm.local_reference(xq, idx, weights, d1, d2, begin))
+
+
+def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local):
+    tokens, hidden = x_codes.shape
+    inter = l2[0].shape[2] * 2
+    dev = "cuda"
+    w1, s1 = ops.megamoe_prepare_weights(torch.from_numpy(l1[0]).to(dev), torch.from_numpy(l1[1]).reshape(local, 2 * inter, -1).to(dev), True)
+    w2, s2 = ops.megamoe_prepare_weights(torch.from_numpy(l2[0]).to(dev), torch.from_numpy(l2[1]).reshape(local, hidden, -1).to(dev), False)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, idx.shape[1], hidden, inter, local))
+    y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+    ops.megamoe_forward(
+        ws, torch.from_numpy(x_codes).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(x_scales).to(dev),
+        torch.from_numpy(idx).to(dev), torch.from_numpy(weights).to(dev), w1, s1, w2, s2, experts, begin, local, y, counts,
+    )
+    torch.cuda.synchronize()
+    out = y.float().cpu().numpy(), counts.cpu().numpy()
+    ws.destroy()
+    return out
+
+
+@pytest.mark.parametrize(
+    "tokens,hidden,inter,experts,begin,local,topk",
+    [
+        (64, 256, 256, 4, 0, 4, 2),      # every expert local, tiny
+        (300, 512, 256, 8, 2, 3, 4),     # ragged rows, local range inside E, partial tiles
+        (257, 1024, 512, 6, 0, 6, 6),    # every token hits every expert
+        (96, 256, 256, 8, 6, 2, 1),      # some local experts may be empty
+    ],
+)
+def test_megamoe_forward_matches_oracle(ops, tokens, hidden, inter, experts, begin, local, topk):
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, begin, local, topk)
+    got, counts = _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local)
+    want = _oracle(x_codes, x_scales, l1, l2, idx, weights, begin)
+    np.testing.assert_array_equal(counts, np.bincount(idx.ravel(), minlength=experts)[begin : begin + local])
+    assert np.isfinite(got).all()
+    err = mm.relative_frobenius(got, want)
+    assert err <= 2e-2, err
+    untouched = ~((idx >= begin) & (idx < begin + local)).any(axis=1)
+    assert not got[untouched].any()  # tokens without a local expert receive zeros
+
+
+def test_megamoe_forward_rank_share_shape(ops):
+    # one EP rank's share at reduced token count: H=7168, I=2048, 6 local experts of 384, top-8
+    tokens, hidden, inter, experts, local, topk = 2048, 7168, 2048, 384, 6, 8
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, local, topk, seed=1)
+    got, counts = _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, 0, local)
+    want = _oracle(x_codes, x_scales, l1, l2, idx, weights, 0)
+    np.testing.assert_array_equal(counts, np.bincount(idx.ravel(), minlength=experts)[:local])
+    err = mm.relative_frobenius(got, want)
+    assert err <= 2e-2, err
