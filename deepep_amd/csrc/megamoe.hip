@@ -130,10 +130,22 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
 // =====================================================================================================
 // Grouped GEMM
 // =====================================================================================================
+// Workgroup = 4 waves (2 row halves x 2 column halves), tile 128 rows x 256 columns, k tile 128.
+// Everything the main loop reads arrives through asynchronous global->LDS copies into a ring of
+// kStages k tiles; the only synchronisation per k tile is one vmcnt wait plus one barrier.
 constexpr int kBM = 128;           // rows per workgroup tile
-constexpr int kBK = 128;           // k bytes of A staged in LDS per step (two MFMA k steps of 64)
-constexpr int kAStride = kBK + 16; // padded LDS row: 16 consecutive rows hit 16 distinct 16-byte slots
-constexpr int kGemmThreads = 256;  // 4 waves: 2 (rows) x 2 (columns)
+constexpr int kBK = 128;           // k per LDS stage (two MFMA k steps of 64)
+constexpr int kCT = 4;             // 32-column MFMA tiles per wave
+constexpr int kBN = 2 * kCT * 32;  // columns per workgroup tile
+constexpr int kGemmThreads = 256;
+constexpr int kStages = 4;         // LDS ring depth; copies run kStages-1 k tiles ahead
+constexpr int kStageA = 0;                         // 128 rows x 128 B, 16-byte chunks XOR-swizzled
+constexpr int kStageB = kBM * kBK;                 // 8 column tiles x 2 k steps x 1 KiB fragments
+constexpr int kStageSA = kStageB + kBN * 64;       // 128 row scale words (+128 duplicates)
+constexpr int kStageSB = kStageSA + 1024;          // 8 column tiles x 64 lanes x 2 B
+constexpr int kStageBytes = kStageSB + 1024;
+constexpr int kCopiesPerTile = 10;                 // per thread: 4 A + 4 B + 1 A-scale + 1 B-scale
+constexpr int kGemmLdsBytes = kStages * kStageBytes;
 
 struct GemmParams {
     const uint8_t* a_codes;    // [*, K] e4m3
@@ -150,26 +162,45 @@ struct GemmParams {
     uint16_t* out;             // second GEMM: [rows, N] bf16
 };
 
+// gate / (1 + exp(-gate)) * up with the hardware exponential and reciprocal (about 1 ulp each; the
+// result is rounded to BF16 right after).  The clamp keeps exp finite, like the reference's clip(+-80).
 __device__ __forceinline__ float silu_mul(float gate, float up)
 {
     const float clipped = fminf(fmaxf(-gate, -80.0f), 80.0f);
-    return gate / (1.0f + expf(clipped)) * up;
+    return gate * __frcp_rn(1.0f + __expf(clipped)) * up;
 }
 
-// CT = 32-column MFMA tiles per wave (workgroup covers 2*CT*32 columns); kGateUp selects the epilogue.
-template <int CT, bool kGateUp>
+// Asynchronous copy global -> LDS: lane l's bytes land at lds_base + l * size.  lds_base is wave-uniform.
+// Written as assembly so that the compiler's own wait-count bookkeeping does not serialise the ring;
+// completion is awaited explicitly with wait_copies<N>().
+__device__ __forceinline__ void copy16_to_lds(const void* src, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(src) : "memory");
+}
+__device__ __forceinline__ void copy4_to_lds(const void* src, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(src) : "memory");
+}
+template <int kOutstanding>
+__device__ __forceinline__ void wait_copies_then_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
+}
+
+template <bool kGateUp>
 __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParams p)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][kBM * kAStride];
-    __shared__ uint32_t lds_sa[2][kBM];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     __shared__ int tile_base[DPEP_MAX_LOCAL_EXPERTS + 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int g = lane >> 5, lr = lane & 31;
-    constexpr int kBN = 2 * CT * 32;
     const int n_tiles = p.n / kBN;
     const int ksteps = p.k / 64, ktiles = p.k / kBK;
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
 
     // Tiles per expert: ceil(rows/128) row tiles x n_tiles column tiles, expert-major.
     if (tid == 0) {
@@ -189,6 +220,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     const int per_xcd = (gridDim.x + 7) / 8;
     const int first = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
 
+    // Per-thread constants of the copy pattern.
+    const int a_swizzle = (wave * 4 + (lane >> 4)) & 7;            // ((row >> 1) & 7) of this thread's A rows
+    const int a_chunk = ((lane & 7) ^ a_swizzle) * 16;              // byte offset inside the 128-byte k tile
+    const uint32_t lds_wave_a = wave * 1024;                        // + copy * 4096
+    const uint32_t lds_wave_s = wave * 256;
+
     for (int tile = first; tile < total_tiles; tile += per_xcd * 8) {
         int e = 0;
         while (tile >= tile_base[e + 1]) ++e;
@@ -199,139 +236,169 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         const int m0 = mt * kBM;
         const int valid_rows = min(kBM, rows - m0);
 
-        // ---- A loader: 128 rows x 8 chunks of 16 bytes = 4 chunks per thread ----
-        const int a_col = (tid & 7) * 16;
+        // A: copy i of wave w fills LDS rows i*32 + w*8 + lane/8.
         const uint8_t* a_src[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int r = min((tid >> 3) + 32 * i, valid_rows - 1);
+            const int r = min(i * 32 + wave * 8 + (lane >> 3), valid_rows - 1);
             int src = row_begin + m0 + r;
             if (p.row_to_route != nullptr) src = p.row_to_route[src] / p.topk;
-            a_src[i] = p.a_codes + static_cast<size_t>(src) * p.k + a_col;
+            a_src[i] = p.a_codes + static_cast<size_t>(src) * p.k + a_chunk;
         }
-        const uint8_t* sa_src = nullptr;
-        if (tid < kBM) {
-            const int r = min(tid, valid_rows - 1);
+        const uint8_t* sa_src;
+        {
+            const int r = min(tid & (kBM - 1), valid_rows - 1);
             int src = row_begin + m0 + r;
             if (p.row_to_route != nullptr) src = p.row_to_route[src] / p.topk;
             sa_src = p.a_scales + static_cast<size_t>(src) * (p.k / 32);
         }
+        // B: fragment q = copy*4 + wave of the 16 (column tile, k step) fragments of one k tile.
+        const uint8_t* w_block = p.w + static_cast<size_t>(e) * p.n * (p.k / 2) +
+                                 static_cast<size_t>(nt) * (2 * kCT) * ksteps * 1024 + lane * 16;
+        const uint8_t* b_src[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int q = j * 4 + wave;
+            b_src[j] = w_block + (static_cast<size_t>(q >> 1) * ksteps + (q & 1)) * 1024;
+        }
+        const uint8_t* sb_src = p.ws + static_cast<size_t>(e) * p.n * (p.k / 32) +
+                                (static_cast<size_t>(nt) * (2 * kCT) + (tid >> 5)) * ktiles * 128 + (tid & 31) * 4;
 
-        // ---- B fragments: prepared layout, [expert][column tile][k step][lane][16 B] ----
-        const int ctile0 = nt * (2 * CT) + wn * CT;
-        const uint8_t* w_base = p.w + static_cast<size_t>(e) * p.n * (p.k / 2) +
-                                static_cast<size_t>(ctile0) * ksteps * 1024 + lane * 16;
-        const uint8_t* ws_base = p.ws + static_cast<size_t>(e) * p.n * (p.k / 32) +
-                                 static_cast<size_t>(ctile0) * ktiles * 128 + lane * 2;
+        auto issue_tile = [&](int kt) {
+            const uint32_t stage = lds0 + (kt & (kStages - 1)) * kStageBytes;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                copy16_to_lds(a_src[i] + static_cast<size_t>(kt) * kBK, stage + kStageA + i * 4096 + lds_wave_a);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                copy16_to_lds(b_src[j] + static_cast<size_t>(kt) * 2048, stage + kStageB + (j * 4 + wave) * 1024);
+            copy4_to_lds(sa_src + kt * 4, stage + kStageSA + lds_wave_s);
+            copy4_to_lds(sb_src + kt * 128, stage + kStageSB + lds_wave_s);
+        };
 
-        v16f acc[2][CT];
+        v16f acc[2][kCT];
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int c = 0; c < CT; ++c)
+            for (int c = 0; c < kCT; ++c)
 #pragma unroll
                 for (int j = 0; j < 16; ++j) acc[i][c][j] = 0.0f;
 
-        // Prologue: A tile 0 to LDS, A tile 1 into staging registers, B ring primed with k steps 0..3.
-        u32x4 stage[4];
-        uint32_t stage_s = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) stage[i] = load16(a_src[i]);
-        if (tid < kBM) stage_s = *reinterpret_cast<const uint32_t*>(sa_src);
-        u32x4 bring[4][CT];
-        uint32_t bscale[2][CT];
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-#pragma unroll
-            for (int c = 0; c < CT; ++c)
-                bring[s][c] = load16(w_base + (static_cast<size_t>(c) * ksteps + s) * 1024);
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int c = 0; c < CT; ++c)
-                bscale[t][c] = *reinterpret_cast<const uint16_t*>(ws_base + (static_cast<size_t>(c) * ktiles + t) * 128);
-        __syncthreads();  // previous tile's LDS reads are complete
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<u32x4*>(&lds_a[0][((tid >> 3) + 32 * i) * kAStride + a_col]) = stage[i];
-        if (tid < kBM) lds_sa[0][tid] = stage_s;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) stage[i] = load16(a_src[i] + kBK);
-        if (tid < kBM) stage_s = *reinterpret_cast<const uint32_t*>(sa_src + 4);
-        __syncthreads();
+        for (int kt = 0; kt < kStages - 1; ++kt) issue_tile(min(kt, ktiles - 1));
 
-        // Main loop over pairs of k tiles (k = 256 per iteration; K is a multiple of 256).
-        for (int kt2 = 0; kt2 < ktiles; kt2 += 2) {
+        // Fragment addresses inside a stage.
+        int a_addr[2][2][2];  // [row tile][k step][lo/hi 16 bytes]
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int kt = kt2 + half;
-                const uint8_t* a_tile = lds_a[half];
+        for (int i = 0; i < 2; ++i) {
+            const int row = wm * 64 + i * 32 + lr;
+            const int sw = (row >> 1) & 7;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    const int ring = half * 2 + kb;
-                    v8i afrag[2];
-                    int ascale[2];
-#pragma unroll
-                    for (int i = 0; i < 2; ++i) {
-                        const int row = wm * 64 + i * 32 + lr;
-                        const u32x4 lo = *reinterpret_cast<const u32x4*>(a_tile + row * kAStride + kb * 64 + g * 16);
-                        const u32x4 hi = *reinterpret_cast<const u32x4*>(a_tile + row * kAStride + kb * 64 + 32 + g * 16);
-                        afrag[i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-                        ascale[i] = static_cast<int>(lds_sa[half][row] >> (8 * g));
-                    }
-#pragma unroll
-                    for (int c = 0; c < CT; ++c) {
-                        const u32x4 b = bring[ring][c];
-                        const v8i bfrag = v8i{(int)b[0], (int)b[1], (int)b[2], (int)b[3], 0, 0, 0, 0};
-                        const int bs = static_cast<int>(bscale[half][c]);
-#pragma unroll
-                        for (int i = 0; i < 2; ++i) {
-                            if (kb == 0)
-                                acc[i][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(afrag[i], bfrag, acc[i][c], 0, 4, 0,
-                                                                                            ascale[i], 0, bs);
-                            else
-                                acc[i][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(afrag[i], bfrag, acc[i][c], 0, 4, 2,
-                                                                                            ascale[i], 1, bs);
-                        }
-                    }
-                    // Refill this ring slot with the k step four ahead.
-                    const int next_ks = kt * 2 + kb + 4;
-                    if (next_ks < ksteps) {
-#pragma unroll
-                        for (int c = 0; c < CT; ++c)
-                            bring[ring][c] = load16(w_base + (static_cast<size_t>(c) * ksteps + next_ks) * 1024);
-                    }
-                }
-                if (kt + 2 < ktiles) {
-#pragma unroll
-                    for (int c = 0; c < CT; ++c)
-                        bscale[half][c] =
-                            *reinterpret_cast<const uint16_t*>(ws_base + (static_cast<size_t>(c) * ktiles + kt + 2) * 128);
-                }
-                // Staged A tile kt+1 goes to the other buffer; then fetch tile kt+2.
-                if (kt + 1 < ktiles) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        *reinterpret_cast<u32x4*>(&lds_a[half ^ 1][((tid >> 3) + 32 * i) * kAStride + a_col]) = stage[i];
-                    if (tid < kBM) lds_sa[half ^ 1][tid] = stage_s;
-                    if (kt + 2 < ktiles) {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) stage[i] = load16(a_src[i] + static_cast<size_t>(kt + 2) * kBK);
-                        if (tid < kBM) stage_s = *reinterpret_cast<const uint32_t*>(sa_src + (kt + 2) * 4);
-                    }
-                }
-                __syncthreads();
+            for (int kb = 0; kb < 2; ++kb) {
+                a_addr[i][kb][0] = kStageA + row * kBK + (((kb * 4 + g) ^ sw) << 4);
+                a_addr[i][kb][1] = kStageA + row * kBK + (((kb * 4 + 2 + g) ^ sw) << 4);
             }
         }
+        const int sa_addr = kStageSA + (wm * 64 + lr) * 4;
+        const int b_addr = kStageB + wn * kCT * 2048 + lane * 16;
+        const int sb_addr = kStageSB + wn * kCT * 128 + lane * 2;
 
-        // ---- Epilogue ----
-        const int out_row0 = row_begin + m0 + wm * 64;
-        if (kGateUp) {
-            // Column tiles alternate gate / up for the same 32 activation columns: SwiGLU is lane-local.
-            const int act_width = p.n / 2;
+        // Software pipeline over k steps of 64: while the MFMAs of one k step run, the fragments of the
+        // next one are already on their way out of LDS.  Per k tile there is one wait + barrier, placed
+        // between the two k steps so that the reads issued right after it have a full k step to land.
+        v8i afrag[2][2];     // [k step][row tile]
+        u32x4 bfrag[2][kCT]; // [k step][column tile]
+        int ascale[2][2];    // [current/next k tile][row tile]
+        int bscale[2][kCT];
+        auto read_step = [&](const uint8_t* stage, int kb) {
 #pragma unroll
-            for (int pair = 0; pair < CT / 2; ++pair) {
-                const int act_col0 = (nt * CT + wn * (CT / 2) + pair) * 32;
+            for (int i = 0; i < 2; ++i) {
+                const u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][0]);
+                const u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][1]);
+                afrag[kb][i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+            }
+#pragma unroll
+            for (int c = 0; c < kCT; ++c) bfrag[kb][c] = *reinterpret_cast<const u32x4*>(stage + b_addr + (c * 2 + kb) * 1024);
+        };
+        auto read_scales = [&](const uint8_t* stage, int slot) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(stage + sa_addr + i * 128));
+#pragma unroll
+            for (int c = 0; c < kCT; ++c)
+                bscale[slot][c] = static_cast<int>(*reinterpret_cast<const uint16_t*>(stage + sb_addr + c * 128));
+        };
+        auto mfma_step = [&](int kb, int slot) {
+            // The row-scale word holds the four k blocks of the tile; the upper lane half owns the odd ones.
+            // (Shifted here, not at the read, so that the read does not have to be waited for early.)
+            const int sa0 = ascale[slot][0] >> (8 * g), sa1 = ascale[slot][1] >> (8 * g);
+#pragma unroll
+            for (int c = 0; c < kCT; ++c) {
+                const u32x4 b = bfrag[kb][c];
+                const v8i bf = v8i{(int)b[0], (int)b[1], (int)b[2], (int)b[3], 0, 0, 0, 0};
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+#ifdef DPEP_DEBUG_NO_MFMA
+                    acc[i][c][0] += __int_as_float(afrag[kb][i][0] ^ bf[0] ^ (i ? sa1 : sa0) ^ bscale[slot][c]);
+#else
+                    if (kb == 0)
+                        acc[i][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(afrag[0][i], bf, acc[i][c], 0, 4, 0,
+                                                                                    i ? sa1 : sa0, 0, bscale[slot][c]);
+                    else
+                        acc[i][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(afrag[1][i], bf, acc[i][c], 0, 4, 2,
+                                                                                    i ? sa1 : sa0, 1, bscale[slot][c]);
+#endif
+                }
+            }
+        };
+
+        // k tile 0 has landed once each thread has at most kStages-2 tiles of its own copies in flight.
+        wait_copies_then_barrier<(kStages - 2) * kCopiesPerTile>();
+        read_step(lds, 0);
+        read_scales(lds, 0);
+        for (int kt2 = 0; kt2 < ktiles; kt2 += 2) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {  // unrolled by two so the scale slots are compile-time
+                const int kt = kt2 + half;
+                const uint8_t* stage = lds + (kt & (kStages - 1)) * kStageBytes;
+                const uint8_t* next_stage = lds + ((kt + 1) & (kStages - 1)) * kStageBytes;
+#ifndef DPEP_DEBUG_NO_READ
+                read_step(stage, 1);
+#endif
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_step(0, half);
+                __builtin_amdgcn_sched_barrier(0);
+                // k tile kt+1 has landed everywhere, and every wave is past its reads of the stage that
+                // the next copies overwrite (the one read during k tile kt-1).
+#ifndef DPEP_DEBUG_NO_BARRIER
+                wait_copies_then_barrier<(kStages - 3) * kCopiesPerTile>();
+#endif
+#ifndef DPEP_DEBUG_NO_COPY
+                issue_tile(min(kt + kStages - 1, ktiles - 1));
+#endif
+#ifndef DPEP_DEBUG_NO_READ
+                read_step(next_stage, 0);
+                read_scales(next_stage, half ^ 1);
+#endif
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_step(1, half);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // Drain the tail copies and make sure every wave has left the ring before it is refilled.
+        wait_copies_then_barrier<0>();
+
+        // ---- Epilogue: through LDS (the ring is idle now) so that global stores are 16 bytes wide ----
+        const int out_row0 = row_begin + m0 + wm * 64;
+        const int wave_rows = min(64, valid_rows - wm * 64);  // may be <= 0 for the lower row half
+        if (kGateUp) {
+            // Column tiles alternate gate / up for the same 32 activation columns, so SwiGLU is lane-local.
+            // The wave's 64 rows x 64 activation columns are staged as BF16 (row stride 144 B), then each
+            // lane requantises one row: two blocks of 32 -> e8m0 byte + 32 e4m3 codes each.
+            constexpr int kRowStride = 144;
+            uint8_t* region = lds + wave * (64 * kRowStride);
+#pragma unroll
+            for (int pair = 0; pair < kCT / 2; ++pair) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -339,35 +406,74 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                         const int r = i * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
                         const float gate = bf16_to_f32(f32_to_bf16(acc[i][2 * pair][j]));
                         const float up = bf16_to_f32(f32_to_bf16(acc[i][2 * pair + 1][j]));
-                        const float act = bf16_to_f32(f32_to_bf16(silu_mul(gate, up)));
-                        float amax = fabsf(act);
-#pragma unroll
-                        for (int d = 1; d < 32; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
-                        const int byte = mx_scale_byte(amax);
-                        const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(mx_scaled(act, byte), 0.0f, 0, false);
-                        if (wm * 64 + r < valid_rows) {
-                            const size_t row = static_cast<size_t>(out_row0 + r);
-                            p.act_codes[row * act_width + act_col0 + lr] = static_cast<uint8_t>(packed & 0xff);
-                            if (lr == 0) p.act_scales[row * (act_width / 32) + (act_col0 >> 5)] = static_cast<uint8_t>(byte);
-                        }
+                        *reinterpret_cast<uint16_t*>(region + r * kRowStride + (pair * 32 + lr) * 2) =
+                            static_cast<uint16_t>(f32_to_bf16(silu_mul(gate, up)));
                     }
                 }
             }
-        } else {
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            const int act_width = p.n / 2;
+            const int act_col0 = (nt * kCT + wn * (kCT / 2)) * 32;
+            if (lane < wave_rows) {
+                const size_t row = static_cast<size_t>(out_row0 + lane);
 #pragma unroll
-            for (int c = 0; c < CT; ++c) {
-                const int col = nt * kBN + (wn * CT + c) * 32 + lr;
+                for (int blk = 0; blk < kCT / 2; ++blk) {
+                    float v[32];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const u32x4 raw = *reinterpret_cast<const u32x4*>(region + lane * kRowStride + blk * 64 + q * 16);
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            v[q * 8 + 2 * t] = bf16_to_f32(raw[t] & 0xffffu);
+                            v[q * 8 + 2 * t + 1] = bf16_to_f32(raw[t] >> 16);
+                        }
+                    }
+                    float amax = 0.0f;
+#pragma unroll
+                    for (int t = 0; t < 32; ++t) amax = fmaxf(amax, fabsf(v[t]));
+                    const int byte = mx_scale_byte(amax);
+                    u32x4 codes[2];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        codes[t >> 2][t & 3] = pack4_e4m3(mx_scaled(v[4 * t], byte), mx_scaled(v[4 * t + 1], byte),
+                                                          mx_scaled(v[4 * t + 2], byte), mx_scaled(v[4 * t + 3], byte));
+                    uint8_t* dst = p.act_codes + row * act_width + act_col0 + blk * 32;
+                    *reinterpret_cast<u32x4*>(dst) = codes[0];
+                    *reinterpret_cast<u32x4*>(dst + 16) = codes[1];
+                    p.act_scales[row * (act_width / 32) + (act_col0 >> 5) + blk] = static_cast<uint8_t>(byte);
+                }
+            }
+        } else {
+            // The wave's 64 rows x 128 columns are staged as BF16 (row stride 272 B) and leave as 16-byte
+            // chunks: 16 lanes cover one 256-byte row segment.
+            constexpr int kRowStride = 272;
+            uint8_t* region = lds + wave * (64 * kRowStride);
+#pragma unroll
+            for (int c = 0; c < kCT; ++c) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
                         const int r = i * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
-                        if (wm * 64 + r < valid_rows)
-                            p.out[static_cast<size_t>(out_row0 + r) * p.n + col] = static_cast<uint16_t>(f32_to_bf16(acc[i][c][j]));
+                        *reinterpret_cast<uint16_t*>(region + r * kRowStride + (c * 32 + lr) * 2) =
+                            static_cast<uint16_t>(f32_to_bf16(acc[i][c][j]));
                     }
                 }
             }
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            const int col0 = nt * kBN + wn * kCT * 32;
+#pragma unroll
+            for (int it = 0; it < 16; ++it) {
+                const int r = it * 4 + (lane >> 4), ch = lane & 15;
+                if (r < wave_rows) {
+                    const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kRowStride + ch * 16);
+                    store16_nt(p.out + static_cast<size_t>(out_row0 + r) * p.n + col0 + ch * 8, chunk);
+                }
+            }
         }
+        __syncthreads();  // the staging regions overlap the ring: finish reading before the next tile refills it
     }
 }
 
@@ -386,23 +492,34 @@ int gemm_grid()
         int value = 0;
         if (hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0) cus = value;
     }
-    return cus * 2;
+    return cus;  // one resident workgroup per CU (the LDS ring takes most of the 160 KiB)
+}
+
+template <bool kGateUp>
+int launch_gemm(const GemmParams& p, hipStream_t stream, const char* what)
+{
+    static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
+    if (!configured) {
+        DPEP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<kGateUp>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
+        configured = true;
+    }
+    hipLaunchKernelGGL((grouped_gemm_kernel<kGateUp>), dim3(gemm_grid()), dim3(kGemmThreads), kGemmLdsBytes, stream, p);
+    return launch_status(what);
 }
 
 }  // namespace
 
 int launch_gemm1(const GemmParams& p, hipStream_t stream)
 {
-    if (int rc = check_gemm("gemm1", p.n, p.k, p.num_local, 256)) return rc;
-    hipLaunchKernelGGL((grouped_gemm_kernel<4, true>), dim3(gemm_grid()), dim3(kGemmThreads), 0, stream, p);
-    return launch_status("grouped_gemm1");
+    if (int rc = check_gemm("gemm1", p.n, p.k, p.num_local, kBN)) return rc;
+    return launch_gemm<true>(p, stream, "grouped_gemm1");
 }
 
 int launch_gemm2(const GemmParams& p, hipStream_t stream)
 {
-    if (int rc = check_gemm("gemm2", p.n, p.k, p.num_local, 256)) return rc;
-    hipLaunchKernelGGL((grouped_gemm_kernel<4, false>), dim3(gemm_grid()), dim3(kGemmThreads), 0, stream, p);
-    return launch_status("grouped_gemm2");
+    if (int rc = check_gemm("gemm2", p.n, p.k, p.num_local, kBN)) return rc;
+    return launch_gemm<false>(p, stream, "grouped_gemm2");
 }
 
 }  // namespace dpep
