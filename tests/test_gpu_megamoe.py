@@ -112,3 +112,58 @@ def test_megamoe_forward_rank_share_shape(ops):
     np.testing.assert_array_equal(counts, np.bincount(idx.ravel(), minlength=experts)[:local])
     err = mm.relative_frobenius(got, want)
     assert err <= 2e-2, err
+
+
+def test_public_api_workflow():
+    # the reference's public workflow (experiments/megamoe/tests/test_public_api.py:193-260) on real kernels
+    from deepep_amd import megamoe
+
+    tokens, hidden, inter, experts, topk = 17, 1024, 256, 4, 2
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, experts, topk, seed=5)
+    buf = megamoe.SymmBuffer(None, experts, tokens, topk, hidden, inter)
+    try:
+        assert tuple(buf.x.shape) == (17, 1024) and tuple(buf.x_sf.shape) == (17, 32)
+        raw1 = (torch.from_numpy(l1[0]).cuda(), torch.from_numpy(l1[1]).cuda().view(torch.float8_e8m0fnu))
+        raw2 = (torch.from_numpy(l2[0]).cuda().view(torch.int8), torch.from_numpy(l2[1]).cuda())
+        p1, p2 = megamoe.transform_weights_for_mega_moe(raw1, raw2)
+        buf.x.view(torch.uint8).copy_(torch.from_numpy(x_codes))
+        buf.x_sf.view(torch.uint8).copy_(torch.from_numpy(x_scales))
+        buf.topk_idx.copy_(torch.from_numpy(idx))
+        buf.topk_weights.copy_(torch.from_numpy(weights))
+        buf.validate_inputs(tokens)
+        buf.prepare(tokens)
+        first_ws = buf._workspace
+        buf.prepare(tokens)
+        assert buf._workspace is first_ws and buf.workspace_bytes > 0
+        y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device="cuda")
+        stats = torch.tensor([7, 11, 0, 1], dtype=torch.int32, device="cuda")
+        per_call = np.bincount(idx.ravel(), minlength=experts)
+        assert megamoe.fp8_fp4_mega_moe(y, p1, p2, buf, cumulative_local_expert_recv_stats=stats) is None
+        assert stats.cpu().tolist() == (np.array([7, 11, 0, 1]) + per_call).tolist()
+        megamoe.fp8_fp4_mega_moe(y, p1, p2, buf, cumulative_local_expert_recv_stats=stats)
+        assert stats.cpu().tolist() == (np.array([7, 11, 0, 1]) + 2 * per_call).tolist()
+        want = _oracle(x_codes, x_scales, l1, l2, idx, weights, 0)
+        assert mm.relative_frobenius(y.float().cpu().numpy(), want) <= 2e-2
+        # explicit-input API returns (y, counts); BF16 override is quantised internally
+        xb = torch.from_numpy(mm.mx_dequantize(x_codes, x_scales)).bfloat16().cuda()
+        y2, counts = megamoe.mega_moe(xb, buf.topk_idx[:tokens], buf.topk_weights[:tokens], p1, p2, buf)
+        assert counts.cpu().tolist() == per_call.tolist()
+        want2 = _oracle(*mm.mx_quantize(xb.float().cpu().numpy()), l1, l2, idx, weights, 0)
+        assert mm.relative_frobenius(y2.float().cpu().numpy(), want2) <= 2e-2
+        # error contract
+        with pytest.raises(ValueError, match="alias"):
+            megamoe.mega_moe(xb, buf.topk_idx[:tokens], buf.topk_weights[:tokens], p1, p2, buf, out=xb)
+        with pytest.raises(ValueError, match="prepared"):
+            megamoe.mega_moe(xb, buf.topk_idx[:tokens], buf.topk_weights[:tokens], raw1, raw2, buf)
+        with pytest.raises(RuntimeError, match="DEEPEP_MEGAMOE_TIMER"):
+            buf.allocate_timer()
+        for bad in (-1, 4, int(idx[0, 1])):
+            saved = buf.topk_idx[0, 0].item()
+            buf.topk_idx[0, 0] = bad
+            with pytest.raises(ValueError, match=r"rank=0.*token=0"):
+                buf.validate_inputs(tokens)
+            buf.topk_idx[0, 0] = saved
+    finally:
+        buf.destroy()
+    with pytest.raises(RuntimeError, match="destroyed"):
+        megamoe.fp8_fp4_mega_moe(y, p1, p2, buf)

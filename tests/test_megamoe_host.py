@@ -1,0 +1,36 @@
+"""MegaMoE host-side checks that need no GPU: argument gates and the routing preflight
+(experiments/megamoe/tests/test_public_api.py:233-238, validation.py:10-22)."""
+
+import pytest
+
+from deepep_amd.megamoe import LocalGroup, SymmBuffer, check_routing
+
+
+def test_check_routing_messages():
+    check_routing([[0, 1], [2, 3]], [[0.5, 0.5], [0.1, 0.9]], 4, 2)
+    for bad in (-1, 4, 1):
+        with pytest.raises(ValueError, match=r"rank=0.*token=0"):
+            check_routing([[bad, 1]], [[0.5, 0.5]], 4, 2)
+    with pytest.raises(ValueError, match="finite"):
+        check_routing([[0, 1]], [[float("nan"), 0.5]], 4, 2)
+    with pytest.raises(ValueError, match="top-k"):
+        check_routing([[0]], [[0.5]], 4, 2)
+    with pytest.raises(ValueError, match="rank=3"):
+        check_routing([[0, 0]], [[0.5, 0.5]], 4, 2, rank=3)
+
+
+def test_symm_buffer_argument_gates():
+    for kwargs in (
+        dict(num_experts=0), dict(num_topk=0), dict(hidden=512), dict(hidden=1024 + 64), dict(intermediate_hidden=128),
+        dict(num_topk=5), dict(num_experts=6, group=LocalGroup(0, 4)),
+    ):
+        args = dict(group=None, num_experts=4, num_max_tokens_per_rank=17, num_topk=2, hidden=1024, intermediate_hidden=256)
+        args.update(kwargs)
+        with pytest.raises(ValueError):
+            SymmBuffer(**args)
+    with pytest.raises(NotImplementedError):
+        SymmBuffer(None, 4, 17, 2, 1024, 256, num_shared_experts=1)
+    with pytest.raises(TypeError):
+        SymmBuffer(object(), 4, 17, 2, 1024, 256)
+    with pytest.raises(ValueError):
+        LocalGroup(2, 2)
