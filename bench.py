@@ -92,6 +92,47 @@ def cpu_baseline(x, idx, w, grads, cfg, nbytes):
     )
 
 
+MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 (the mixed FP8 x FP4 MFMA issues at the FP8 cadence)
+
+
+def megamoe_bench(torch, ops, dev, iters):
+    """W4A8 fused expert FFN for one EP64 rank's share: 64 source ranks x 256 tokens, 384 experts of which
+    6 are local, top-8 uniform routing (about 2048 rows), H=7168, I=2048.  Random codes: the arithmetic
+    does not depend on the values.  FLOPs = 2*R*H*2I + 2*R*I*H for the R rows that reach a local expert."""
+    tokens, hidden, inter, experts, local, topk = 64 * 256, 7168, 2048, 384, 6, 8
+    gen = torch.Generator().manual_seed(0)
+    idx = torch.multinomial(torch.ones(tokens, experts), topk, generator=gen).to(torch.int32).to(dev)
+    w = torch.softmax(torch.randn(tokens, topk, generator=gen), -1).to(dev)
+    x_codes = torch.randint(0, 120, (tokens, hidden), dtype=torch.uint8, generator=gen).to(dev).view(torch.float8_e4m3fn)
+    x_scales = torch.full((tokens, hidden // 32), 127, dtype=torch.uint8, device=dev)
+    w1 = torch.randint(0, 256, (local, 2 * inter, hidden // 2), dtype=torch.uint8, device=dev)
+    s1 = torch.full((local, 2 * inter, hidden // 32), 119, dtype=torch.uint8, device=dev)
+    w2 = torch.randint(0, 256, (local, hidden, inter // 2), dtype=torch.uint8, device=dev)
+    s2 = torch.full((local, hidden, inter // 32), 119, dtype=torch.uint8, device=dev)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local))
+    y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+
+    def run():
+        ops.megamoe_forward(ws, x_codes, x_scales, idx, w, w1, s1, w2, s2, experts, 0, local, y, counts)
+
+    us = time_kernel(run, iters, torch)
+    rows = int(counts.sum().item())
+    flops = 2.0 * rows * hidden * 2 * inter + 2.0 * rows * inter * hidden
+    ws.destroy()
+    return {
+        "workload": "EP64 rank share: 16384 candidate tokens, 6 of 384 experts local, top-8, H=7168, I=2048, "
+        "MXFP8 activations x MXFP4 weights; layout + GMM1(+SwiGLU+requant) + GMM2 + weighted reduce",
+        "rows": rows,
+        "us_forward": us,
+        "gflop": flops / 1e9,
+        "tflops_forward": flops / us / 1e6,
+        "roofline": {"bound": "mfma", "achieved": flops / us / 1e6, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
+                     "note": "whole forward (5 launches); per-kernel GEMM times are in profiles/"},
+    }
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -99,6 +140,10 @@ def main():
     parser.add_argument("--warmup", type=int, default=10)
     parser.add_argument("--kernel-iters", type=int, default=50)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-megamoe", action="store_true", help="skip the W4A8 expert-FFN measurement")
+    parser.add_argument("--calibrate-copy", action="store_true",
+                        help="also launch a plain copy of known size (identity dispatch of [32768,7168] BF16: 469.76 MB "
+                        "read + 469.76 MB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share; --gpus must be 1 (no multi-GPU path in this build)", file=sys.stderr)
@@ -204,6 +249,13 @@ def main():
         "kernels": kernels,
         "dispatch_plus_combine_us": us["dispatch_fp8_quant"] + us["combine"],
     }
+    if args.calibrate_copy:
+        ident = torch.arange(rows, dtype=torch.int32, device=dev)
+        for _ in range(5):
+            ops.dispatch_copy(gd[:rows], None, None, ident.view(rows, 1), ident, rows)
+        torch.cuda.synchronize()
+    if not args.no_megamoe:
+        result["megamoe"] = megamoe_bench(torch, ops, dev, args.kernel_iters)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(x, idx, w, grads, cfg, nbytes)
     ws.destroy()

@@ -14,7 +14,13 @@
 namespace dpep {
 namespace {
 
-constexpr int kMaxThreads = 256;
+#ifndef DPEP_TUNE_MAX_THREADS
+#define DPEP_TUNE_MAX_THREADS 256
+#endif
+#ifndef DPEP_TUNE_TARGET_BLOCKS
+#define DPEP_TUNE_TARGET_BLOCKS 1000000  // split every token row into 1-2 KiB parts: measured best at all sizes
+#endif
+constexpr int kMaxThreads = DPEP_TUNE_MAX_THREADS;
 constexpr int kBatch = 8;  // rows fetched per thread before the dependent adds start
 
 // kWeights: 0 = plain sum, 1 = weight per expert row (w[row]), 2 = weight per route (w[t*K + s]).
@@ -79,11 +85,15 @@ struct CombineGrid {
     int parts, per_part, threads;
 };
 
-CombineGrid combine_grid(int num_tokens, int vec)
+// Dense routing (at least one row per token on average): split every token row into 1-2 KiB parts.
+// Sparse receive shares (most tokens own no row and only get zero-filled): one workgroup per token
+// while that still fills the chip.
+CombineGrid combine_grid(int num_tokens, int num_rows, int vec)
 {
     CombineGrid g;
+    const int target = num_rows >= num_tokens ? DPEP_TUNE_TARGET_BLOCKS : 2048;
     int parts = 1;
-    while (num_tokens * parts < 2048 && vec / (parts * 2) >= 64 && parts < 16) parts *= 2;
+    while (num_tokens * parts < target && vec / (parts * 2) >= 64 && parts < 16) parts *= 2;
     g.per_part = (vec + parts - 1) / parts;
     g.parts = (vec + g.per_part - 1) / g.per_part;
     int threads = (g.per_part + 63) / 64 * 64;
@@ -95,10 +105,10 @@ CombineGrid combine_grid(int num_tokens, int vec)
 
 // Route-weighted reduce used by the MegaMoE forward: out[t] = bf16( sum_s w[t,s] * float(y[row(t,s)]) ).
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
-                   int hidden, void* out, hipStream_t stream)
+                   int num_rows_hint, int hidden, void* out, hipStream_t stream)
 {
     const int vec = hidden / 8;
-    const CombineGrid g = combine_grid(num_tokens, vec);
+    const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
     hipLaunchKernelGGL(combine_kernel<2>, dim3(num_tokens * g.parts), dim3(g.threads), 0, stream,
                        static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk, vec, g.per_part, g.parts,
                        static_cast<u32x4*>(out), nullptr, nullptr);
@@ -123,7 +133,7 @@ int dpep_combine(const void* y, const float* row_weights, const int32_t* route_t
     DPEP_REQUIRE(route_to_row != nullptr && out != nullptr && aligned16(out), "combine: NULL or misaligned buffer");
     DPEP_REQUIRE(num_rows == 0 || (y != nullptr && aligned16(y)), "combine: y must be 16-byte aligned");
     const int vec = hidden / 8;
-    const CombineGrid g = combine_grid(num_tokens, vec);
+    const CombineGrid g = combine_grid(num_tokens, num_rows, vec);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (row_weights != nullptr)
         hipLaunchKernelGGL(combine_kernel<1>, dim3(num_tokens * g.parts), dim3(g.threads), 0, s,

@@ -11,7 +11,17 @@
 namespace dpep {
 namespace {
 
-constexpr int kMaxThreads = 256;
+#ifndef DPEP_TUNE_MAX_THREADS
+#define DPEP_TUNE_MAX_THREADS 256
+#endif
+#ifndef DPEP_TUNE_TARGET_BLOCKS
+#define DPEP_TUNE_TARGET_BLOCKS 2048
+#endif
+constexpr int kMaxThreads = DPEP_TUNE_MAX_THREADS;
+constexpr int kMaxScaleCols = 1024;  // hidden <= 131072 for the fused quantiser
+#ifndef DPEP_TUNE_ROW_MAJOR_RATIO
+#define DPEP_TUNE_ROW_MAJOR_RATIO 1  // row-major kernels when rows <= ratio * tokens
+#endif
 
 // ---- token-major copy: one workgroup per (token, column part); read once, write K times -----------
 __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
@@ -136,6 +146,7 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
 {
     __shared__ int rows[DPEP_MAX_TOPK];
     __shared__ int any_valid;
+    __shared__ float part_scales[kMaxScaleCols];
     const int token = blockIdx.x / parts, part = blockIdx.x % parts;
     if (threadIdx.x == 0) any_valid = 0;
     __syncthreads();
@@ -155,10 +166,18 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
         const Quant16 q = quantize16(load16_nt(src + 2 * u), load16_nt(src + 2 * u + 1));
         for (int s = 0; s < num_topk; ++s) {
             const int row = rows[s];
-            if (row < 0) continue;
-            store16_nt(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
-            if ((u & 7) == 0) out_scales[static_cast<size_t>(row) * scale_cols + (u >> 3)] = q.scale;
+            if (row >= 0) store16_nt(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
         }
+        if ((u & 7) == 0) part_scales[(u - u_begin) >> 3] = q.scale;
+    }
+    __syncthreads();
+    // The part's scales leave as contiguous runs (consecutive lanes, consecutive floats) instead of one
+    // 4-byte store per block of 128, which would turn every scale row into read-modify-write traffic.
+    const int part_cols = (u_end - u_begin) >> 3, col0 = u_begin >> 3;
+    for (int i = threadIdx.x; i < num_topk * part_cols; i += blockDim.x) {
+        const int s = i / part_cols, c = i - s * part_cols;
+        const int row = rows[s];
+        if (row >= 0) out_scales[static_cast<size_t>(row) * scale_cols + col0 + c] = part_scales[c];
     }
     if (part == 0 && weights != nullptr && threadIdx.x < num_topk && rows[threadIdx.x] >= 0)
         out_weights[rows[threadIdx.x]] = weights[static_cast<size_t>(token) * num_topk + threadIdx.x];
@@ -195,7 +214,7 @@ struct Split {
 Split choose_split(int rows, int units, int granule)
 {
     Split s;
-    const int target_blocks = 2048;
+    const int target_blocks = DPEP_TUNE_TARGET_BLOCKS;
     int parts = 1;
     while (rows * parts < target_blocks && units / (parts * 2) >= 64 && parts < 16) parts *= 2;
     int per_part = (units + parts - 1) / parts;
@@ -238,7 +257,7 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
     DPEP_REQUIRE(x != nullptr && out != nullptr && aligned16(x) && aligned16(out), "dispatch_copy: x/out must be 16-byte aligned");
     const int vec = row_bytes / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (num_rows > num_tokens) {
+    if (static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
         const Split sp = choose_split(num_tokens, vec, 1);
         hipLaunchKernelGGL(dispatch_copy_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
                            static_cast<const u32x4*>(x), scales, topk_weights, route_to_row, num_topk, vec, sp.per_part,
@@ -258,13 +277,14 @@ int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int3
 {
     using namespace dpep;
     if (int rc = check_common("dispatch_quant_fp8", num_tokens, num_topk, num_rows, route_to_row, row_to_route)) return rc;
-    DPEP_REQUIRE(hidden > 0 && hidden % 128 == 0, "dispatch_quant_fp8: hidden=%d must be a positive multiple of 128", hidden);
+    DPEP_REQUIRE(hidden > 0 && hidden % 128 == 0 && hidden / 128 <= kMaxScaleCols,
+                 "dispatch_quant_fp8: hidden=%d must be a positive multiple of 128, at most %d", hidden, 128 * kMaxScaleCols);
     DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "dispatch_quant_fp8: weights and out_weights go together");
     if (num_rows == 0) return DPEP_OK;
     DPEP_REQUIRE(x && out && out_scales && aligned16(x) && aligned16(out), "dispatch_quant_fp8: x/out must be 16-byte aligned");
     const int units = hidden / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (num_rows > num_tokens) {
+    if (static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
         const Split sp = choose_split(num_tokens, units, 8);
         hipLaunchKernelGGL(dispatch_quant_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
                            static_cast<const u32x4*>(x), topk_weights, route_to_row, num_topk, units, sp.per_part,

@@ -21,7 +21,7 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
                int num_local, int32_t* counts, int32_t* psum, int32_t* offsets, int32_t* route_to_row,
                int32_t* row_to_route, int32_t* num_rows, hipStream_t stream);
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
-                   int hidden, void* out, hipStream_t stream);
+                   int num_rows_hint, int hidden, void* out, hipStream_t stream);
 
 namespace {
 
@@ -648,7 +648,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g2.k = intermediate;
     g2.out = reinterpret_cast<uint16_t*>(base + l.out2);
     if (int rc = launch_gemm2(g2, s)) return rc;
-    return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk, hidden, y, s);
+    // Expected rows (the true count stays on the device): tokens * topk * local / experts.
+    const long long expected_rows = static_cast<long long>(num_tokens) * num_topk * num_local / num_experts;
+    return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,
+                          static_cast<int>(expected_rows), hidden, y, s);
 }
 
 }  // extern "C"
