@@ -244,7 +244,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": dominant["GBps"] / HBM_PEAK_GBS,
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of known
+            # size (factors 1.991 / 1.000): 468.7 MB read + 58.7 MB written (profiles/prefill_hbm_traffic_pmc.md)
+            "traffic": 527.5e6,
         },
         "kernels": kernels,
         "dispatch_plus_combine_us": us["dispatch_fp8_quant"] + us["combine"],
