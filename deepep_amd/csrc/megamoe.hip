@@ -130,27 +130,43 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
 // =====================================================================================================
 // Grouped GEMM
 // =====================================================================================================
-// Workgroup = 4 waves (2 row halves x 2 column halves), tile 128 rows x 256 columns, k tile 128.
-// Everything the main loop reads arrives through asynchronous global->LDS copies into a ring of
-// kStages k tiles; the only synchronisation per k tile is one vmcnt wait plus one barrier.
-constexpr int kBM = 128;           // rows per workgroup tile
-constexpr int kBK = 128;           // k per LDS stage (two MFMA k steps of 64)
+// Workgroup = 4 waves (2 row halves x 2 column halves), tile (64*RT) rows x 256 columns, k tile 128
+// (two MFMA k steps) per LDS stage.  Workgroups are persistent (one per CU) and treat their tiles as ONE
+// flat stream of (tile, k tile) items: asynchronous global->LDS copies run kAhead items ahead of the
+// MFMAs and roll straight into the next tile, so a tile's epilogue overlaps the next tile's first copies.
+// Per item there is one vmcnt wait + one barrier, placed between the two k steps; the fragments of the
+// next k step leave LDS while the MFMAs of the current one run.  The gather indices of the NEXT tile
+// are copied into LDS with every item, so switching tiles needs no blocking global load.
+// Rows are fetched 128 bytes at a time (full cache lines): the texture path handles about one line per
+// cycle and CU, which a 64-byte k tile would saturate.
+constexpr int kBK = 128;           // k per LDS stage = two MFMA k steps
 constexpr int kCT = 4;             // 32-column MFMA tiles per wave
 constexpr int kBN = 2 * kCT * 32;  // columns per workgroup tile
 constexpr int kGemmThreads = 256;
-constexpr int kStages = 4;         // LDS ring depth; copies run kStages-1 k tiles ahead
-constexpr int kStageA = 0;                         // 128 rows x 128 B, 16-byte chunks XOR-swizzled
-constexpr int kStageB = kBM * kBK;                 // 8 column tiles x 2 k steps x 1 KiB fragments
-constexpr int kStageSA = kStageB + kBN * 64;       // 128 row scale words (+128 duplicates)
-constexpr int kStageSB = kStageSA + 1024;          // 8 column tiles x 64 lanes x 2 B
-constexpr int kStageBytes = kStageSB + 1024;
-constexpr int kCopiesPerTile = 10;                 // per thread: 4 A + 4 B + 1 A-scale + 1 B-scale
-constexpr int kGemmLdsBytes = kStages * kStageBytes;
+constexpr int kMaxMoeExperts = 128;
+constexpr int kStagingRowStride = 80;  // 32 BF16 + 16 B pad: conflict-free 16-byte reads
+
+template <int RT, bool kGather>
+struct GemmCfg {
+    static constexpr int kBM = 64 * RT;
+    static constexpr int kStages = RT == 2 ? 4 : 3;
+    static constexpr int kAhead = kStages - 1;
+    static constexpr int kOffA = 0;                    // kBM rows x 128 B, 16-byte chunks XOR-swizzled
+    static constexpr int kOffB = kBM * kBK;            // 8 column tiles x 2 k steps x 1 KiB fragments
+    static constexpr int kOffSA = kOffB + 16384;       // 256 row-scale words (rows >= kBM are padding)
+    static constexpr int kOffSB = kOffSA + 1024;       // 8 column tiles x 64 lanes x 2 B
+    static constexpr int kStageBytes = kOffSB + 1024;
+    // per thread and item: A, B, row scales, column scales, next tile's gather indices
+    static constexpr int kCopies = 2 * RT + 4 + 1 + 1 + (kGather ? 1 : 0);
+    static constexpr int kStagingWave = 32 * RT * kStagingRowStride;
+    static constexpr int kOffStaging = kStages * kStageBytes;
+    static constexpr int kLdsBytes = kOffStaging + 4 * kStagingWave;
+};
 
 struct GemmParams {
     const uint8_t* a_codes;    // [*, K] e4m3
     const uint8_t* a_scales;   // [*, K/32] e8m0
-    const int* row_to_route;   // gather: source row = row_to_route[r] / topk; nullptr = identity
+    const int* row_to_route;   // first GEMM: source row = row_to_route[r] / topk
     int topk;
     const int* offsets;        // [L+1] exclusive row prefix per expert
     int num_local;
@@ -172,7 +188,7 @@ __device__ __forceinline__ float silu_mul(float gate, float up)
 
 // Asynchronous copy global -> LDS: lane l's bytes land at lds_base + l * size.  lds_base is wave-uniform.
 // Written as assembly so that the compiler's own wait-count bookkeeping does not serialise the ring;
-// completion is awaited explicitly with wait_copies<N>().
+// completion is awaited explicitly with wait_copies_then_barrier<N>().
 __device__ __forceinline__ void copy16_to_lds(const void* src, uint32_t lds_base)
 {
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
@@ -189,25 +205,67 @@ __device__ __forceinline__ void wait_copies_then_barrier()
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
-template <bool kGateUp>
+// One scaled MFMA (FP8 A, FP4 B) as a volatile asm statement: volatile statements keep their source order,
+// which is what lets the copies and the barrier be placed between individual MFMAs (builtin MFMAs are pure
+// and the compiler gathers them into bursts).  kSecond selects scale bytes 2|3 of A and byte 1 of B.
+// The compiler cannot see an MFMA in here, so the code that reads an accumulator afterwards has to
+// provide the wait states itself (settle_accumulators).
+template <bool kSecond>
+__device__ __forceinline__ void mfma_fp8_fp4(v16f& acc, const v8i& a, const u32x4& b, int scale_a, int scale_b)
+{
+    if (!kSecond)
+        asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] blgp:4"
+                     : "+a"(acc)
+                     : "v"(a), "v"(b), "v"(scale_a), "v"(scale_b));
+    else
+        asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[0,1,0] op_sel_hi:[1,0,0] blgp:4"
+                     : "+a"(acc)
+                     : "v"(a), "v"(b), "v"(scale_a), "v"(scale_b));
+}
+// 16-pass MFMA results may be read by other instruction types 19 wait states after issue at the earliest.
+__device__ __forceinline__ void settle_accumulators() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
+
+#ifdef DPEP_DEBUG_TIMING
+__device__ unsigned long long g_debug_times[16];
+#define DPEP_STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) g_debug_times[(i) + (kGateUp ? 0 : 8)] = wall_clock64(); } while (0)
+#else
+#define DPEP_STAMP(i) do { } while (0)
+#endif
+
+struct TileInfo {
+    int expert, nt, row0, valid;  // row0 = first row of the tile in the expanded layout; valid rows <= kBM
+};
+
+template <int RT, bool kGateUp>
 __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParams p)
 {
+    constexpr bool kGather = kGateUp;
+    using Cfg = GemmCfg<RT, kGather>;
+    constexpr int kBM = Cfg::kBM, kStages = Cfg::kStages, kAhead = Cfg::kAhead, kStageBytes = Cfg::kStageBytes;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    __shared__ int tile_base[DPEP_MAX_LOCAL_EXPERTS + 1];
+    __shared__ int tile_base[kMaxMoeExperts + 1];
+    __shared__ int row_offsets[kMaxMoeExperts + 1];
+    __shared__ int next_index[kGemmThreads];  // row_to_route of the next tile's rows
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS copy targets in SGPRs
     const int wm = wave >> 1, wn = wave & 1;
     const int g = lane >> 5, lr = lane & 31;
     const int n_tiles = p.n / kBN;
     const int ksteps = p.k / 64, ktiles = p.k / kBK;
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+    const uint32_t lds_index = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(next_index));
 
-    // Tiles per expert: ceil(rows/128) row tiles x n_tiles column tiles, expert-major.
+    DPEP_STAMP(0);
+    // Tiles per expert: ceil(rows/kBM) row tiles x n_tiles column tiles, expert-major, row tile fastest.
+    // (The offsets are fetched by one thread each, in parallel; only the tiny scan is serial.)
+    if (tid <= p.num_local) row_offsets[tid] = p.offsets[tid];
+    __syncthreads();
     if (tid == 0) {
         int total = 0;
         for (int e = 0; e < p.num_local; ++e) {
             tile_base[e] = total;
-            const int rows = p.offsets[e + 1] - p.offsets[e];
+            const int rows = row_offsets[e + 1] - row_offsets[e];
             total += (rows + kBM - 1) / kBM * n_tiles;
         }
         tile_base[p.num_local] = total;
@@ -219,269 +277,327 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     // a contiguous range of tiles so that its L2 sees each weight tile from one place.
     const int per_xcd = (gridDim.x + 7) / 8;
     const int first = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    const int stride = per_xcd * 8;
+    if (first >= total_tiles) return;
+    const int my_tiles = (total_tiles - first + stride - 1) / stride;
 
-    // Per-thread constants of the copy pattern.
-    const int a_swizzle = (wave * 4 + (lane >> 4)) & 7;            // ((row >> 1) & 7) of this thread's A rows
-    const int a_chunk = ((lane & 7) ^ a_swizzle) * 16;              // byte offset inside the 128-byte k tile
-    const uint32_t lds_wave_a = wave * 1024;                        // + copy * 4096
-    const uint32_t lds_wave_s = wave * 256;
-
-    for (int tile = first; tile < total_tiles; tile += per_xcd * 8) {
+    auto decode = [&](int tile) {
         int e = 0;
         while (tile >= tile_base[e + 1]) ++e;
-        const int row_begin = p.offsets[e], rows = p.offsets[e + 1] - row_begin;
+        const int row_begin = row_offsets[e], rows = row_offsets[e + 1] - row_begin;
         const int m_tiles = (rows + kBM - 1) / kBM;
         const int local = tile - tile_base[e];
-        const int nt = local / m_tiles, mt = local % m_tiles;
-        const int m0 = mt * kBM;
-        const int valid_rows = min(kBM, rows - m0);
+        TileInfo info;
+        info.expert = e;
+        info.nt = local / m_tiles;
+        const int m0 = (local % m_tiles) * kBM;
+        info.row0 = row_begin + m0;
+        info.valid = min(kBM, rows - m0);
+        return info;
+    };
 
-        // A: copy i of wave w fills LDS rows i*32 + w*8 + lane/8.
-        const uint8_t* a_src[4];
+    // ---- copy cursor -------------------------------------------------------------------------------
+    // copy i of wave w fills LDS rows i*32 + w*8 + lane/8; chunk (lane%8) ^ ((row>>1)&7) of the 128-byte row
+    const int a_chunk = ((lane & 7) ^ ((wave * 4 + (lane >> 4)) & 7)) * 16;
+    const uint8_t* a_src[2 * RT];
+    const uint8_t* sa_src;
+    const uint8_t* b_src[4];
+    const uint8_t* sb_src;
+    const int* index_src = p.row_to_route;
+    int copy_tile = first, copy_kt = 0, copy_stage = 0;
+    TileInfo next_info = decode(first);
+
+    auto point_at_tile = [&](const TileInfo& info) {
+        // rows past the tile's end repeat its last row
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = min(i * 32 + wave * 8 + (lane >> 3), valid_rows - 1);
-            int src = row_begin + m0 + r;
-            if (p.row_to_route != nullptr) src = p.row_to_route[src] / p.topk;
+        for (int i = 0; i < 2 * RT; ++i) {
+            const int r = min(i * 32 + wave * 8 + (lane >> 3), info.valid - 1);
+            const int src = kGather ? next_index[r] / p.topk : info.row0 + r;
             a_src[i] = p.a_codes + static_cast<size_t>(src) * p.k + a_chunk;
         }
-        const uint8_t* sa_src;
         {
-            const int r = min(tid & (kBM - 1), valid_rows - 1);
-            int src = row_begin + m0 + r;
-            if (p.row_to_route != nullptr) src = p.row_to_route[src] / p.topk;
+            const int r = min(tid, info.valid - 1);
+            const int src = kGather ? next_index[r] / p.topk : info.row0 + r;
             sa_src = p.a_scales + static_cast<size_t>(src) * (p.k / 32);
         }
-        // B: fragment q = copy*4 + wave of the 16 (column tile, k step) fragments of one k tile.
-        const uint8_t* w_block = p.w + static_cast<size_t>(e) * p.n * (p.k / 2) +
-                                 static_cast<size_t>(nt) * (2 * kCT) * ksteps * 1024 + lane * 16;
-        const uint8_t* b_src[4];
+        const uint8_t* w_block = p.w + static_cast<size_t>(info.expert) * p.n * (p.k / 2) +
+                                 static_cast<size_t>(info.nt) * (2 * kCT) * ksteps * 1024 + lane * 16;
+        // fragment q = copy*4 + wave of the 16 (column tile, k step) fragments of one k tile
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int q = j * 4 + wave;
             b_src[j] = w_block + (static_cast<size_t>(q >> 1) * ksteps + (q & 1)) * 1024;
         }
-        const uint8_t* sb_src = p.ws + static_cast<size_t>(e) * p.n * (p.k / 32) +
-                                (static_cast<size_t>(nt) * (2 * kCT) + (tid >> 5)) * ktiles * 128 + (tid & 31) * 4;
+        sb_src = p.ws + static_cast<size_t>(info.expert) * p.n * (p.k / 32) +
+                 (static_cast<size_t>(info.nt) * (2 * kCT) + (tid >> 5)) * ktiles * 128 + (tid & 31) * 4;
+    };
+    auto aim_index_prefetch = [&](const TileInfo& info) {
+        if (kGather) index_src = p.row_to_route + info.row0 + min(tid, info.valid - 1);
+    };
 
-        auto issue_tile = [&](int kt) {
-            const uint32_t stage = lds0 + (kt & (kStages - 1)) * kStageBytes;
+    // Copy number c (compile-time) of the item under the copy cursor; the pieces are issued between MFMAs.
+    auto issue_copy = [&](int c) {
+        const uint32_t stage = lds0 + copy_stage * kStageBytes;
+        if (c < 2 * RT)
+            copy16_to_lds(a_src[c] + static_cast<size_t>(copy_kt) * kBK, stage + Cfg::kOffA + c * 4096 + wave * 1024);
+        else if (c < 2 * RT + 4)
+            copy16_to_lds(b_src[c - 2 * RT] + static_cast<size_t>(copy_kt) * 2048,
+                          stage + Cfg::kOffB + ((c - 2 * RT) * 4 + wave) * 1024);
+        else if (c == 2 * RT + 4)
+            copy4_to_lds(sa_src + copy_kt * 4, stage + Cfg::kOffSA + wave * 256);
+        else if (c == 2 * RT + 5)
+            copy4_to_lds(sb_src + copy_kt * 128, stage + Cfg::kOffSB + wave * 256);
+        else if (kGather)
+            copy4_to_lds(index_src, lds_index + wave * 256);
+    };
+    auto advance_copy_cursor = [&]() {
+        copy_stage = copy_stage + 1 == kStages ? 0 : copy_stage + 1;
+        if (++copy_kt == ktiles) {
+            if (copy_tile + stride < total_tiles) {
+                // The next tile's indices have been landing in next_index since the previous switch
+                // (at least kAhead items ago because ktiles >= kAhead), so this needs no global load.
+                copy_tile += stride;
+                copy_kt = 0;
+                point_at_tile(next_info);
+                if (copy_tile + stride < total_tiles) next_info = decode(copy_tile + stride);
+                aim_index_prefetch(next_info);
+            } else {
+                copy_kt = ktiles - 1;  // past the last tile: keep re-copying its last item (never read)
+            }
+        }
+    };
+    auto issue_item = [&]() {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                copy16_to_lds(a_src[i] + static_cast<size_t>(kt) * kBK, stage + kStageA + i * 4096 + lds_wave_a);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                copy16_to_lds(b_src[j] + static_cast<size_t>(kt) * 2048, stage + kStageB + (j * 4 + wave) * 1024);
-            copy4_to_lds(sa_src + kt * 4, stage + kStageSA + lds_wave_s);
-            copy4_to_lds(sb_src + kt * 128, stage + kStageSB + lds_wave_s);
-        };
+        for (int c = 0; c < Cfg::kCopies; ++c) issue_copy(c);
+        advance_copy_cursor();
+    };
 
-        v16f acc[2][kCT];
+    DPEP_STAMP(1);
+    // First tile: fetch its gather indices synchronously, then aim the prefetch at the second tile.
+    if (kGather) {
+        aim_index_prefetch(next_info);
+        copy4_to_lds(index_src, lds_index + wave * 256);
+        wait_copies_then_barrier<0>();
+    }
+    point_at_tile(next_info);
+    if (first + stride < total_tiles) next_info = decode(first + stride);
+    aim_index_prefetch(next_info);
+
+    // ---- fragment addresses inside a stage ---------------------------------------------------------
+    int a_addr[RT][2][2];  // [row tile][k step][lo/hi 16 bytes]
+    int sa_addr[RT];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < RT; ++i) {
+        const int row = wm * 32 * RT + i * 32 + lr;
+        const int sw = (row >> 1) & 7;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            a_addr[i][kb][0] = Cfg::kOffA + row * kBK + (((kb * 4 + g) ^ sw) << 4);
+            a_addr[i][kb][1] = Cfg::kOffA + row * kBK + (((kb * 4 + 2 + g) ^ sw) << 4);
+        }
+        sa_addr[i] = Cfg::kOffSA + row * 4;
+    }
+    const int b_addr = Cfg::kOffB + wn * kCT * 2048 + lane * 16;
+    const int sb_addr = Cfg::kOffSB + wn * kCT * 128 + lane * 2;
+
+    v8i afrag[2][RT];     // [k step][row tile]
+    u32x4 bfrag[2][kCT];  // [k step][column tile]
+    int ascale[2][RT];    // [item parity][row tile]
+    int bscale[2][kCT];
+    auto read_step = [&](int stage_index, int kb) {
+        const uint8_t* stage = lds + stage_index * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            const u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][0]);
+            const u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][1]);
+            afrag[kb][i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+        }
+#pragma unroll
+        for (int c = 0; c < kCT; ++c) bfrag[kb][c] = *reinterpret_cast<const u32x4*>(stage + b_addr + (c * 2 + kb) * 1024);
+    };
+    auto read_scales = [&](int stage_index, int slot) {
+        const uint8_t* stage = lds + stage_index * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < RT; ++i) ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(stage + sa_addr[i]));
+#pragma unroll
+        for (int c = 0; c < kCT; ++c)
+            bscale[slot][c] = static_cast<int>(*reinterpret_cast<const uint16_t*>(stage + sb_addr + c * 128));
+    };
+
+    v16f acc[RT][kCT];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
 #pragma unroll
             for (int c = 0; c < kCT; ++c)
 #pragma unroll
                 for (int j = 0; j < 16; ++j) acc[i][c][j] = 0.0f;
+    };
+    // The row-scale word holds the four k blocks of the k tile; the upper lane half owns the odd ones
+    // (shifted at use, not at the read, so that the read does not have to be waited for early).
+    constexpr int kMfmas = RT * kCT;  // per k step
+    int ashift[2][RT];  // row scale word moved so that this lane half's first k block is byte 0
+    auto mfma_one = [&](int kb, int slot, int n) {
+        const int c = n / RT, i = n % RT;
+        if (kb == 0) mfma_fp8_fp4<false>(acc[i][c], afrag[0][i], bfrag[0][c], ashift[slot][i], bscale[slot][c]);
+        else mfma_fp8_fp4<true>(acc[i][c], afrag[1][i], bfrag[1][c], ashift[slot][i], bscale[slot][c]);
+    };
+    auto shift_scales = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < RT; ++i) ashift[slot][i] = ascale[slot][i] >> (8 * g);
+    };
 
+    // ---- epilogue of one tile (per-wave staging region, no workgroup synchronisation) ----------------
+    uint8_t* region = lds + Cfg::kOffStaging + wave * Cfg::kStagingWave;
+    auto epilogue = [&](const TileInfo& info) {
+        const int wave_rows = min(32 * RT, info.valid - wm * 32 * RT);  // may be <= 0 for the lower row half
+        const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT;
+        constexpr int kPasses = kGateUp ? kCT / 2 : kCT;
 #pragma unroll
-        for (int kt = 0; kt < kStages - 1; ++kt) issue_tile(min(kt, ktiles - 1));
-
-        // Fragment addresses inside a stage.
-        int a_addr[2][2][2];  // [row tile][k step][lo/hi 16 bytes]
+        for (int pass = 0; pass < kPasses; ++pass) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int row = wm * 64 + i * 32 + lr;
-            const int sw = (row >> 1) & 7;
+            for (int i = 0; i < RT; ++i) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                a_addr[i][kb][0] = kStageA + row * kBK + (((kb * 4 + g) ^ sw) << 4);
-                a_addr[i][kb][1] = kStageA + row * kBK + (((kb * 4 + 2 + g) ^ sw) << 4);
-            }
-        }
-        const int sa_addr = kStageSA + (wm * 64 + lr) * 4;
-        const int b_addr = kStageB + wn * kCT * 2048 + lane * 16;
-        const int sb_addr = kStageSB + wn * kCT * 128 + lane * 2;
-
-        // Software pipeline over k steps of 64: while the MFMAs of one k step run, the fragments of the
-        // next one are already on their way out of LDS.  Per k tile there is one wait + barrier, placed
-        // between the two k steps so that the reads issued right after it have a full k step to land.
-        v8i afrag[2][2];     // [k step][row tile]
-        u32x4 bfrag[2][kCT]; // [k step][column tile]
-        int ascale[2][2];    // [current/next k tile][row tile]
-        int bscale[2][kCT];
-        auto read_step = [&](const uint8_t* stage, int kb) {
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][0]);
-                const u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][1]);
-                afrag[kb][i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-            }
-#pragma unroll
-            for (int c = 0; c < kCT; ++c) bfrag[kb][c] = *reinterpret_cast<const u32x4*>(stage + b_addr + (c * 2 + kb) * 1024);
-        };
-        auto read_scales = [&](const uint8_t* stage, int slot) {
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(stage + sa_addr + i * 128));
-#pragma unroll
-            for (int c = 0; c < kCT; ++c)
-                bscale[slot][c] = static_cast<int>(*reinterpret_cast<const uint16_t*>(stage + sb_addr + c * 128));
-        };
-        auto mfma_step = [&](int kb, int slot) {
-            // The row-scale word holds the four k blocks of the tile; the upper lane half owns the odd ones.
-            // (Shifted here, not at the read, so that the read does not have to be waited for early.)
-            const int sa0 = ascale[slot][0] >> (8 * g), sa1 = ascale[slot][1] >> (8 * g);
-#pragma unroll
-            for (int c = 0; c < kCT; ++c) {
-                const u32x4 b = bfrag[kb][c];
-                const v8i bf = v8i{(int)b[0], (int)b[1], (int)b[2], (int)b[3], 0, 0, 0, 0};
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-#ifdef DPEP_DEBUG_NO_MFMA
-                    acc[i][c][0] += __int_as_float(afrag[kb][i][0] ^ bf[0] ^ (i ? sa1 : sa0) ^ bscale[slot][c]);
-#else
-                    if (kb == 0)
-                        acc[i][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(afrag[0][i], bf, acc[i][c], 0, 4, 0,
-                                                                                    i ? sa1 : sa0, 0, bscale[slot][c]);
-                    else
-                        acc[i][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(afrag[1][i], bf, acc[i][c], 0, 4, 2,
-                                                                                    i ? sa1 : sa0, 1, bscale[slot][c]);
-#endif
-                }
-            }
-        };
-
-        // k tile 0 has landed once each thread has at most kStages-2 tiles of its own copies in flight.
-        wait_copies_then_barrier<(kStages - 2) * kCopiesPerTile>();
-        read_step(lds, 0);
-        read_scales(lds, 0);
-        for (int kt2 = 0; kt2 < ktiles; kt2 += 2) {
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {  // unrolled by two so the scale slots are compile-time
-                const int kt = kt2 + half;
-                const uint8_t* stage = lds + (kt & (kStages - 1)) * kStageBytes;
-                const uint8_t* next_stage = lds + ((kt + 1) & (kStages - 1)) * kStageBytes;
-#ifndef DPEP_DEBUG_NO_READ
-                read_step(stage, 1);
-#endif
-                __builtin_amdgcn_sched_barrier(0);
-                mfma_step(0, half);
-                __builtin_amdgcn_sched_barrier(0);
-                // k tile kt+1 has landed everywhere, and every wave is past its reads of the stage that
-                // the next copies overwrite (the one read during k tile kt-1).
-#ifndef DPEP_DEBUG_NO_BARRIER
-                wait_copies_then_barrier<(kStages - 3) * kCopiesPerTile>();
-#endif
-#ifndef DPEP_DEBUG_NO_COPY
-                issue_tile(min(kt + kStages - 1, ktiles - 1));
-#endif
-#ifndef DPEP_DEBUG_NO_READ
-                read_step(next_stage, 0);
-                read_scales(next_stage, half ^ 1);
-#endif
-                __builtin_amdgcn_sched_barrier(0);
-                mfma_step(1, half);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        // Drain the tail copies and make sure every wave has left the ring before it is refilled.
-        wait_copies_then_barrier<0>();
-
-        // ---- Epilogue: through LDS (the ring is idle now) so that global stores are 16 bytes wide ----
-        const int out_row0 = row_begin + m0 + wm * 64;
-        const int wave_rows = min(64, valid_rows - wm * 64);  // may be <= 0 for the lower row half
-        if (kGateUp) {
-            // Column tiles alternate gate / up for the same 32 activation columns, so SwiGLU is lane-local.
-            // The wave's 64 rows x 64 activation columns are staged as BF16 (row stride 144 B), then each
-            // lane requantises one row: two blocks of 32 -> e8m0 byte + 32 e4m3 codes each.
-            constexpr int kRowStride = 144;
-            uint8_t* region = lds + wave * (64 * kRowStride);
-#pragma unroll
-            for (int pair = 0; pair < kCT / 2; ++pair) {
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        const int r = i * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
-                        const float gate = bf16_to_f32(f32_to_bf16(acc[i][2 * pair][j]));
-                        const float up = bf16_to_f32(f32_to_bf16(acc[i][2 * pair + 1][j]));
-                        *reinterpret_cast<uint16_t*>(region + r * kRowStride + (pair * 32 + lr) * 2) =
-                            static_cast<uint16_t>(f32_to_bf16(silu_mul(gate, up)));
+                for (int j = 0; j < 16; ++j) {
+                    const int r = i * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
+                    float value;
+                    if (kGateUp) {
+                        // column tiles alternate gate / up for the same 32 activation columns
+                        const float gate = bf16_to_f32(f32_to_bf16(acc[i][2 * pass][j]));
+                        const float up = bf16_to_f32(f32_to_bf16(acc[i][2 * pass + 1][j]));
+                        value = silu_mul(gate, up);
+                    } else {
+                        value = acc[i][pass][j];
                     }
+                    *reinterpret_cast<uint16_t*>(region + r * kStagingRowStride + lr * 2) = static_cast<uint16_t>(f32_to_bf16(value));
                 }
             }
-            __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            const int act_width = p.n / 2;
-            const int act_col0 = (nt * kCT + wn * (kCT / 2)) * 32;
-            if (lane < wave_rows) {
-                const size_t row = static_cast<size_t>(out_row0 + lane);
+            __builtin_amdgcn_wave_barrier();
+            if (kGateUp) {
+                // each lane requantises whole rows: 32 BF16 -> e8m0 byte + 32 e4m3 codes
+                const int act_width = p.n / 2;
+                const int act_col = (info.nt * kCT + wn * (kCT / 2) + pass) * 32;
 #pragma unroll
-                for (int blk = 0; blk < kCT / 2; ++blk) {
-                    float v[32];
+                for (int rr = 0; rr < (32 * RT + 63) / 64; ++rr) {
+                    const int r = rr * 64 + lane;
+                    if (r < wave_rows) {
+                        float v[32];
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const u32x4 raw = *reinterpret_cast<const u32x4*>(region + lane * kRowStride + blk * 64 + q * 16);
+                        for (int q = 0; q < 4; ++q) {
+                            const u32x4 raw = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + q * 16);
 #pragma unroll
-                        for (int t = 0; t < 4; ++t) {
-                            v[q * 8 + 2 * t] = bf16_to_f32(raw[t] & 0xffffu);
-                            v[q * 8 + 2 * t + 1] = bf16_to_f32(raw[t] >> 16);
+                            for (int t = 0; t < 4; ++t) {
+                                v[q * 8 + 2 * t] = bf16_to_f32(raw[t] & 0xffffu);
+                                v[q * 8 + 2 * t + 1] = bf16_to_f32(raw[t] >> 16);
+                            }
                         }
+                        float amax = 0.0f;
+#pragma unroll
+                        for (int t = 0; t < 32; ++t) amax = fmaxf(amax, fabsf(v[t]));
+                        const int byte = mx_scale_byte(amax);
+                        u32x4 codes[2];
+#pragma unroll
+                        for (int t = 0; t < 8; ++t)
+                            codes[t >> 2][t & 3] = pack4_e4m3(mx_scaled(v[4 * t], byte), mx_scaled(v[4 * t + 1], byte),
+                                                              mx_scaled(v[4 * t + 2], byte), mx_scaled(v[4 * t + 3], byte));
+                        uint8_t* dst = p.act_codes + (out_row0 + r) * act_width + act_col;
+                        *reinterpret_cast<u32x4*>(dst) = codes[0];
+                        *reinterpret_cast<u32x4*>(dst + 16) = codes[1];
+                        p.act_scales[(out_row0 + r) * (act_width / 32) + (act_col >> 5)] = static_cast<uint8_t>(byte);
                     }
-                    float amax = 0.0f;
-#pragma unroll
-                    for (int t = 0; t < 32; ++t) amax = fmaxf(amax, fabsf(v[t]));
-                    const int byte = mx_scale_byte(amax);
-                    u32x4 codes[2];
-#pragma unroll
-                    for (int t = 0; t < 8; ++t)
-                        codes[t >> 2][t & 3] = pack4_e4m3(mx_scaled(v[4 * t], byte), mx_scaled(v[4 * t + 1], byte),
-                                                          mx_scaled(v[4 * t + 2], byte), mx_scaled(v[4 * t + 3], byte));
-                    uint8_t* dst = p.act_codes + row * act_width + act_col0 + blk * 32;
-                    *reinterpret_cast<u32x4*>(dst) = codes[0];
-                    *reinterpret_cast<u32x4*>(dst + 16) = codes[1];
-                    p.act_scales[row * (act_width / 32) + (act_col0 >> 5) + blk] = static_cast<uint8_t>(byte);
                 }
-            }
-        } else {
-            // The wave's 64 rows x 128 columns are staged as BF16 (row stride 272 B) and leave as 16-byte
-            // chunks: 16 lanes cover one 256-byte row segment.
-            constexpr int kRowStride = 272;
-            uint8_t* region = lds + wave * (64 * kRowStride);
+            } else {
+                // 4 lanes carry one 64-byte row segment
+                const int col = info.nt * kBN + (wn * kCT + pass) * 32 + (lane & 3) * 8;
 #pragma unroll
-            for (int c = 0; c < kCT; ++c) {
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        const int r = i * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
-                        *reinterpret_cast<uint16_t*>(region + r * kRowStride + (c * 32 + lr) * 2) =
-                            static_cast<uint16_t>(f32_to_bf16(acc[i][c][j]));
+                for (int it = 0; it < 2 * RT; ++it) {
+                    const int r = it * 16 + (lane >> 2);
+                    if (r < wave_rows) {
+                        const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
+                        store16_nt(p.out + (out_row0 + r) * p.n + col, chunk);
                     }
                 }
             }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            const int col0 = nt * kBN + wn * kCT * 32;
+        }
+    };
+
+    DPEP_STAMP(2);
+    // ---- the flat item stream --------------------------------------------------------------------------
 #pragma unroll
-            for (int it = 0; it < 16; ++it) {
-                const int r = it * 4 + (lane >> 4), ch = lane & 15;
-                if (r < wave_rows) {
-                    const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kRowStride + ch * 16);
-                    store16_nt(p.out + static_cast<size_t>(out_row0 + r) * p.n + col0 + ch * 8, chunk);
+    for (int j = 0; j < kAhead; ++j) issue_item();
+    wait_copies_then_barrier<(kAhead - 1) * Cfg::kCopies>();  // item 0 has landed
+    read_step(0, 0);
+    read_scales(0, 0);
+    clear_acc();
+    asm volatile("s_nop 3");
+    DPEP_STAMP(3);
+    int stage_now = 0;  // stage of the item whose MFMAs run
+    int tile = first, kt = 0;
+    TileInfo info = decode(first);
+    const long long total_items = static_cast<long long>(my_tiles) * ktiles;
+    for (long long item = 0; item < total_items; item += 2) {
+#pragma unroll
+        for (int parity = 0; parity < 2; ++parity) {  // ktiles is even, so tiles start on even items
+            const int stage_next = stage_now + 1 == kStages ? 0 : stage_now + 1;
+            // A wave issues in order and owns its SIMD alone, so whatever is not an MFMA should sit in the
+            // shadow of one: after the barrier the copies of the item kAhead ahead and the fragment reads of
+            // the next item are dealt out between the MFMAs.
+            read_step(stage_now, 1);
+            shift_scales(parity);
+#pragma unroll
+            for (int n = 0; n < kMfmas / 2; ++n) mfma_one(0, parity, n);
+            // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies in
+            // flight; past the barrier every wave has also finished reading the stage refilled next.
+            wait_copies_then_barrier<(kAhead - 2) * Cfg::kCopies>();
+            constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
+#pragma unroll
+            for (int n = kMfmas / 2; n < kMfmas; ++n) {
+                mfma_one(0, parity, n);
+                const int slot = n - kMfmas / 2;
+#pragma unroll
+                for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
+            }
+            read_step(stage_next, 0);
+            read_scales(stage_next, parity ^ 1);
+#pragma unroll
+            for (int n = 0; n < kMfmas; ++n) {
+                mfma_one(1, parity, n);
+                const int slot = n + kMfmas / 2;
+                if (slot < kSlots) {
+#pragma unroll
+                    for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
                 }
             }
+            advance_copy_cursor();
+            stage_now = stage_next;
         }
-        __syncthreads();  // the staging regions overlap the ring: finish reading before the next tile refills it
+        kt += 2;
+        if (kt == ktiles) {
+            DPEP_STAMP(4);
+            settle_accumulators();
+            epilogue(info);
+            DPEP_STAMP(5);
+            clear_acc();
+            asm volatile("s_nop 3");  // accumulator writes settle before the next MFMA reads them
+            kt = 0;
+            tile += stride;
+            if (tile < total_tiles) info = decode(tile);
+        }
     }
+    // No copy may still be in flight into this workgroup's LDS when it retires.
+    wait_copies_then_barrier<0>();
+    DPEP_STAMP(6);
 }
 
-int check_gemm(const char* what, int n, int k, int num_local, int block_n)
+int check_gemm(const char* what, int n, int k, int num_local)
 {
-    DPEP_REQUIRE(num_local >= 1 && num_local <= DPEP_MAX_LOCAL_EXPERTS, "%s: bad number of local experts %d", what, num_local);
-    DPEP_REQUIRE(k > 0 && k % 256 == 0, "%s: K=%d must be a positive multiple of 256", what, k);
-    DPEP_REQUIRE(n > 0 && n % block_n == 0, "%s: N=%d must be a positive multiple of %d", what, n, block_n);
+    DPEP_REQUIRE(num_local >= 1 && num_local <= kMaxMoeExperts, "%s: number of local experts %d outside [1, %d]", what,
+                 num_local, kMaxMoeExperts);
+    DPEP_REQUIRE(k >= 512 && k % 256 == 0, "%s: K=%d must be a multiple of 256, at least 512", what, k);
+    DPEP_REQUIRE(n > 0 && n % kBN == 0, "%s: N=%d must be a positive multiple of %d", what, n, kBN);
     return DPEP_OK;
 }
 
@@ -492,39 +608,75 @@ int gemm_grid()
         int value = 0;
         if (hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0) cus = value;
     }
-    return cus;  // one resident workgroup per CU (the LDS ring takes most of the 160 KiB)
+    return cus / 8 * 8;  // one resident workgroup per CU (the LDS ring takes most of the 160 KiB)
 }
 
-template <bool kGateUp>
-int launch_gemm(const GemmParams& p, hipStream_t stream, const char* what)
+template <int RT, bool kGateUp>
+int launch_gemm_rt(const GemmParams& p, hipStream_t stream, const char* what)
 {
+    constexpr int kLds = GemmCfg<RT, kGateUp>::kLdsBytes;
     static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
     if (!configured) {
-        DPEP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<kGateUp>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
+        DPEP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<RT, kGateUp>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
         configured = true;
     }
-    hipLaunchKernelGGL((grouped_gemm_kernel<kGateUp>), dim3(gemm_grid()), dim3(kGemmThreads), kGemmLdsBytes, stream, p);
+    hipLaunchKernelGGL((grouped_gemm_kernel<RT, kGateUp>), dim3(gemm_grid()), dim3(kGemmThreads), kLds, stream, p);
     return launch_status(what);
+}
+
+// Row-tile height: the cheaper of 128 / 192 rows, whose tile count fits one round of workgroups, judged
+// from the expected rows per expert (the true counts stay on the device).
+template <bool kGateUp>
+int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t stream, const char* what)
+{
+    const int cus = gemm_grid();
+    const int n_tiles = p.n / kBN;
+    int best = 2;
+    double best_cost = 1e30;
+    for (int rt = 2; rt <= 3; ++rt) {
+        const int bm = 64 * rt;
+        const int m_tiles = (expected_rows_per_expert + bm - 1) / bm;
+        const long long tiles = static_cast<long long>(p.num_local) * (m_tiles > 0 ? m_tiles : 1) * n_tiles;
+        const long long rounds = (tiles + cus - 1) / cus;
+        const double cost = static_cast<double>(rounds) * rt;  // time of a tile grows with its height
+        if (cost < best_cost - 1e-9) {
+            best_cost = cost;
+            best = rt;
+        }
+    }
+#ifdef DPEP_TUNE_GEMM_RT
+    best = DPEP_TUNE_GEMM_RT;
+#endif
+    if (best == 2) return launch_gemm_rt<2, kGateUp>(p, stream, what);
+    return launch_gemm_rt<3, kGateUp>(p, stream, what);
 }
 
 }  // namespace
 
-int launch_gemm1(const GemmParams& p, hipStream_t stream)
+int launch_gemm1(const GemmParams& p, int expected_rows_per_expert, hipStream_t stream)
 {
-    if (int rc = check_gemm("gemm1", p.n, p.k, p.num_local, kBN)) return rc;
-    return launch_gemm<true>(p, stream, "grouped_gemm1");
+    if (int rc = check_gemm("gemm1", p.n, p.k, p.num_local)) return rc;
+    DPEP_REQUIRE(p.row_to_route != nullptr && p.topk >= 1, "gemm1: needs the row -> route map");
+    return launch_gemm<true>(p, expected_rows_per_expert, stream, "grouped_gemm1");
 }
 
-int launch_gemm2(const GemmParams& p, hipStream_t stream)
+int launch_gemm2(const GemmParams& p, int expected_rows_per_expert, hipStream_t stream)
 {
-    if (int rc = check_gemm("gemm2", p.n, p.k, p.num_local, kBN)) return rc;
-    return launch_gemm<false>(p, stream, "grouped_gemm2");
+    if (int rc = check_gemm("gemm2", p.n, p.k, p.num_local)) return rc;
+    return launch_gemm<false>(p, expected_rows_per_expert, stream, "grouped_gemm2");
 }
 
 }  // namespace dpep
 
 extern "C" {
+
+#ifdef DPEP_DEBUG_TIMING
+int dpep_debug_times(unsigned long long* host16)
+{
+    return hipMemcpyFromSymbol(host16, HIP_SYMBOL(dpep::g_debug_times), 16 * sizeof(unsigned long long)) == hipSuccess ? 0 : -2;
+}
+#endif
 
 int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* scales, void* stream)
 {
@@ -600,9 +752,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     DPEP_REQUIRE(w != nullptr, "megamoe_forward: not a live workspace");
     DPEP_REQUIRE(num_tokens >= 1 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "megamoe_forward: bad B=%d K=%d",
                  num_tokens, num_topk);
-    DPEP_REQUIRE(hidden % 256 == 0 && intermediate % 256 == 0 && hidden > 0 && intermediate > 0,
-                 "megamoe_forward: hidden=%d and intermediate=%d must be positive multiples of 256", hidden, intermediate);
-    DPEP_REQUIRE(num_local >= 1 && num_local <= DPEP_MAX_LOCAL_EXPERTS && expert_begin >= 0 &&
+    DPEP_REQUIRE(hidden % 256 == 0 && intermediate % 256 == 0 && hidden >= 512 && intermediate >= 512,
+                 "megamoe_forward: hidden=%d and intermediate=%d must be multiples of 256, at least 512", hidden,
+                 intermediate);
+    DPEP_REQUIRE(num_local >= 1 && num_local <= 128 && expert_begin >= 0 &&
                      expert_begin + num_local <= num_experts,
                  "megamoe_forward: bad expert range E=%d begin=%d L=%d", num_experts, expert_begin, num_local);
     DPEP_REQUIRE(x_codes && x_scales && topk_idx && topk_weights && w1 && s1 && w2 && s2 && y && expert_token_nums,
@@ -634,7 +787,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g1.k = hidden;
     g1.act_codes = base + l.act_codes;
     g1.act_scales = base + l.act_scales;
-    if (int rc = launch_gemm1(g1, s)) return rc;
+    // Expected rows (the true counts stay on the device): tokens * topk / experts per expert.
+    const long long expected_rows = static_cast<long long>(num_tokens) * num_topk * num_local / num_experts;
+    const int per_expert = static_cast<int>((expected_rows + num_local - 1) / num_local);
+    if (int rc = launch_gemm1(g1, per_expert, s)) return rc;
     GemmParams g2{};
     g2.a_codes = base + l.act_codes;
     g2.a_scales = base + l.act_scales;
@@ -647,9 +803,7 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g2.n = hidden;
     g2.k = intermediate;
     g2.out = reinterpret_cast<uint16_t*>(base + l.out2);
-    if (int rc = launch_gemm2(g2, s)) return rc;
-    // Expected rows (the true count stays on the device): tokens * topk * local / experts.
-    const long long expected_rows = static_cast<long long>(num_tokens) * num_topk * num_local / num_experts;
+    if (int rc = launch_gemm2(g2, per_expert, s)) return rc;
     return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,
                           static_cast<int>(expected_rows), hidden, y, s);
 }

@@ -9,7 +9,7 @@ transform_weights_for_mega_moe :311-379, mega_moe :382-413, fp8_fp4_mega_moe :52
     (capacity ``world_size * num_max_tokens_per_rank`` rows).  The reference needs 2..128 real ranks;
   * prepared weights are this library's fragment order (``dpep_megamoe_prepare_weights``), not Ascend NZ;
   * shared experts and FP8xFP8 weights are not built; hidden and intermediate_hidden must be multiples
-    of 256 (the reference: 64 and 128).
+    of 256 with intermediate_hidden >= 512 (the reference: multiples of 64 and 128, from 256).
 """
 
 from __future__ import annotations
@@ -95,7 +95,7 @@ class SymmBuffer:
         _integer("num_max_tokens_per_rank", num_max_tokens_per_rank, 1, 65536)
         _integer("num_topk", num_topk, 1, min(32, num_experts))
         _integer("hidden", hidden, 1024, 8192)
-        _integer("intermediate_hidden", intermediate_hidden, 256, 4096)
+        _integer("intermediate_hidden", intermediate_hidden, 512, 4096)
         _integer("num_shared_experts", num_shared_experts, 0, 8)
         _integer("ranks_per_node", ranks_per_node, 0, size)
         _integer("timeout", timeout, 1, 300)

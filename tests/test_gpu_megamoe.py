@@ -85,10 +85,10 @@ def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local):
 @pytest.mark.parametrize(
     "tokens,hidden,inter,experts,begin,local,topk",
     [
-        (64, 256, 256, 4, 0, 4, 2),      # every expert local, tiny
-        (300, 512, 256, 8, 2, 3, 4),     # ragged rows, local range inside E, partial tiles
+        (64, 512, 512, 4, 0, 4, 2),      # every expert local, tiny
+        (300, 512, 512, 8, 2, 3, 4),     # ragged rows, local range inside E, partial tiles
         (257, 1024, 512, 6, 0, 6, 6),    # every token hits every expert
-        (96, 256, 256, 8, 6, 2, 1),      # some local experts may be empty
+        (96, 512, 768, 8, 6, 2, 1),      # some local experts may be empty
     ],
 )
 def test_megamoe_forward_matches_oracle(ops, tokens, hidden, inter, experts, begin, local, topk):
@@ -118,7 +118,7 @@ def test_public_api_workflow():
     # the reference's public workflow (experiments/megamoe/tests/test_public_api.py:193-260) on real kernels
     from deepep_amd import megamoe
 
-    tokens, hidden, inter, experts, topk = 17, 1024, 256, 4, 2
+    tokens, hidden, inter, experts, topk = 17, 1024, 512, 4, 2
     x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, experts, topk, seed=5)
     buf = megamoe.SymmBuffer(None, experts, tokens, topk, hidden, inter)
     try:

@@ -21,16 +21,16 @@ def test_check_routing_messages():
 
 def test_symm_buffer_argument_gates():
     for kwargs in (
-        dict(num_experts=0), dict(num_topk=0), dict(hidden=512), dict(hidden=1024 + 64), dict(intermediate_hidden=128),
+        dict(num_experts=0), dict(num_topk=0), dict(hidden=512), dict(hidden=1024 + 64), dict(intermediate_hidden=256),
         dict(num_topk=5), dict(num_experts=6, group=LocalGroup(0, 4)),
     ):
-        args = dict(group=None, num_experts=4, num_max_tokens_per_rank=17, num_topk=2, hidden=1024, intermediate_hidden=256)
+        args = dict(group=None, num_experts=4, num_max_tokens_per_rank=17, num_topk=2, hidden=1024, intermediate_hidden=512)
         args.update(kwargs)
         with pytest.raises(ValueError):
             SymmBuffer(**args)
     with pytest.raises(NotImplementedError):
-        SymmBuffer(None, 4, 17, 2, 1024, 256, num_shared_experts=1)
+        SymmBuffer(None, 4, 17, 2, 1024, 512, num_shared_experts=1)
     with pytest.raises(TypeError):
-        SymmBuffer(object(), 4, 17, 2, 1024, 256)
+        SymmBuffer(object(), 4, 17, 2, 1024, 512)
     with pytest.raises(ValueError):
         LocalGroup(2, 2)
