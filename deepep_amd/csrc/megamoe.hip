@@ -153,13 +153,16 @@ struct GemmCfg {
     static constexpr int kAhead = kStages - 1;
     static constexpr int kOffA = 0;                    // kBM rows x 128 B, 16-byte chunks XOR-swizzled
     static constexpr int kOffB = kBM * kBK;            // 8 column tiles x 2 k steps x 1 KiB fragments
-    static constexpr int kOffSA = kOffB + 16384;       // 256 row-scale words (rows >= kBM are padding)
-    static constexpr int kOffSB = kOffSA + 1024;       // 8 column tiles x 64 lanes x 2 B
+    static constexpr int kOffSB = kOffB + 16384;       // 8 column tiles x 64 lanes x 2 B
     static constexpr int kStageBytes = kOffSB + 1024;
-    // per thread and item: A, B, row scales, column scales, next tile's gather indices
-    static constexpr int kCopies = 2 * RT + 4 + 1 + 1 + (kGather ? 1 : 0);
-    static constexpr int kStagingWave = 32 * RT * kStagingRowStride;
-    static constexpr int kOffStaging = kStages * kStageBytes;
+    // per thread and item: A, B, column scales, next tile's gather indices.  The row scales travel apart:
+    // 16 bytes per row cover k = 512 and are copied once per four items into a two-slot ring, because a
+    // 4-byte copy per row and item costs a cache-line lookup per lane, as many as the whole A tile.
+    static constexpr int kCopies = 2 * RT + 4 + 1 + (kGather ? 1 : 0);
+    static constexpr int kRowScaleSlot = kBM * 16;
+    static constexpr int kOffRowScales = kStages * kStageBytes;
+    static constexpr int kStagingWave = 64 * kStagingRowStride;  // the epilogue handles 64 rows at a time
+    static constexpr int kOffStaging = kOffRowScales + 2 * kRowScaleSlot;
     static constexpr int kLdsBytes = kOffStaging + 4 * kStagingWave;
 };
 
@@ -198,6 +201,18 @@ __device__ __forceinline__ void copy4_to_lds(const void* src, uint32_t lds_base)
 {
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(src) : "memory");
+}
+// The same 16-byte copy, skipped when the (wave-uniform) value skip is not zero.  The jump stays inside
+// the asm statement so that the loop body around it remains straight-line code.
+__device__ __forceinline__ void copy16_to_lds_unless(const void* src, uint32_t lds_base, int skip)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    const int flag = __builtin_amdgcn_readfirstlane(skip);
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_cmp_lg_u32 %2, 0\n\ts_cbranch_scc1 .Lskip_copy_%=\n\t"
+        "global_load_lds_dwordx4 %1, off\n.Lskip_copy_%=:" ::"s"(base),
+        "v"(src), "s"(flag)
+        : "memory", "scc");
 }
 template <int kOutstanding>
 __device__ __forceinline__ void wait_copies_then_barrier()
@@ -304,7 +319,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     const uint8_t* b_src[4];
     const uint8_t* sb_src;
     const int* index_src = p.row_to_route;
-    int copy_tile = first, copy_kt = 0, copy_stage = 0;
+    int copy_tile = first, copy_kt = 0, copy_stage = 0, copy_span = -1;
+    const int scale_bytes = p.k / 32;  // per row
     TileInfo next_info = decode(first);
 
     auto point_at_tile = [&](const TileInfo& info) {
@@ -316,9 +332,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             a_src[i] = p.a_codes + static_cast<size_t>(src) * p.k + a_chunk;
         }
         {
-            const int r = min(tid, info.valid - 1);
+            // thread t serves row t % kBM (surplus waves repeat rows, which keeps every wave's copy count equal)
+            const int r = min(tid % kBM, info.valid - 1);
             const int src = kGather ? next_index[r] / p.topk : info.row0 + r;
-            sa_src = p.a_scales + static_cast<size_t>(src) * (p.k / 32);
+            sa_src = p.a_scales + static_cast<size_t>(src) * scale_bytes;
         }
         const uint8_t* w_block = p.w + static_cast<size_t>(info.expert) * p.n * (p.k / 2) +
                                  static_cast<size_t>(info.nt) * (2 * kCT) * ksteps * 1024 + lane * 16;
@@ -337,6 +354,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 
     // Copy number c (compile-time) of the item under the copy cursor; the pieces are issued between MFMAs.
     auto issue_copy = [&](int c) {
+#ifdef DPEP_X_NOCOPY
+        return;
+#endif
+#ifdef DPEP_X_NOSMALL
+        if (c >= 2 * RT + 4) return;
+#endif
         const uint32_t stage = lds0 + copy_stage * kStageBytes;
         if (c < 2 * RT)
             copy16_to_lds(a_src[c] + static_cast<size_t>(copy_kt) * kBK, stage + Cfg::kOffA + c * 4096 + wave * 1024);
@@ -344,11 +367,18 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             copy16_to_lds(b_src[c - 2 * RT] + static_cast<size_t>(copy_kt) * 2048,
                           stage + Cfg::kOffB + ((c - 2 * RT) * 4 + wave) * 1024);
         else if (c == 2 * RT + 4)
-            copy4_to_lds(sa_src + copy_kt * 4, stage + Cfg::kOffSA + wave * 256);
-        else if (c == 2 * RT + 5)
             copy4_to_lds(sb_src + copy_kt * 128, stage + Cfg::kOffSB + wave * 256);
         else if (kGather)
             copy4_to_lds(index_src, lds_index + wave * 256);
+    };
+    // Every fourth item starts a new 16-byte window of row scales (clamped so that it never leaves the
+    // row: k % 512 may be 256).  The extra copy only makes the counted waits stricter.
+    auto issue_row_scales = [&]() {
+        copy_span += (copy_kt & 3) == 0 ? 1 : 0;
+        const int window = min((copy_kt & ~3) * 4, scale_bytes - 16);
+        copy16_to_lds_unless(sa_src + window,
+                             lds0 + Cfg::kOffRowScales + (copy_span & 1) * Cfg::kRowScaleSlot + ((wave * 64) % kBM) * 16,
+                             copy_kt & 3);
     };
     auto advance_copy_cursor = [&]() {
         copy_stage = copy_stage + 1 == kStages ? 0 : copy_stage + 1;
@@ -369,6 +399,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     auto issue_item = [&]() {
 #pragma unroll
         for (int c = 0; c < Cfg::kCopies; ++c) issue_copy(c);
+        issue_row_scales();
         advance_copy_cursor();
     };
 
@@ -395,7 +426,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             a_addr[i][kb][0] = Cfg::kOffA + row * kBK + (((kb * 4 + g) ^ sw) << 4);
             a_addr[i][kb][1] = Cfg::kOffA + row * kBK + (((kb * 4 + 2 + g) ^ sw) << 4);
         }
-        sa_addr[i] = Cfg::kOffSA + row * 4;
+        sa_addr[i] = Cfg::kOffRowScales + row * 16;
     }
     const int b_addr = Cfg::kOffB + wn * kCT * 2048 + lane * 16;
     const int sb_addr = Cfg::kOffSB + wn * kCT * 128 + lane * 2;
@@ -415,10 +446,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 #pragma unroll
         for (int c = 0; c < kCT; ++c) bfrag[kb][c] = *reinterpret_cast<const u32x4*>(stage + b_addr + (c * 2 + kb) * 1024);
     };
-    auto read_scales = [&](int stage_index, int slot) {
+    // scale_at = byte offset of the item's row-scale word: ring slot + position inside the 16-byte window
+    auto read_scales = [&](int stage_index, int slot, int scale_at) {
         const uint8_t* stage = lds + stage_index * kStageBytes;
 #pragma unroll
-        for (int i = 0; i < RT; ++i) ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(stage + sa_addr[i]));
+        for (int i = 0; i < RT; ++i) ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + sa_addr[i] + scale_at));
 #pragma unroll
         for (int c = 0; c < kCT; ++c)
             bscale[slot][c] = static_cast<int>(*reinterpret_cast<const uint16_t*>(stage + sb_addr + c * 128));
@@ -450,38 +482,43 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     // ---- epilogue of one tile (per-wave staging region, no workgroup synchronisation) ----------------
     uint8_t* region = lds + Cfg::kOffStaging + wave * Cfg::kStagingWave;
     auto epilogue = [&](const TileInfo& info) {
-        const int wave_rows = min(32 * RT, info.valid - wm * 32 * RT);  // may be <= 0 for the lower row half
-        const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT;
         constexpr int kPasses = kGateUp ? kCT / 2 : kCT;
+        // The staging region holds 64 rows (two row tiles) x 32 columns; larger wave tiles take several turns.
 #pragma unroll
-        for (int pass = 0; pass < kPasses; ++pass) {
+        for (int i0 = 0; i0 < RT; i0 += 2) {
+            constexpr int kTilesMax = 2;
+            const int tiles_here = RT - i0 < kTilesMax ? RT - i0 : kTilesMax;
+            const int chunk_rows = min(32 * tiles_here, info.valid - wm * 32 * RT - 32 * i0);  // may be <= 0
+            const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT + 32 * i0;
 #pragma unroll
-            for (int i = 0; i < RT; ++i) {
+            for (int pass = 0; pass < kPasses; ++pass) {
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    const int r = i * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
-                    float value;
-                    if (kGateUp) {
-                        // column tiles alternate gate / up for the same 32 activation columns
-                        const float gate = bf16_to_f32(f32_to_bf16(acc[i][2 * pass][j]));
-                        const float up = bf16_to_f32(f32_to_bf16(acc[i][2 * pass + 1][j]));
-                        value = silu_mul(gate, up);
-                    } else {
-                        value = acc[i][pass][j];
+                for (int ii = 0; ii < kTilesMax; ++ii) {
+                    if (i0 + ii >= RT) continue;
+                    const int i = i0 + ii;
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const int r = ii * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
+                        float value;
+                        if (kGateUp) {
+                            // column tiles alternate gate / up for the same 32 activation columns
+                            const float gate = bf16_to_f32(f32_to_bf16(acc[i][2 * pass][j]));
+                            const float up = bf16_to_f32(f32_to_bf16(acc[i][2 * pass + 1][j]));
+                            value = silu_mul(gate, up);
+                        } else {
+                            value = acc[i][pass][j];
+                        }
+                        *reinterpret_cast<uint16_t*>(region + r * kStagingRowStride + lr * 2) = static_cast<uint16_t>(f32_to_bf16(value));
                     }
-                    *reinterpret_cast<uint16_t*>(region + r * kStagingRowStride + lr * 2) = static_cast<uint16_t>(f32_to_bf16(value));
                 }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            if (kGateUp) {
-                // each lane requantises whole rows: 32 BF16 -> e8m0 byte + 32 e4m3 codes
-                const int act_width = p.n / 2;
-                const int act_col = (info.nt * kCT + wn * (kCT / 2) + pass) * 32;
-#pragma unroll
-                for (int rr = 0; rr < (32 * RT + 63) / 64; ++rr) {
-                    const int r = rr * 64 + lane;
-                    if (r < wave_rows) {
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                if (kGateUp) {
+                    // each lane requantises a whole row: 32 BF16 -> e8m0 byte + 32 e4m3 codes
+                    const int act_width = p.n / 2;
+                    const int act_col = (info.nt * kCT + wn * (kCT / 2) + pass) * 32;
+                    const int r = lane;
+                    if (r < chunk_rows) {
                         float v[32];
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
@@ -506,21 +543,21 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                         *reinterpret_cast<u32x4*>(dst + 16) = codes[1];
                         p.act_scales[(out_row0 + r) * (act_width / 32) + (act_col >> 5)] = static_cast<uint8_t>(byte);
                     }
-                }
-            } else {
-                // 4 lanes carry one 64-byte row segment
-                const int col = info.nt * kBN + (wn * kCT + pass) * 32 + (lane & 3) * 8;
+                } else {
+                    // 4 lanes carry one 64-byte row segment
+                    const int col = info.nt * kBN + (wn * kCT + pass) * 32 + (lane & 3) * 8;
 #pragma unroll
-                for (int it = 0; it < 2 * RT; ++it) {
-                    const int r = it * 16 + (lane >> 2);
-                    if (r < wave_rows) {
-                        const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
-                        store16_nt(p.out + (out_row0 + r) * p.n + col, chunk);
+                    for (int it = 0; it < 2 * kTilesMax; ++it) {
+                        const int r = it * 16 + (lane >> 2);
+                        if (r < chunk_rows) {
+                            const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
+                            store16_nt(p.out + (out_row0 + r) * p.n + col, chunk);
+                        }
                     }
                 }
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
         }
     };
 
@@ -529,8 +566,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 #pragma unroll
     for (int j = 0; j < kAhead; ++j) issue_item();
     wait_copies_then_barrier<(kAhead - 1) * Cfg::kCopies>();  // item 0 has landed
+    // Row-scale bookkeeping of the item whose fragments are read next: span counter (ring slot) and k tile.
+    int read_span = -1, read_kt = 0;
+    auto next_scale_offset = [&]() {
+        if ((read_kt & 3) == 0) ++read_span;
+        const int window = min((read_kt & ~3) * 4, scale_bytes - 16);
+        const int at = (read_span & 1) * Cfg::kRowScaleSlot + (read_kt * 4 - window);
+        read_kt = read_kt + 1 == ktiles ? 0 : read_kt + 1;
+        return at;
+    };
     read_step(0, 0);
-    read_scales(0, 0);
+    read_scales(0, 0, next_scale_offset());
     clear_acc();
     asm volatile("s_nop 3");
     DPEP_STAMP(3);
@@ -551,7 +597,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             for (int n = 0; n < kMfmas / 2; ++n) mfma_one(0, parity, n);
             // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies in
             // flight; past the barrier every wave has also finished reading the stage refilled next.
+#ifndef DPEP_X_NOBARRIER
             wait_copies_then_barrier<(kAhead - 2) * Cfg::kCopies>();
+#endif
             constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
 #pragma unroll
             for (int n = kMfmas / 2; n < kMfmas; ++n) {
@@ -561,7 +609,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                 for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
             }
             read_step(stage_next, 0);
-            read_scales(stage_next, parity ^ 1);
+            read_scales(stage_next, parity ^ 1, next_scale_offset());
 #pragma unroll
             for (int n = 0; n < kMfmas; ++n) {
                 mfma_one(1, parity, n);
@@ -571,6 +619,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                     for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
                 }
             }
+            issue_row_scales();
             advance_copy_cursor();
             stage_now = stage_next;
         }
