@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
         }
         u32x4 packed;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16(acc[2 * i]) | (f32_to_bf16(acc[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) packed[i] = pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
         store16_nt(out + static_cast<size_t>(token) * vec_per_row + v, packed);
     }
 }

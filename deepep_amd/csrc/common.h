@@ -44,13 +44,16 @@ constexpr int kWave = 64;
 // ---- device helpers -------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
-// Round-to-nearest-even fp32 -> bf16 bits (finite inputs; NaN keeps a quiet payload).
-__device__ __forceinline__ uint32_t f32_to_bf16(float v)
+// Round-to-nearest-even fp32 -> bf16 bits, two at a time: lo in bits 0-15, hi in bits 16-31
+// (v_cvt_pk_bf16_f32; NaN stays a quiet NaN).
+typedef float dpep_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 dpep_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 {
-    uint32_t bits = __float_as_uint(v);
-    if ((bits & 0x7fffffffu) > 0x7f800000u) return (bits >> 16) | 0x40u;
-    return (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+    const dpep_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, dpep_bf16x2));
 }
+__device__ __forceinline__ uint32_t f32_to_bf16(float v) { return pack_bf16x2(v, 0.0f) & 0xffffu; }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));

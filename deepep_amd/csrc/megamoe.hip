@@ -113,17 +113,27 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
         const uint8_t* src = w + (e * n + row) * (k / 2) + ks * 32 + (lane >> 5) * 16;
         reinterpret_cast<u32x4*>(w_out)[id] = *reinterpret_cast<const u32x4*>(src);
     }
-    if (id < scale_pairs) {  // two scale bytes: k blocks (2*kb + g) of one k=128 tile
-        const int lane = id & 63;
-        long long rest = id >> 6;
-        const int kt = rest % ktiles;
-        rest /= ktiles;
-        const int c = rest % ctiles;
-        const long long e = rest / ctiles;
-        const int row = source_row(c * 32 + (lane & 31), n, gate_up);
-        const uint8_t* src = s + (e * n + row) * (k / 32) + kt * 4 + (lane >> 5);
-        s_out[id * 2] = src[0];
-        s_out[id * 2 + 1] = src[2];
+    if (id < scale_pairs) {
+        // Scales: per (expert, block of 8 column tiles, span of 4 k tiles) one 4 KiB block
+        // [column tile 8][lane 64][k tile 4][2 bytes = k blocks (2*kb + g) of that k tile]; a span is what
+        // the GEMM copies in one go.  The last span is padded when k % 512 != 0.
+        const int spans = (ktiles + 3) / 4;
+        const int kq = id & 3, lane = (id >> 2) & 63, c8 = (id >> 8) & 7;
+        long long rest = id >> 11;
+        const int span = rest % spans;
+        rest /= spans;
+        const int nb = rest % (n / 256);
+        const long long e = rest / (n / 256);
+        const int kt = span * 4 + kq;
+        uint8_t lo = 127, hi = 127;
+        if (kt < ktiles) {
+            const int row = source_row((nb * 8 + c8) * 32 + (lane & 31), n, gate_up);
+            const uint8_t* src = s + (e * n + row) * (k / 32) + kt * 4 + (lane >> 5);
+            lo = src[0];
+            hi = src[2];
+        }
+        s_out[id * 2] = lo;
+        s_out[id * 2 + 1] = hi;
     }
 }
 
@@ -153,16 +163,18 @@ struct GemmCfg {
     static constexpr int kAhead = kStages - 1;
     static constexpr int kOffA = 0;                    // kBM rows x 128 B, 16-byte chunks XOR-swizzled
     static constexpr int kOffB = kBM * kBK;            // 8 column tiles x 2 k steps x 1 KiB fragments
-    static constexpr int kOffSB = kOffB + 16384;       // 8 column tiles x 64 lanes x 2 B
-    static constexpr int kStageBytes = kOffSB + 1024;
-    // per thread and item: A, B, column scales, next tile's gather indices.  The row scales travel apart:
-    // 16 bytes per row cover k = 512 and are copied once per four items into a two-slot ring, because a
-    // 4-byte copy per row and item costs a cache-line lookup per lane, as many as the whole A tile.
-    static constexpr int kCopies = 2 * RT + 4 + 1 + (kGather ? 1 : 0);
+    static constexpr int kStageBytes = kOffB + 16384;
+    static constexpr int kCopies = 2 * RT + 4;  // per thread and item: A and B, 16 bytes each
+    // Scales travel apart, once per span of four items, into two-slot rings: 16 bytes per row cover
+    // k = 512 of row scales, and one 4 KiB block holds the column scales of the span.  (4-byte copies
+    // are several times slower per instruction than 16-byte ones, and a 4-byte copy per row costs a
+    // cache-line lookup per lane.)
     static constexpr int kRowScaleSlot = kBM * 16;
+    static constexpr int kColScaleSlot = 4096;
     static constexpr int kOffRowScales = kStages * kStageBytes;
-    static constexpr int kStagingWave = 64 * kStagingRowStride;  // the epilogue handles 64 rows at a time
-    static constexpr int kOffStaging = kOffRowScales + 2 * kRowScaleSlot;
+    static constexpr int kOffColScales = kOffRowScales + 2 * kRowScaleSlot;
+    static constexpr int kStagingWave = 32 * kStagingRowStride;  // the epilogue handles one 32-row tile at a time
+    static constexpr int kOffStaging = kOffColScales + 2 * kColScaleSlot;
     static constexpr int kLdsBytes = kOffStaging + 4 * kStagingWave;
 };
 
@@ -214,6 +226,16 @@ __device__ __forceinline__ void copy16_to_lds_unless(const void* src, uint32_t l
         "v"(src), "s"(flag)
         : "memory", "scc");
 }
+__device__ __forceinline__ void copy4_to_lds_unless(const void* src, uint32_t lds_base, int skip)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    const int flag = __builtin_amdgcn_readfirstlane(skip);
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_cmp_lg_u32 %2, 0\n\ts_cbranch_scc1 .Lskip_copy_%=\n\t"
+        "global_load_lds_dword %1, off\n.Lskip_copy_%=:" ::"s"(base),
+        "v"(src), "s"(flag)
+        : "memory", "scc");
+}
 template <int kOutstanding>
 __device__ __forceinline__ void wait_copies_then_barrier()
 {
@@ -260,7 +282,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     __shared__ int tile_base[kMaxMoeExperts + 1];
     __shared__ int row_offsets[kMaxMoeExperts + 1];
-    __shared__ int next_index[kGemmThreads];  // row_to_route of the next tile's rows
+    __shared__ int tile_index[2][kGemmThreads];  // row_to_route of a tile's rows; slots alternate per tile
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS copy targets in SGPRs
@@ -269,7 +291,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     const int n_tiles = p.n / kBN;
     const int ksteps = p.k / 64, ktiles = p.k / kBK;
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
-    const uint32_t lds_index = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(next_index));
+    const uint32_t lds_index = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&tile_index[0][0]));
 
     DPEP_STAMP(0);
     // Tiles per expert: ceil(rows/kBM) row tiles x n_tiles column tiles, expert-major, row tile fastest.
@@ -319,22 +341,25 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     const uint8_t* b_src[4];
     const uint8_t* sb_src;
     const int* index_src = p.row_to_route;
-    int copy_tile = first, copy_kt = 0, copy_stage = 0, copy_span = -1;
+    int copy_tile = first, copy_kt = 0, copy_stage = 0, copy_span = -1, copy_ordinal = 0;
     const int scale_bytes = p.k / 32;  // per row
+    const int spans = (ktiles + 3) / 4;
     TileInfo next_info = decode(first);
 
+    // Tile number j of this workgroup keeps its gather indices in tile_index[j & 1].
     auto point_at_tile = [&](const TileInfo& info) {
+        const int* index = tile_index[copy_ordinal & 1];
         // rows past the tile's end repeat its last row
 #pragma unroll
         for (int i = 0; i < 2 * RT; ++i) {
             const int r = min(i * 32 + wave * 8 + (lane >> 3), info.valid - 1);
-            const int src = kGather ? next_index[r] / p.topk : info.row0 + r;
+            const int src = kGather ? index[r] / p.topk : info.row0 + r;
             a_src[i] = p.a_codes + static_cast<size_t>(src) * p.k + a_chunk;
         }
         {
             // thread t serves row t % kBM (surplus waves repeat rows, which keeps every wave's copy count equal)
             const int r = min(tid % kBM, info.valid - 1);
-            const int src = kGather ? next_index[r] / p.topk : info.row0 + r;
+            const int src = kGather ? index[r] / p.topk : info.row0 + r;
             sa_src = p.a_scales + static_cast<size_t>(src) * scale_bytes;
         }
         const uint8_t* w_block = p.w + static_cast<size_t>(info.expert) * p.n * (p.k / 2) +
@@ -345,8 +370,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             const int q = j * 4 + wave;
             b_src[j] = w_block + (static_cast<size_t>(q >> 1) * ksteps + (q & 1)) * 1024;
         }
-        sb_src = p.ws + static_cast<size_t>(info.expert) * p.n * (p.k / 32) +
-                 (static_cast<size_t>(info.nt) * (2 * kCT) + (tid >> 5)) * ktiles * 128 + (tid & 31) * 4;
+        sb_src = p.ws + (static_cast<size_t>(info.expert) * n_tiles + info.nt) * spans * Cfg::kColScaleSlot + tid * 16;
     };
     auto aim_index_prefetch = [&](const TileInfo& info) {
         if (kGather) index_src = p.row_to_route + info.row0 + min(tid, info.valid - 1);
@@ -357,37 +381,43 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 #ifdef DPEP_X_NOCOPY
         return;
 #endif
-#ifdef DPEP_X_NOSMALL
-        if (c >= 2 * RT + 4) return;
-#endif
         const uint32_t stage = lds0 + copy_stage * kStageBytes;
+#ifdef DPEP_X_SAMEADDR
+        copy16_to_lds(p.w + (DPEP_X_SAMEADDR ? lane * 16 : 0), stage + c * 4096 + wave * 1024);
+        return;
+#endif
         if (c < 2 * RT)
             copy16_to_lds(a_src[c] + static_cast<size_t>(copy_kt) * kBK, stage + Cfg::kOffA + c * 4096 + wave * 1024);
-        else if (c < 2 * RT + 4)
+        else
             copy16_to_lds(b_src[c - 2 * RT] + static_cast<size_t>(copy_kt) * 2048,
                           stage + Cfg::kOffB + ((c - 2 * RT) * 4 + wave) * 1024);
-        else if (c == 2 * RT + 4)
-            copy4_to_lds(sb_src + copy_kt * 128, stage + Cfg::kOffSB + wave * 256);
-        else if (kGather)
-            copy4_to_lds(index_src, lds_index + wave * 256);
     };
-    // Every fourth item starts a new 16-byte window of row scales (clamped so that it never leaves the
-    // row: k % 512 may be 256).  The extra copy only makes the counted waits stricter.
-    auto issue_row_scales = [&]() {
+    // Every fourth item starts a new span: a 16-byte window of row scales per row (clamped so that it never
+    // leaves the row: k % 512 may be 256) and the span's 4 KiB of column scales.  A tile's first item also
+    // fetches the gather indices of the workgroup's next tile.  These extra copies only make the counted
+    // waits stricter.
+    auto issue_span_copies = [&]() {
+#ifdef DPEP_X_NOCOPY
+        return;
+#endif
         copy_span += (copy_kt & 3) == 0 ? 1 : 0;
         const int window = min((copy_kt & ~3) * 4, scale_bytes - 16);
-        copy16_to_lds_unless(sa_src + window,
-                             lds0 + Cfg::kOffRowScales + (copy_span & 1) * Cfg::kRowScaleSlot + ((wave * 64) % kBM) * 16,
+        const int slot = copy_span & 1;
+        copy16_to_lds_unless(sa_src + window, lds0 + Cfg::kOffRowScales + slot * Cfg::kRowScaleSlot + ((wave * 64) % kBM) * 16,
                              copy_kt & 3);
+        copy16_to_lds_unless(sb_src + static_cast<size_t>(copy_kt >> 2) * Cfg::kColScaleSlot,
+                             lds0 + Cfg::kOffColScales + slot * Cfg::kColScaleSlot + wave * 1024, copy_kt & 3);
+        if (kGather) copy4_to_lds_unless(index_src, lds_index + ((copy_ordinal + 1) & 1) * (kGemmThreads * 4) + wave * 256, copy_kt);
     };
     auto advance_copy_cursor = [&]() {
         copy_stage = copy_stage + 1 == kStages ? 0 : copy_stage + 1;
         if (++copy_kt == ktiles) {
             if (copy_tile + stride < total_tiles) {
-                // The next tile's indices have been landing in next_index since the previous switch
-                // (at least kAhead items ago because ktiles >= kAhead), so this needs no global load.
+                // The next tile's indices were fetched with this tile's first item (at least kAhead items
+                // ago because ktiles >= kAhead), so switching needs no global load.
                 copy_tile += stride;
                 copy_kt = 0;
+                ++copy_ordinal;
                 point_at_tile(next_info);
                 if (copy_tile + stride < total_tiles) next_info = decode(copy_tile + stride);
                 aim_index_prefetch(next_info);
@@ -399,7 +429,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     auto issue_item = [&]() {
 #pragma unroll
         for (int c = 0; c < Cfg::kCopies; ++c) issue_copy(c);
-        issue_row_scales();
+        issue_span_copies();
         advance_copy_cursor();
     };
 
@@ -429,7 +459,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         sa_addr[i] = Cfg::kOffRowScales + row * 16;
     }
     const int b_addr = Cfg::kOffB + wn * kCT * 2048 + lane * 16;
-    const int sb_addr = Cfg::kOffSB + wn * kCT * 128 + lane * 2;
+    const int sb_addr = Cfg::kOffColScales + wn * kCT * 512 + lane * 8;
 
     v8i afrag[2][RT];     // [k step][row tile]
     u32x4 bfrag[2][kCT];  // [k step][column tile]
@@ -446,14 +476,13 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 #pragma unroll
         for (int c = 0; c < kCT; ++c) bfrag[kb][c] = *reinterpret_cast<const u32x4*>(stage + b_addr + (c * 2 + kb) * 1024);
     };
-    // scale_at = byte offset of the item's row-scale word: ring slot + position inside the 16-byte window
-    auto read_scales = [&](int stage_index, int slot, int scale_at) {
-        const uint8_t* stage = lds + stage_index * kStageBytes;
+    // row_at / col_at = byte offsets of the item's scales: ring slot + position inside the span
+    auto read_scales = [&](int slot, int row_at, int col_at) {
 #pragma unroll
-        for (int i = 0; i < RT; ++i) ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + sa_addr[i] + scale_at));
+        for (int i = 0; i < RT; ++i) ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + sa_addr[i] + row_at));
 #pragma unroll
         for (int c = 0; c < kCT; ++c)
-            bscale[slot][c] = static_cast<int>(*reinterpret_cast<const uint16_t*>(stage + sb_addr + c * 128));
+            bscale[slot][c] = static_cast<int>(*reinterpret_cast<const uint16_t*>(lds + sb_addr + c * 512 + col_at));
     };
 
     v16f acc[RT][kCT];
@@ -483,73 +512,71 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     uint8_t* region = lds + Cfg::kOffStaging + wave * Cfg::kStagingWave;
     auto epilogue = [&](const TileInfo& info) {
         constexpr int kPasses = kGateUp ? kCT / 2 : kCT;
-        // The staging region holds 64 rows (two row tiles) x 32 columns; larger wave tiles take several turns.
+        // The staging region holds one 32 x 32 tile as BF16 rows.
 #pragma unroll
-        for (int i0 = 0; i0 < RT; i0 += 2) {
-            constexpr int kTilesMax = 2;
-            const int tiles_here = RT - i0 < kTilesMax ? RT - i0 : kTilesMax;
-            const int chunk_rows = min(32 * tiles_here, info.valid - wm * 32 * RT - 32 * i0);  // may be <= 0
-            const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT + 32 * i0;
+        for (int i = 0; i < RT; ++i) {
+            const int tile_rows = min(32, info.valid - wm * 32 * RT - 32 * i);  // may be <= 0
+            const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT + 32 * i;
 #pragma unroll
             for (int pass = 0; pass < kPasses; ++pass) {
 #pragma unroll
-                for (int ii = 0; ii < kTilesMax; ++ii) {
-                    if (i0 + ii >= RT) continue;
-                    const int i = i0 + ii;
+                for (int j = 0; j < 16; j += 2) {
+                    float value[2];
 #pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        const int r = ii * 32 + (j >> 2) * 8 + g * 4 + (j & 3);
-                        float value;
+                    for (int d = 0; d < 2; ++d) {
                         if (kGateUp) {
                             // column tiles alternate gate / up for the same 32 activation columns
-                            const float gate = bf16_to_f32(f32_to_bf16(acc[i][2 * pass][j]));
-                            const float up = bf16_to_f32(f32_to_bf16(acc[i][2 * pass + 1][j]));
-                            value = silu_mul(gate, up);
+                            const uint32_t rounded = pack_bf16x2(acc[i][2 * pass][j + d], acc[i][2 * pass + 1][j + d]);
+                            value[d] = silu_mul(__uint_as_float(rounded << 16), __uint_as_float(rounded & 0xffff0000u));
                         } else {
-                            value = acc[i][pass][j];
+                            value[d] = acc[i][pass][j + d];
                         }
-                        *reinterpret_cast<uint16_t*>(region + r * kStagingRowStride + lr * 2) = static_cast<uint16_t>(f32_to_bf16(value));
                     }
+                    const uint32_t pair = pack_bf16x2(value[0], value[1]);  // rows r and r + 1 of this lane's column
+                    const int r = (j >> 2) * 8 + g * 4 + (j & 3);
+                    uint8_t* cell = region + r * kStagingRowStride + lr * 2;
+                    *reinterpret_cast<uint16_t*>(cell) = static_cast<uint16_t>(pair);
+                    *reinterpret_cast<uint16_t*>(cell + kStagingRowStride) = static_cast<uint16_t>(pair >> 16);
                 }
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 if (kGateUp) {
-                    // each lane requantises a whole row: 32 BF16 -> e8m0 byte + 32 e4m3 codes
+                    // two lanes requantise one row: 2 x 16 BF16 -> e8m0 byte + 32 e4m3 codes
                     const int act_width = p.n / 2;
                     const int act_col = (info.nt * kCT + wn * (kCT / 2) + pass) * 32;
-                    const int r = lane;
-                    if (r < chunk_rows) {
-                        float v[32];
+                    const int r = lane >> 1, half = lane & 1;
+                    float v[16];
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const u32x4 raw = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + q * 16);
+                    for (int q = 0; q < 2; ++q) {
+                        const u32x4 raw = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + half * 32 + q * 16);
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) {
-                                v[q * 8 + 2 * t] = bf16_to_f32(raw[t] & 0xffffu);
-                                v[q * 8 + 2 * t + 1] = bf16_to_f32(raw[t] >> 16);
-                            }
+                        for (int t = 0; t < 4; ++t) {
+                            v[q * 8 + 2 * t] = bf16_to_f32(raw[t] & 0xffffu);
+                            v[q * 8 + 2 * t + 1] = bf16_to_f32(raw[t] >> 16);
                         }
-                        float amax = 0.0f;
+                    }
+                    float amax = 0.0f;
 #pragma unroll
-                        for (int t = 0; t < 32; ++t) amax = fmaxf(amax, fabsf(v[t]));
-                        const int byte = mx_scale_byte(amax);
-                        u32x4 codes[2];
+                    for (int t = 0; t < 16; ++t) amax = fmaxf(amax, fabsf(v[t]));
+                    amax = fmaxf(amax, __shfl_xor(amax, 1));
+                    const int byte = mx_scale_byte(amax);
+                    u32x4 codes;
 #pragma unroll
-                        for (int t = 0; t < 8; ++t)
-                            codes[t >> 2][t & 3] = pack4_e4m3(mx_scaled(v[4 * t], byte), mx_scaled(v[4 * t + 1], byte),
-                                                              mx_scaled(v[4 * t + 2], byte), mx_scaled(v[4 * t + 3], byte));
-                        uint8_t* dst = p.act_codes + (out_row0 + r) * act_width + act_col;
-                        *reinterpret_cast<u32x4*>(dst) = codes[0];
-                        *reinterpret_cast<u32x4*>(dst + 16) = codes[1];
-                        p.act_scales[(out_row0 + r) * (act_width / 32) + (act_col >> 5)] = static_cast<uint8_t>(byte);
+                    for (int t = 0; t < 4; ++t)
+                        codes[t] = pack4_e4m3(mx_scaled(v[4 * t], byte), mx_scaled(v[4 * t + 1], byte),
+                                              mx_scaled(v[4 * t + 2], byte), mx_scaled(v[4 * t + 3], byte));
+                    if (r < tile_rows) {
+                        *reinterpret_cast<u32x4*>(p.act_codes + (out_row0 + r) * act_width + act_col + half * 16) = codes;
+                        if (half == 0)
+                            p.act_scales[(out_row0 + r) * (act_width / 32) + (act_col >> 5)] = static_cast<uint8_t>(byte);
                     }
                 } else {
                     // 4 lanes carry one 64-byte row segment
                     const int col = info.nt * kBN + (wn * kCT + pass) * 32 + (lane & 3) * 8;
 #pragma unroll
-                    for (int it = 0; it < 2 * kTilesMax; ++it) {
+                    for (int it = 0; it < 2; ++it) {
                         const int r = it * 16 + (lane >> 2);
-                        if (r < chunk_rows) {
+                        if (r < tile_rows) {
                             const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
                             store16_nt(p.out + (out_row0 + r) * p.n + col, chunk);
                         }
@@ -566,17 +593,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 #pragma unroll
     for (int j = 0; j < kAhead; ++j) issue_item();
     wait_copies_then_barrier<(kAhead - 1) * Cfg::kCopies>();  // item 0 has landed
-    // Row-scale bookkeeping of the item whose fragments are read next: span counter (ring slot) and k tile.
+    // Scale bookkeeping of the item whose fragments are read next: span counter (ring slot) and k tile.
     int read_span = -1, read_kt = 0;
-    auto next_scale_offset = [&]() {
+    auto read_next_scales = [&](int slot) {
         if ((read_kt & 3) == 0) ++read_span;
         const int window = min((read_kt & ~3) * 4, scale_bytes - 16);
-        const int at = (read_span & 1) * Cfg::kRowScaleSlot + (read_kt * 4 - window);
+        const int ring = read_span & 1;
+        read_scales(slot, ring * Cfg::kRowScaleSlot + (read_kt * 4 - window), ring * Cfg::kColScaleSlot + (read_kt & 3) * 2);
         read_kt = read_kt + 1 == ktiles ? 0 : read_kt + 1;
-        return at;
     };
     read_step(0, 0);
-    read_scales(0, 0, next_scale_offset());
+    read_next_scales(0);
     clear_acc();
     asm volatile("s_nop 3");
     DPEP_STAMP(3);
@@ -597,7 +624,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             for (int n = 0; n < kMfmas / 2; ++n) mfma_one(0, parity, n);
             // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies in
             // flight; past the barrier every wave has also finished reading the stage refilled next.
-#ifndef DPEP_X_NOBARRIER
+#ifdef DPEP_X_LOOSEWAIT
+            wait_copies_then_barrier<(kAhead - 1) * Cfg::kCopies>();
+#elif !defined(DPEP_X_NOBARRIER)
             wait_copies_then_barrier<(kAhead - 2) * Cfg::kCopies>();
 #endif
             constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
@@ -609,7 +638,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                 for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
             }
             read_step(stage_next, 0);
-            read_scales(stage_next, parity ^ 1, next_scale_offset());
+            read_next_scales(parity ^ 1);
 #pragma unroll
             for (int n = 0; n < kMfmas; ++n) {
                 mfma_one(1, parity, n);
@@ -619,7 +648,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                     for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
                 }
             }
-            issue_row_scales();
+            issue_span_copies();
             advance_copy_cursor();
             stage_now = stage_next;
         }
@@ -742,19 +771,25 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
     return launch_status("mx_quant");
 }
 
+size_t dpep_megamoe_prepared_scale_bytes(int num_local, int n, int k)
+{
+    if (num_local < 1 || n < 1 || k < 1) return 0;
+    const size_t spans = (static_cast<size_t>(k) / 128 + 3) / 4;  // groups of four k tiles, the last one padded
+    return static_cast<size_t>(num_local) * n * spans * 16;
+}
+
 int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scales, int num_local, int n, int k,
                                  int gate_up, uint8_t* out_packed, uint8_t* out_scales, void* stream)
 {
     using namespace dpep;
     DPEP_REQUIRE(num_local >= 1, "prepare_weights: bad expert count %d", num_local);
-    DPEP_REQUIRE(k > 0 && k % 128 == 0, "prepare_weights: K=%d must be a positive multiple of 128", k);
-    DPEP_REQUIRE(n > 0 && n % (gate_up ? 64 : 32) == 0, "prepare_weights: N=%d must be a positive multiple of %d", n,
-                 gate_up ? 64 : 32);
+    DPEP_REQUIRE(k > 0 && k % 256 == 0, "prepare_weights: K=%d must be a positive multiple of 256", k);
+    DPEP_REQUIRE(n > 0 && n % kBN == 0, "prepare_weights: N=%d must be a positive multiple of %d", n, kBN);
     DPEP_REQUIRE(w_packed && w_scales && out_packed && out_scales && aligned16(w_packed) && aligned16(out_packed),
                  "prepare_weights: NULL or misaligned buffer");
     DPEP_REQUIRE(w_packed != out_packed && w_scales != out_scales, "prepare_weights: cannot run in place");
     const long long chunks = static_cast<long long>(num_local) * n * (k / 2) / 16;
-    const long long pairs = static_cast<long long>(num_local) * n * (k / 32) / 2;
+    const long long pairs = static_cast<long long>(dpep_megamoe_prepared_scale_bytes(num_local, n, k) / 2);
     const unsigned blocks = static_cast<unsigned>((chunks + 255) / 256);
     hipLaunchKernelGGL(prepare_weights_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), w_packed,
                        w_scales, n, k, gate_up, out_packed, out_scales, chunks, pairs);

@@ -240,8 +240,15 @@ def megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_loca
     return int(_lib.load().dpep_megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local))
 
 
+def megamoe_prepared_scale_cols(k: int) -> int:
+    """Bytes per output column of a prepared scale tensor: spans of k = 512 (16 bytes each), the last one padded."""
+    return (k // 128 + 3) // 4 * 16
+
+
 def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
-    """Raw packed FP4 uint8 [L,N,K/2] + e8m0 uint8 [L,N,K/32] -> the kernel's streaming order (same sizes)."""
+    """Raw packed FP4 uint8 [L,N,K/2] + e8m0 uint8 [L,N,K/32] -> the kernel's streaming order.
+
+    Returns (packed [L,N,K/2], scales [L,N,megamoe_prepared_scale_cols(K)])."""
     lib = _lib.load()
     _require("w_packed", w_packed, torch.uint8)
     if w_packed.ndim != 3:
@@ -250,7 +257,9 @@ def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
     k = half_k * 2
     _require("w_scales", w_scales.reshape(experts, n, -1), torch.uint8, (experts, n, k // 32), w_packed.device)
     out_w = torch.empty_like(w_packed)
-    out_s = torch.empty((experts, n, k // 32), dtype=torch.uint8, device=w_packed.device)
+    out_s = torch.empty((experts, n, megamoe_prepared_scale_cols(k)), dtype=torch.uint8, device=w_packed.device)
+    if out_s.numel() != lib.dpep_megamoe_prepared_scale_bytes(experts, n, k):
+        raise RuntimeError("prepared scale size disagrees with the library")
     with torch.cuda.device(w_packed.device):
         status = lib.dpep_megamoe_prepare_weights(
             _ptr(w_packed), _ptr(w_scales), experts, n, k, int(bool(gate_up)), _ptr(out_w), _ptr(out_s),
@@ -276,9 +285,9 @@ def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s
     if w1.ndim != 3 or w1.shape[0] != num_local or w1.shape[2] * 2 != hidden or w1.shape[1] % 2:
         raise ValueError("w1 must be prepared [L, 2I, H/2]")
     intermediate = w1.shape[1] // 2
-    _require("s1", s1, torch.uint8, (num_local, 2 * intermediate, hidden // 32), dev)
+    _require("s1", s1, torch.uint8, (num_local, 2 * intermediate, megamoe_prepared_scale_cols(hidden)), dev)
     _require("w2", w2, torch.uint8, (num_local, hidden, intermediate // 2), dev)
-    _require("s2", s2, torch.uint8, (num_local, hidden, intermediate // 32), dev)
+    _require("s2", s2, torch.uint8, (num_local, hidden, megamoe_prepared_scale_cols(intermediate)), dev)
     _require("y", y, torch.bfloat16, (tokens, hidden), dev)
     _require("expert_token_nums", expert_token_nums, torch.int32, (num_local,), dev)
     with torch.cuda.device(dev):

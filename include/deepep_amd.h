@@ -102,9 +102,15 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
 /* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480). */
 size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, int intermediate, int num_local);
 
+/* Bytes of the prepared scale buffer of one weight tensor: the scales are stored in spans of four k tiles
+ * (k = 512), the last span padded, so this equals L*N*K/32 when K % 512 == 0 and is larger otherwise.
+ * (Part of the transform_weights_for_mega_moe contract below.) */
+size_t dpep_megamoe_prepared_scale_bytes(int num_local, int n, int k);
+
 /* One-off weight re-layout (transform_weights_for_mega_moe, experiments/megamoe/python/.../api.py:311-379):
- * raw packed FP4 [L,N,K/2] + e8m0 [L,N,K/32]  ->  the tile order the GEMM kernel streams.
- * Byte shuffle only; out buffers have the same sizes as the inputs.  gate_up != 0 (first GEMM, N = 2I,
+ * raw packed FP4 [L,N,K/2] + e8m0 [L,N,K/32]  ->  the tile order the GEMM kernel streams
+ * (N % 256 == 0, K % 256 == 0).  Byte shuffle only; out_packed has the size of w_packed, out_scales has
+ * dpep_megamoe_prepared_scale_bytes(L, N, K) bytes.  gate_up != 0 (first GEMM, N = 2I,
  * gate rows then up rows) interleaves gate and up in groups of 32 output columns so SwiGLU is lane-local
  * (the counterpart of _interleave_gate_up_128, api.py:285-293). */
 int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scales, int num_local, int n,
@@ -115,7 +121,8 @@ int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scale
  * layout -> gather rows -> GMM1 (MXFP8 x MXFP4) -> bf16 -> SwiGLU -> MXFP8 requant -> GMM2 -> bf16 ->
  * route-weighted fp32 reduce per token -> bf16.
  *   x_codes e4m3 [B,H], x_scales e8m0 [B,H/32], topk_idx int32 [B,K] (distinct, in [0,E)), topk_weights fp32 [B,K]
- *   w1/s1: prepared GMM1 weights [L,2I,H/2] / [L,2I,H/32]; w2/s2: prepared GMM2 weights [L,H,I/2] / [L,H,I/32]
+ *   w1/s1: prepared GMM1 weights [L,2I,H/2] and scales; w2/s2: prepared GMM2 weights [L,H,I/2] and scales
+ *   (scale sizes: dpep_megamoe_prepared_scale_bytes)
  *   y bf16 [B,H]; expert_token_nums int32 [L] */
 int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales, const int32_t* topk_idx,
                          const float* topk_weights, const uint8_t* w1, const uint8_t* s1, const uint8_t* w2,
