@@ -43,9 +43,17 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
         if (part == 0 && return_out != nullptr && threadIdx.x < num_topk)
             return_out[static_cast<size_t>(token) * num_topk + threadIdx.x] = row >= 0 ? return_in[row] : 0.0f;
     }
-    __syncthreads();
+    // Tokens without any row (the common case of a sparse receive share) are plain zero fill.  Streaming
+    // stores: cached ones would push the rows read next, and the caller's other data, out of the caches.
+    const bool any_row = __syncthreads_or(threadIdx.x < num_topk && rows[threadIdx.x] >= 0) != 0;
     const int v_begin = part * vec_per_part;
     const int v_end = min(v_begin + vec_per_part, vec_per_row);
+    if (!any_row) {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x)
+            store16_nt(out + static_cast<size_t>(token) * vec_per_row + v, zero);
+        return;
+    }
     for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x) {
         float acc[8];
 #pragma unroll
@@ -82,8 +90,12 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
 }
 
 struct CombineGrid {
-    int parts, per_part, threads;
+    int parts, per_part, threads, blocks;
 };
+#ifndef DPEP_TUNE_SPARSE_TARGET
+#define DPEP_TUNE_SPARSE_TARGET 2048
+#endif
+
 
 // Dense routing (at least one row per token on average): split every token row into 1-2 KiB parts.
 // Sparse receive shares (most tokens own no row and only get zero-filled): one workgroup per token
@@ -91,14 +103,24 @@ struct CombineGrid {
 CombineGrid combine_grid(int num_tokens, int num_rows, int vec)
 {
     CombineGrid g;
-    const int target = num_rows >= num_tokens ? DPEP_TUNE_TARGET_BLOCKS : 2048;
+    const int target = num_rows >= num_tokens ? DPEP_TUNE_TARGET_BLOCKS : DPEP_TUNE_SPARSE_TARGET;
     int parts = 1;
     while (num_tokens * parts < target && vec / (parts * 2) >= 64 && parts < 16) parts *= 2;
     g.per_part = (vec + parts - 1) / parts;
     g.parts = (vec + g.per_part - 1) / g.per_part;
     int threads = (g.per_part + 63) / 64 * 64;
     g.threads = threads > kMaxThreads ? kMaxThreads : (threads < 64 ? 64 : threads);
+    g.blocks = num_tokens * g.parts;
     return g;
+}
+
+template <int kWeights>
+void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, const float* weights, const int32_t* route_to_row,
+                    int num_topk, int vec, void* out, const float* return_in, float* return_out)
+{
+    hipLaunchKernelGGL(combine_kernel<kWeights>, dim3(g.blocks), dim3(g.threads), 0, stream, static_cast<const u32x4*>(y),
+                       weights, route_to_row, num_topk, vec, g.per_part, g.parts, static_cast<u32x4*>(out), return_in,
+                       return_out);
 }
 
 }  // namespace
@@ -109,9 +131,7 @@ int combine_routes(const void* y, const float* route_weights, const int32_t* rou
 {
     const int vec = hidden / 8;
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
-    hipLaunchKernelGGL(combine_kernel<2>, dim3(num_tokens * g.parts), dim3(g.threads), 0, stream,
-                       static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk, vec, g.per_part, g.parts,
-                       static_cast<u32x4*>(out), nullptr, nullptr);
+    launch_combine<2>(g, stream, y, route_weights, route_to_row, num_topk, vec, out, nullptr, nullptr);
     return launch_status("combine_routes");
 }
 
@@ -136,13 +156,9 @@ int dpep_combine(const void* y, const float* row_weights, const int32_t* route_t
     const CombineGrid g = combine_grid(num_tokens, num_rows, vec);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (row_weights != nullptr)
-        hipLaunchKernelGGL(combine_kernel<1>, dim3(num_tokens * g.parts), dim3(g.threads), 0, s,
-                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, g.per_part, g.parts,
-                           static_cast<u32x4*>(out), return_in, return_out);
+        launch_combine<1>(g, s, y, row_weights, route_to_row, num_topk, vec, out, return_in, return_out);
     else
-        hipLaunchKernelGGL(combine_kernel<0>, dim3(num_tokens * g.parts), dim3(g.threads), 0, s,
-                           static_cast<const u32x4*>(y), row_weights, route_to_row, num_topk, vec, g.per_part, g.parts,
-                           static_cast<u32x4*>(out), return_in, return_out);
+        launch_combine<0>(g, s, y, nullptr, route_to_row, num_topk, vec, out, return_in, return_out);
     return launch_status("combine");
 }
 

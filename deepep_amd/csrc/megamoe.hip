@@ -209,6 +209,14 @@ __device__ __forceinline__ void copy16_to_lds(const void* src, uint32_t lds_base
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(src) : "memory");
 }
+// The same with the address split into a wave-uniform 64-bit base (SGPR pair) and a 32-bit lane offset.
+__device__ __forceinline__ void copy16_to_lds(const void* uniform_base, uint32_t lane_offset, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(base), "v"(lane_offset),
+                 "s"(uniform_base)
+                 : "memory");
+}
 __device__ __forceinline__ void copy4_to_lds(const void* src, uint32_t lds_base)
 {
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
@@ -336,9 +344,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     // ---- copy cursor -------------------------------------------------------------------------------
     // copy i of wave w fills LDS rows i*32 + w*8 + lane/8; chunk (lane%8) ^ ((row>>1)&7) of the 128-byte row
     const int a_chunk = ((lane & 7) ^ ((wave * 4 + (lane >> 4)) & 7)) * 16;
-    const uint8_t* a_src[2 * RT];
+    uint32_t a_off[2 * RT];  // lane offsets from p.a_codes: source row * K + chunk
     const uint8_t* sa_src;
-    const uint8_t* b_src[4];
+    uint32_t b_off[4];       // lane offsets from the tile's first weight fragment
+    const uint8_t* b_base = p.w;
     const uint8_t* sb_src;
     const int* index_src = p.row_to_route;
     int copy_tile = first, copy_kt = 0, copy_stage = 0, copy_span = -1, copy_ordinal = 0;
@@ -354,7 +363,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         for (int i = 0; i < 2 * RT; ++i) {
             const int r = min(i * 32 + wave * 8 + (lane >> 3), info.valid - 1);
             const int src = kGather ? index[r] / p.topk : info.row0 + r;
-            a_src[i] = p.a_codes + static_cast<size_t>(src) * p.k + a_chunk;
+            a_off[i] = static_cast<uint32_t>(src) * static_cast<uint32_t>(p.k) + a_chunk;
         }
         {
             // thread t serves row t % kBM (surplus waves repeat rows, which keeps every wave's copy count equal)
@@ -362,13 +371,13 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             const int src = kGather ? index[r] / p.topk : info.row0 + r;
             sa_src = p.a_scales + static_cast<size_t>(src) * scale_bytes;
         }
-        const uint8_t* w_block = p.w + static_cast<size_t>(info.expert) * p.n * (p.k / 2) +
-                                 static_cast<size_t>(info.nt) * (2 * kCT) * ksteps * 1024 + lane * 16;
+        b_base = p.w + static_cast<size_t>(info.expert) * p.n * (p.k / 2) +
+                 static_cast<size_t>(info.nt) * (2 * kCT) * ksteps * 1024;
         // fragment q = copy*4 + wave of the 16 (column tile, k step) fragments of one k tile
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int q = j * 4 + wave;
-            b_src[j] = w_block + (static_cast<size_t>(q >> 1) * ksteps + (q & 1)) * 1024;
+            b_off[j] = static_cast<uint32_t>(((q >> 1) * ksteps + (q & 1)) * 1024 + lane * 16);
         }
         sb_src = p.ws + (static_cast<size_t>(info.expert) * n_tiles + info.nt) * spans * Cfg::kColScaleSlot + tid * 16;
     };
@@ -387,9 +396,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         return;
 #endif
         if (c < 2 * RT)
-            copy16_to_lds(a_src[c] + static_cast<size_t>(copy_kt) * kBK, stage + Cfg::kOffA + c * 4096 + wave * 1024);
+            copy16_to_lds(p.a_codes + static_cast<size_t>(copy_kt) * kBK, a_off[c], stage + Cfg::kOffA + c * 4096 + wave * 1024);
         else
-            copy16_to_lds(b_src[c - 2 * RT] + static_cast<size_t>(copy_kt) * 2048,
+            copy16_to_lds(b_base + static_cast<size_t>(copy_kt) * 2048, b_off[c - 2 * RT],
                           stage + Cfg::kOffB + ((c - 2 * RT) * 4 + wave) * 1024);
     };
     // Every fourth item starts a new span: a 16-byte window of row scales per row (clamped so that it never
@@ -578,7 +587,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                         const int r = it * 16 + (lane >> 2);
                         if (r < tile_rows) {
                             const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
-                            store16_nt(p.out + (out_row0 + r) * p.n + col, chunk);
+                            // cached store: the weighted reduce that follows reads these rows back at once
+                            *reinterpret_cast<u32x4*>(p.out + (out_row0 + r) * p.n + col) = chunk;
                         }
                     }
                 }
@@ -845,6 +855,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     DPEP_REQUIRE(x_codes && x_scales && topk_idx && topk_weights && w1 && s1 && w2 && s2 && y && expert_token_nums,
                  "megamoe_forward: NULL buffer");
     DPEP_REQUIRE(aligned16(x_codes) && aligned16(w1) && aligned16(w2) && aligned16(y), "megamoe_forward: misaligned buffer");
+    // the GEMM's copies address activation rows with 32-bit byte offsets
+    DPEP_REQUIRE(static_cast<long long>(num_tokens) * hidden < (1LL << 32) &&
+                     static_cast<long long>(num_tokens) * (num_topk < num_local ? num_topk : num_local) * intermediate < (1LL << 32),
+                 "megamoe_forward: activation tensors of B=%d tokens exceed 4 GiB", num_tokens);
     const MegaLayout l = mega_layout(num_tokens, num_topk, hidden, intermediate, num_local);
     DPEP_REQUIRE(l.total <= w->bytes, "megamoe_forward: workspace too small (%zu needed, %zu available)", l.total, w->bytes);
     hipStream_t s = static_cast<hipStream_t>(stream);
