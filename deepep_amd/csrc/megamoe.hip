@@ -144,9 +144,13 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
 // (two MFMA k steps) per LDS stage.  Workgroups are persistent (one per CU) and treat their tiles as ONE
 // flat stream of (tile, k tile) items: asynchronous global->LDS copies run kAhead items ahead of the
 // MFMAs and roll straight into the next tile, so a tile's epilogue overlaps the next tile's first copies.
-// Per item there is one vmcnt wait + one barrier, placed between the two k steps; the fragments of the
-// next k step leave LDS while the MFMAs of the current one run.  The gather indices of the NEXT tile
-// are copied into LDS with every item, so switching tiles needs no blocking global load.
+// Per item there is one vmcnt wait + one barrier; the fragments of the next k step leave LDS while the
+// MFMAs of the current one run.  A wave owns its SIMD alone and issues in order, so everything that is not
+// an MFMA is placed in the shadow of one: the MFMAs are volatile asm statements (they keep source order;
+// builtin MFMAs get gathered into bursts) and the item's copies are dealt out one after each MFMA.
+// Scales and gather indices do not travel with every item (a 4-byte copy costs more per instruction than
+// a 16-byte one): row scales (16 B per row = k 512), column scales (4 KiB per k 512) and
+// the next tile's gather indices (once per tile) are fetched per span of four items.
 // Rows are fetched 128 bytes at a time (full cache lines): the texture path handles about one line per
 // cycle and CU, which a 64-byte k tile would saturate.
 constexpr int kBK = 128;           // k per LDS stage = two MFMA k steps
