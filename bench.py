@@ -48,6 +48,22 @@ def time_kernel(fn, iters, torch):
     return start.elapsed_time(stop) * 1000.0 / iters
 
 
+def time_kernel_cold(fn, iters, torch, flush):
+    """Per-launch device times with the caches flushed before every launch (a 256 MiB fill, the way the
+    reference's flush_l2_cache does, deep_ep/utils/testing.py:27-35): mean / min / p50 / p95 in microseconds."""
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    fn()
+    for start, stop in pairs:
+        flush.zero_()
+        start.record()
+        fn()
+        stop.record()
+    torch.cuda.synchronize()
+    times = sorted(a.elapsed_time(b) * 1000.0 for a, b in pairs)
+    pick = lambda q: times[min(len(times) - 1, int(q * len(times)))]
+    return dict(mean=sum(times) / len(times), min=times[0], p50=pick(0.5), p95=pick(0.95))
+
+
 def cpu_baseline(x, idx, w, grads, cfg, nbytes):
     """The reference CPU path (torch CPU, all host threads) on the same inputs."""
     import torch
@@ -210,6 +226,12 @@ def main():
         combine=time_kernel(lambda: ops.combine(grows, r2row, out=out_buf), it, torch),
         combine_weighted=time_kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), it, torch),
     )
+    flush = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    cold = dict(
+        dispatch_fp8_quant=time_kernel_cold(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), 30, torch, flush),
+        combine=time_kernel_cold(lambda: ops.combine(grows, r2row, out=out_buf), 30, torch, flush),
+    )
+    del flush
     bf16_dispatch_bytes = tokens * hidden * 2 + tokens * topk * 4 + rows * hidden * 2 + rows * 4
     kernels = {
         "layout": dict(us=us["layout"], bytes=nbytes["layout"]),
@@ -258,6 +280,7 @@ def main():
             "traffic": 527.5e6,
         },
         "kernels": kernels,
+        "kernels_cache_flushed_us": cold,
         "dispatch_plus_combine_us": us["dispatch_fp8_quant"] + us["combine"],
     }
     if args.calibrate_copy:

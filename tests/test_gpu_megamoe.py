@@ -89,6 +89,8 @@ def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local):
         (300, 512, 512, 8, 2, 3, 4),     # ragged rows, local range inside E, partial tiles
         (257, 1024, 512, 6, 0, 6, 6),    # every token hits every expert
         (96, 512, 768, 8, 6, 2, 1),      # some local experts may be empty
+        (200, 768, 1280, 4, 0, 4, 3),    # K of both GEMMs not a multiple of 512 (padded last scale span)
+        (128, 512, 512, 64, 16, 32, 2),  # many local experts, most with a handful of rows, some empty
     ],
 )
 def test_megamoe_forward_matches_oracle(ops, tokens, hidden, inter, experts, begin, local, topk):
