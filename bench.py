@@ -194,7 +194,7 @@ def main():
 
     def step():
         lay = ops.layout(ws, idxd, experts)
-        rows = int(lay["num_rows"].item())  # the read-back a fresh dispatch needs to size its outputs
+        _, rows = ops.layout_wait(ws)  # the host synchronisation a fresh dispatch needs to size its outputs
         recv = ops.dispatch_quant_fp8(xd, wd, lay["route_to_row"], lay["row_to_route"], rows)
         out = ops.combine(gd[:rows], lay["route_to_row"])
         return rows, recv, out

@@ -25,6 +25,7 @@ SIGNATURES = {
     "dpep_workspace_capacity": (_I, (_P, ctypes.POINTER(_Z))),
     "dpep_layout_workspace_bytes": (_Z, (_I, _I, _I)),
     "dpep_layout": (_I, (_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P)),
+    "dpep_layout_wait": (_I, (_P, _P, _I, ctypes.POINTER(ctypes.c_int32), ctypes.c_longlong)),
     "dpep_dispatch_copy": (_I, (_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_dispatch_quant_fp8": (_I, (_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_cast_to_fp8": (_I, (_P, _I, _I, _P, _P, _P)),

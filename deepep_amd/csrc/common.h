@@ -35,7 +35,15 @@ struct Workspace {
     uint32_t magic;
     void* base;
     size_t bytes;
+    // Host mailbox of the routing layout: pinned host memory the layout kernel writes straight into
+    // (word 0 = rows, word 1 = sequence number of the launch, words 2.. = rows per local expert), so that
+    // the host learns the output sizes by polling instead of a device-to-host copy plus a stream wait.
+    uint32_t* mailbox_host;
+    uint32_t* mailbox_device;  // the same memory as the kernels address it
+    uint32_t sequence;         // of the most recent layout launch
+    int mailbox_local;         // its number of local experts
 };
+constexpr int kMailboxWords = 2 + DPEP_MAX_LOCAL_EXPERTS;
 constexpr uint32_t kWorkspaceMagic = 0x44504550u;  // "DPEP"
 Workspace* as_workspace(void* ws);
 

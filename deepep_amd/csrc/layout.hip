@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
     const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int padded_local,
     int nbits, int chunk, int num_chunks, const int* __restrict__ hist, int* __restrict__ counts,
     int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows, int* __restrict__ route_to_row,
-    int* __restrict__ row_to_route)
+    int* __restrict__ row_to_route, uint32_t* __restrict__ mailbox, uint32_t sequence)
 {
     // totals[e]: rows of expert e (later its exclusive offset); running[w][e]: next row of expert e for wave w.
     __shared__ int totals[DPEP_MAX_LOCAL_EXPERTS];
@@ -191,6 +191,7 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
             for (int w = 0; w < kWaves; ++w) running[w][e] += offset;
             if (blockIdx.x == 0) {
                 counts[e] = mine[j];
+                mailbox[2 + e] = static_cast<uint32_t>(mine[j]);  // pinned host memory
                 psum[e] = offset + mine[j];
                 offsets[e + 1] = offset + mine[j];
             }
@@ -201,7 +202,14 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
         offsets[0] = 0;
         num_rows[0] = offset;
     }
+    // The host polls the mailbox's sequence word: publish it (with the row count, one 8-byte store) after
+    // every per-expert count of this workgroup has reached host memory.
+    if (blockIdx.x == 0) __threadfence_system();
     __syncthreads();
+    if (blockIdx.x == 0 && tid == kThreads - 1) {
+        const unsigned long long word = (static_cast<unsigned long long>(sequence) << 32) | static_cast<uint32_t>(offset);
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), word, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 
     const int g = chunk0 + wave;
     if (g >= num_chunks) return;
@@ -281,9 +289,11 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
         if (int rc = launch_status("layout_count")) return rc;
     }
     // With no routes one workgroup still publishes the all-zero counts and prefix sums.
+    w->sequence = w->sequence == 0xffffffffu ? 1u : w->sequence + 1u;  // never 0: that is "nothing launched"
+    w->mailbox_local = num_local;
     hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks > 0 ? blocks : 1), dim3(kThreads), 0, stream, idx,
                        n_routes, num_experts, expert_begin, num_local, padded, nbits, chunk, num_chunks, hist, counts,
-                       psum, offsets, num_rows, route_to_row, row_to_route);
+                       psum, offsets, num_rows, route_to_row, row_to_route, w->mailbox_device, w->sequence);
     return launch_status("layout_assign");
 }
 

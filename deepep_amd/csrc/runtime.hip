@@ -2,6 +2,8 @@
 // SHMEM workspace, csrc/runtime/session.cpp:40-140).
 #include <stdarg.h>
 #include <stdlib.h>
+#include <string.h>
+#include <time.h>
 
 #include "common.h"
 
@@ -44,9 +46,24 @@ int dpep_workspace_create(size_t bytes, void** ws)
         (void)hipFree(base);
         return dpep::fail(DPEP_ERUNTIME, "workspace_create: host allocation failed");
     }
+    void* mailbox = nullptr;
+    void* mailbox_device = nullptr;
+    hipError_t err = hipHostMalloc(&mailbox, dpep::kMailboxWords * sizeof(uint32_t), hipHostMallocMapped);
+    if (err == hipSuccess) err = hipHostGetDevicePointer(&mailbox_device, mailbox, 0);
+    if (err != hipSuccess) {
+        if (mailbox != nullptr) (void)hipHostFree(mailbox);
+        (void)hipFree(base);
+        free(w);
+        return dpep::fail(DPEP_ERUNTIME, "workspace_create: pinned host mailbox: %s", hipGetErrorString(err));
+    }
+    memset(mailbox, 0, dpep::kMailboxWords * sizeof(uint32_t));
     w->magic = dpep::kWorkspaceMagic;
     w->base = base;
     w->bytes = bytes;
+    w->mailbox_host = static_cast<uint32_t*>(mailbox);
+    w->mailbox_device = static_cast<uint32_t*>(mailbox_device);
+    w->sequence = 0;
+    w->mailbox_local = 0;
     *ws = w;
     return DPEP_OK;
 }
@@ -56,9 +73,39 @@ int dpep_workspace_destroy(void* ws)
     dpep::Workspace* w = dpep::as_workspace(ws);
     DPEP_REQUIRE(w != nullptr, "workspace_destroy: not a live workspace");
     hipError_t err = hipFree(w->base);
+    const hipError_t err_host = hipHostFree(w->mailbox_host);
+    if (err == hipSuccess) err = err_host;
     w->magic = 0;
     free(w);
     if (err != hipSuccess) return dpep::fail(DPEP_ERUNTIME, "hipFree failed: %s", hipGetErrorString(err));
+    return DPEP_OK;
+}
+
+int dpep_layout_wait(void* ws, int32_t* counts_host, int num_local, int32_t* num_rows_host, long long timeout_us)
+{
+    dpep::Workspace* w = dpep::as_workspace(ws);
+    DPEP_REQUIRE(w != nullptr, "layout_wait: not a live workspace");
+    DPEP_REQUIRE(w->sequence != 0, "layout_wait: no layout was launched on this workspace");
+    DPEP_REQUIRE(num_rows_host != nullptr, "layout_wait: num_rows_host is NULL");
+    DPEP_REQUIRE(counts_host == nullptr || num_local == w->mailbox_local,
+                 "layout_wait: num_local=%d does not match the launched layout (%d)", num_local, w->mailbox_local);
+    volatile uint32_t* box = w->mailbox_host;
+    timespec start;
+    clock_gettime(CLOCK_MONOTONIC, &start);
+    for (long long spins = 0; box[1] != w->sequence; ++spins) {
+        if ((spins & 1023) == 1023) {
+            timespec now;
+            clock_gettime(CLOCK_MONOTONIC, &now);
+            const long long waited = (now.tv_sec - start.tv_sec) * 1000000ll + (now.tv_nsec - start.tv_nsec) / 1000;
+            if (waited > timeout_us)
+                return dpep::fail(DPEP_ERUNTIME, "layout_wait: the layout kernel did not report within %lld us", timeout_us);
+        }
+        __builtin_ia32_pause();
+    }
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    *num_rows_host = static_cast<int32_t>(box[0]);
+    if (counts_host != nullptr)
+        for (int e = 0; e < num_local; ++e) counts_host[e] = static_cast<int32_t>(box[2 + e]);
     return DPEP_OK;
 }
 

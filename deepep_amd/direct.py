@@ -43,8 +43,9 @@ def expand(
     if expert_alignment != 1:
         raise NotImplementedError("expand supports expert_alignment=1")
     hidden, scales = x if isinstance(x, tuple) else (x, None)
-    plan = ops.layout(_workspace(hidden.device), topk_idx, num_experts)
-    rows = int(plan["num_rows"].item())
+    workspace = _workspace(hidden.device)
+    plan = ops.layout(workspace, topk_idx, num_experts)
+    _, rows = ops.layout_wait(workspace)
     if quantize_fp8:
         if scales is not None:
             raise ValueError("quantize_fp8 expects a BF16 tensor, not an (fp8, scales) pair")

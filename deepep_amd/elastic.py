@@ -541,9 +541,8 @@ class ElasticBuffer:
         with torch.inference_mode(False), torch.no_grad():
             indices = topk_idx.clone() if do_handle_copy else topk_idx
             plan = native.layout(runtime.workspace, indices, num_experts, begin, local)
-            summary = plan["meta"].cpu().tolist()  # counts | psum | offsets | R
-        counts = summary[:local]
-        rows = summary[3 * local + 1]
+            # The single host synchronisation: the kernel reports counts and R through pinned host memory.
+            counts, rows = native.layout_wait(runtime.workspace, local, 100.0)  # num_gpu_timeout_secs
         handle = EPHandle(
             True, num_experts, 1, capacity, 64, indices, None, rows, counts, None, plan["psum"], plan["counts"], None,
             None, None, None,

@@ -102,6 +102,24 @@ def layout(ws: Workspace, topk_idx: torch.Tensor, num_experts: int, expert_begin
                 num_rows=num_rows, meta=meta)
 
 
+def layout_wait(ws: Workspace, num_local: Optional[int] = None, timeout_s: float = 100.0):
+    """The one host synchronisation of a fresh dispatch: waits for the most recent ``layout`` on ``ws`` and
+    returns ``(counts, num_rows)`` as Python ints (``counts`` is None unless ``num_local`` is given).  The layout
+    kernel writes these words into pinned host memory; nothing is copied and no stream is synchronised."""
+    lib = _lib.load()
+    rows = ctypes.c_int32()
+    counts = None
+    buf = None
+    if num_local is not None:
+        buf = (ctypes.c_int32 * num_local)()
+    status = lib.dpep_layout_wait(ws.handle, buf, 0 if num_local is None else num_local, ctypes.byref(rows),
+                                  int(timeout_s * 1e6))
+    _lib.check(status, "layout_wait")
+    if buf is not None:
+        counts = list(buf)
+    return counts, int(rows.value)
+
+
 def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows: int):
     """out[row] = x[token(row)] (+ scale rows, + per-row weights).  x is BF16 [T,H] or FP8 [T,H]."""
     lib = _lib.load()

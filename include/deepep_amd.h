@@ -58,6 +58,17 @@ int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk,
                 int expert_begin, int num_local, int32_t* counts, int32_t* psum, int32_t* offsets,
                 int32_t* route_to_row, int32_t* row_to_route, int32_t* num_rows, void* stream);
 
+/* Host side of the layout's single synchronisation: blocks until the most recent dpep_layout launched on ws has
+ * run, then returns R and (optionally) the rows per local expert.  Replaces the device-to-host read-back that sizes
+ * the outputs of a fresh dispatch (deep_ep/backends/mesh_clos/elastic.py:1476, `.cpu()` of the notify outputs):
+ * the layout kernel writes these few words straight into pinned host memory owned by the workspace and this
+ * call polls them, which costs a few microseconds less than a copy plus a stream wait.
+ *   counts_host   int32 [num_local] host memory, may be NULL; num_local must equal the launched layout's
+ *   num_rows_host int32 [1] host memory
+ *   timeout_us    DPEP_ERUNTIME if the kernel has not reported by then (a layout launch that failed never will)
+ * One layout may be outstanding per workspace; the call does not wait for anything but the layout kernel. */
+int dpep_layout_wait(void* ws, int32_t* counts_host, int num_local, int32_t* num_rows_host, long long timeout_us);
+
 /* Expand-permute payload dispatch: out[row(t,s)] = x[t] for every route with a row.
  * Replaces dispatch() (csrc/ops/dispatch.cpp:82-211 -> dispatch_kernel, csrc/kernels/dispatch/dispatch.cpp:628)
  * and the scatter half of expand() (csrc/direct/kernels/expand/expand.cpp:334-520).

@@ -38,9 +38,14 @@ class FakeNative:
         meta = torch.from_numpy(np.concatenate([out["counts"], out["psum"], out["offsets"], [out["num_rows"]]]).astype(np.int32))
         full = np.zeros(topk_idx.numel(), dtype=np.int32)
         full[: out["num_rows"]] = out["row_to_route"]
+        self.last_layout = ([int(c) for c in out["counts"]], int(out["num_rows"]))
         return dict(counts=meta[:local], psum=meta[local : 2 * local], offsets=meta[2 * local : 3 * local + 1],
                     num_rows=meta[3 * local + 1 :], meta=meta, route_to_row=torch.from_numpy(out["route_to_row"]),
                     row_to_route=torch.from_numpy(full))
+
+    def layout_wait(self, ws, num_local=None, timeout_s=100.0):
+        counts, rows = self.last_layout
+        return (counts if num_local is not None else None), rows
 
     def dispatch_copy(self, x, scales, w, route_to_row, row_to_route, rows):
         if self.fail_next:

@@ -35,6 +35,10 @@ def _check_layout(ops, ws, idx_np, experts, begin=0, local=None):
     idx = torch.from_numpy(np.ascontiguousarray(idx_np, dtype=np.int64)).cuda()
     got = ops.layout(ws, idx, experts, begin, local)
     want = olayout.layout(idx_np, experts, begin, local)
+    # the host mailbox (no copy, no stream wait) must agree with the device tensors
+    host_counts, host_rows = ops.layout_wait(ws, len(want["counts"]))
+    assert host_rows == want["num_rows"] and host_counts == [int(c) for c in want["counts"]]
+    assert ops.layout_wait(ws) == (None, host_rows)  # asking again returns the same launch's result
     rows = int(got["num_rows"].item())
     assert rows == want["num_rows"]
     for key in ("counts", "psum", "offsets", "route_to_row"):
