@@ -390,13 +390,15 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     };
 
     // Copy number c (compile-time) of the item under the copy cursor; the pieces are issued between MFMAs.
+    // (DPEP_ABLATE_COPIES / DPEP_ABLATE_COPY_SOURCE are timing-only builds that drop the copies or aim them
+    // all at one cached kilobyte; their results are wrong by construction.)
     auto issue_copy = [&](int c) {
-#ifdef DPEP_X_NOCOPY
+#ifdef DPEP_ABLATE_COPIES
         return;
 #endif
         const uint32_t stage = lds0 + copy_stage * kStageBytes;
-#ifdef DPEP_X_SAMEADDR
-        copy16_to_lds(p.w + (DPEP_X_SAMEADDR ? lane * 16 : 0), stage + c * 4096 + wave * 1024);
+#ifdef DPEP_ABLATE_COPY_SOURCE
+        copy16_to_lds(p.w + lane * 16, stage + c * 4096 + wave * 1024);  // always the same, cached, kilobyte
         return;
 #endif
         if (c < 2 * RT)
@@ -410,7 +412,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     // fetches the gather indices of the workgroup's next tile.  These extra copies only make the counted
     // waits stricter.
     auto issue_span_copies = [&]() {
-#ifdef DPEP_X_NOCOPY
+#ifdef DPEP_ABLATE_COPIES
         return;
 #endif
         copy_span += (copy_kt & 3) == 0 ? 1 : 0;
@@ -638,11 +640,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             for (int n = 0; n < kMfmas / 2; ++n) mfma_one(0, parity, n);
             // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies in
             // flight; past the barrier every wave has also finished reading the stage refilled next.
-#ifdef DPEP_X_LOOSEWAIT
-            wait_copies_then_barrier<(kAhead - 1) * Cfg::kCopies>();
-#elif !defined(DPEP_X_NOBARRIER)
             wait_copies_then_barrier<(kAhead - 2) * Cfg::kCopies>();
-#endif
             constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
 #pragma unroll
             for (int n = kMfmas / 2; n < kMfmas; ++n) {
