@@ -480,24 +480,28 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     u32x4 bfrag[2][kCT];  // [k step][column tile]
     int ascale[2][RT];    // [item parity][row tile]
     int bscale[2][kCT];
-    auto read_step = [&](int stage_index, int kb) {
+    // Fragment reads of one k step come in kGroups pieces (row tiles first, then column tiles) so that they can
+    // be dealt out between MFMAs; the scale reads of an item likewise.
+    constexpr int kGroups = RT + kCT;
+    auto read_group = [&](int stage_index, int kb, int group) {
         const uint8_t* stage = lds + stage_index * kStageBytes;
-#pragma unroll
-        for (int i = 0; i < RT; ++i) {
+        if (group < RT) {
+            const int i = group;
             const u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][0]);
             const u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][1]);
             afrag[kb][i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+        } else {
+            const int c = group - RT;
+            bfrag[kb][c] = *reinterpret_cast<const u32x4*>(stage + b_addr + (c * 2 + kb) * 1024);
         }
-#pragma unroll
-        for (int c = 0; c < kCT; ++c) bfrag[kb][c] = *reinterpret_cast<const u32x4*>(stage + b_addr + (c * 2 + kb) * 1024);
     };
     // row_at / col_at = byte offsets of the item's scales: ring slot + position inside the span
-    auto read_scales = [&](int slot, int row_at, int col_at) {
-#pragma unroll
-        for (int i = 0; i < RT; ++i) ascale[slot][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + sa_addr[i] + row_at));
-#pragma unroll
-        for (int c = 0; c < kCT; ++c)
-            bscale[slot][c] = static_cast<int>(*reinterpret_cast<const uint16_t*>(lds + sb_addr + c * 512 + col_at));
+    auto read_scale_group = [&](int slot, int row_at, int col_at, int group) {
+        if (group < RT)
+            ascale[slot][group] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + sa_addr[group] + row_at));
+        else
+            bscale[slot][group - RT] =
+                static_cast<int>(*reinterpret_cast<const uint16_t*>(lds + sb_addr + (group - RT) * 512 + col_at));
     };
 
     v16f acc[RT][kCT];
@@ -611,15 +615,21 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     wait_copies_then_barrier<(kAhead - 1) * Cfg::kCopies>();  // item 0 has landed
     // Scale bookkeeping of the item whose fragments are read next: span counter (ring slot) and k tile.
     int read_span = -1, read_kt = 0;
-    auto read_next_scales = [&](int slot) {
+    int row_at = 0, col_at = 0;
+    auto next_scale_offsets = [&]() {
         if ((read_kt & 3) == 0) ++read_span;
         const int window = min((read_kt & ~3) * 4, scale_bytes - 16);
         const int ring = read_span & 1;
-        read_scales(slot, ring * Cfg::kRowScaleSlot + (read_kt * 4 - window), ring * Cfg::kColScaleSlot + (read_kt & 3) * 2);
+        row_at = ring * Cfg::kRowScaleSlot + (read_kt * 4 - window);
+        col_at = ring * Cfg::kColScaleSlot + (read_kt & 3) * 2;
         read_kt = read_kt + 1 == ktiles ? 0 : read_kt + 1;
     };
-    read_step(0, 0);
-    read_next_scales(0);
+    next_scale_offsets();
+#pragma unroll
+    for (int group = 0; group < kGroups; ++group) {
+        read_scale_group(0, row_at, col_at, group);
+        read_group(0, 0, group);
+    }
     clear_acc();
     asm volatile("s_nop 3");
     DPEP_STAMP(3);
@@ -632,25 +642,29 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         for (int parity = 0; parity < 2; ++parity) {  // ktiles is even, so tiles start on even items
             const int stage_next = stage_now + 1 == kStages ? 0 : stage_now + 1;
             // A wave issues in order and owns its SIMD alone, so whatever is not an MFMA should sit in the
-            // shadow of one: after the barrier the copies of the item kAhead ahead and the fragment reads of
-            // the next item are dealt out between the MFMAs.
-            read_step(stage_now, 1);
+            // shadow of one.  First k step: its MFMAs are followed, one piece each, by the LDS reads of the
+            // second k step's fragments and, once the barrier has passed, by the copies of the item kAhead
+            // ahead.  Second k step: the remaining copies and the reads of the next item's scales and first
+            // fragments (whose registers the first k step has released).
             shift_scales(parity);
-#pragma unroll
-            for (int n = 0; n < kMfmas / 2; ++n) mfma_one(0, parity, n);
-            // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies in
-            // flight; past the barrier every wave has also finished reading the stage refilled next.
-            wait_copies_then_barrier<(kAhead - 2) * Cfg::kCopies>();
             constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
+            static_assert(kGroups <= kMfmas, "one fragment read group per MFMA of the first k step");
 #pragma unroll
-            for (int n = kMfmas / 2; n < kMfmas; ++n) {
+            for (int n = 0; n < kMfmas; ++n) {
                 mfma_one(0, parity, n);
-                const int slot = n - kMfmas / 2;
+                if (n < kGroups) read_group(stage_now, 1, n);
+                if (n == kMfmas / 2 - 1) {
+                    // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies
+                    // in flight; past the barrier every wave has also finished reading the stage refilled next.
+                    wait_copies_then_barrier<(kAhead - 2) * Cfg::kCopies>();
+                }
+                if (n >= kMfmas / 2) {
+                    const int slot = n - kMfmas / 2;
 #pragma unroll
-                for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
+                    for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
+                }
             }
-            read_step(stage_next, 0);
-            read_next_scales(parity ^ 1);
+            next_scale_offsets();
 #pragma unroll
             for (int n = 0; n < kMfmas; ++n) {
                 mfma_one(1, parity, n);
@@ -658,6 +672,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                 if (slot < kSlots) {
 #pragma unroll
                     for (int c = slot * Cfg::kCopies / kSlots; c < (slot + 1) * Cfg::kCopies / kSlots; ++c) issue_copy(c);
+                }
+                // 2*kGroups read pieces for the next item: its scales first (they are shifted first), then fragments
+#pragma unroll
+                for (int piece = n * 2 * kGroups / kMfmas; piece < (n + 1) * 2 * kGroups / kMfmas; ++piece) {
+                    if (piece < kGroups) read_scale_group(parity ^ 1, row_at, col_at, piece);
+                    else read_group(stage_next, 0, piece - kGroups);
                 }
             }
             issue_span_copies();
