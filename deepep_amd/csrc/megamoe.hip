@@ -164,7 +164,9 @@ template <int RT, bool kGather>
 struct GemmCfg {
     static constexpr int kBM = 64 * RT;
     static constexpr int kStages = RT == 2 ? 4 : 3;
-    static constexpr int kAhead = kStages - 1;
+    // Copies run a full ring ahead: a stage is refilled in the very item that consumes it, right after the
+    // barrier that follows the last LDS read of it.
+    static constexpr int kAhead = kStages;
     static constexpr int kOffA = 0;                    // kBM rows x 128 B, 16-byte chunks XOR-swizzled
     static constexpr int kOffB = kBM * kBK;            // 8 column tiles x 2 k steps x 1 KiB fragments
     static constexpr int kStageBytes = kOffB + 16384;
@@ -248,10 +250,11 @@ __device__ __forceinline__ void copy4_to_lds_unless(const void* src, uint32_t ld
         "v"(src), "s"(flag)
         : "memory", "scc");
 }
+// Also waits for the wave's own LDS reads: past the barrier nothing reads the stage that is refilled next.
 template <int kOutstanding>
 __device__ __forceinline__ void wait_copies_then_barrier()
 {
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
 // One scaled MFMA (FP8 A, FP4 B) as a volatile asm statement: volatile statements keep their source order,
@@ -648,11 +651,13 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             // fragments (whose registers the first k step has released).
             shift_scales(parity);
             constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
-            static_assert(kGroups <= kMfmas, "one fragment read group per MFMA of the first k step");
+            static_assert((kGroups + 1) / 2 < kMfmas / 2, "the second k step's fragments leave LDS before the barrier");
 #pragma unroll
             for (int n = 0; n < kMfmas; ++n) {
                 mfma_one(0, parity, n);
-                if (n < kGroups) read_group(stage_now, 1, n);
+#pragma unroll
+                for (int group = 2 * n; group < 2 * n + 2; ++group)
+                    if (group < kGroups) read_group(stage_now, 1, group);
                 if (n == kMfmas / 2 - 1) {
                     // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies
                     // in flight; past the barrier every wave has also finished reading the stage refilled next.
