@@ -21,8 +21,32 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device) -> ctypes.c_void_p:
+    """torch's current stream on ``device`` as a raw hipStream_t."""
+    if _raw_stream is not None and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+class _on_device:
+    """``torch.cuda.device(dev)`` that costs nothing when ``dev`` is already current (the usual case)."""
+
+    __slots__ = ("guard",)
+
+    def __init__(self, device):
+        self.guard = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
 
 
 def _require(name, t, dtype, shape=None, device=None):
@@ -92,7 +116,7 @@ def layout(ws: Workspace, topk_idx: torch.Tensor, num_experts: int, expert_begin
     offsets, num_rows = meta[2 * num_local : 3 * num_local + 1], meta[3 * num_local + 1 :]
     route_to_row = torch.empty((tokens, topk), dtype=torch.int32, device=dev)
     row_to_route = torch.empty((tokens * topk,), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         status = lib.dpep_layout(
             ws.handle, _ptr(topk_idx), tokens, topk, num_experts, expert_begin, num_local, _ptr(counts), _ptr(psum),
             _ptr(offsets), _ptr(route_to_row), _ptr(row_to_route), _ptr(num_rows), _stream(dev),
@@ -150,7 +174,7 @@ def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows:
         _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)
         out_weights = torch.empty((num_rows,), dtype=torch.float32, device=dev)
     out = torch.empty((num_rows, hidden), dtype=x.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         status = lib.dpep_dispatch_copy(
             _ptr(x), _ptr(scales), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, num_rows,
             row_bytes, scale_cols, _ptr(out), _ptr(out_scales), _ptr(out_weights), _stream(dev),
@@ -179,7 +203,7 @@ def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: in
         out_weights = torch.empty((num_rows,), dtype=torch.float32, device=dev)
     out = torch.empty((num_rows, hidden), dtype=torch.float8_e4m3fn, device=dev)
     out_scales = torch.empty((num_rows, hidden // 128), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         status = lib.dpep_dispatch_quant_fp8(
             _ptr(x), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, num_rows, hidden,
             _ptr(out), _ptr(out_scales), _ptr(out_weights), _stream(dev),
@@ -197,7 +221,7 @@ def cast_to_fp8(x):
     tokens, hidden = x.shape
     out = torch.empty((tokens, hidden), dtype=torch.float8_e4m3fn, device=x.device)
     scales = torch.empty((tokens, hidden // 128), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         status = lib.dpep_cast_to_fp8(_ptr(x), tokens, hidden, _ptr(out), _ptr(scales), _stream(x.device))
     _lib.check(status, "cast_to_fp8")
     return out, scales
@@ -227,7 +251,7 @@ def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
         out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
     else:
         _require("out", out, torch.bfloat16, (tokens, hidden), dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         status = lib.dpep_combine(
             _ptr(y), _ptr(row_weights), _ptr(route_to_row), tokens, topk, rows, hidden, _ptr(out),
             _ptr(return_values), _ptr(returned), _stream(dev),
@@ -248,7 +272,7 @@ def mx_quant(x):
     rows, hidden = x.shape
     codes = torch.empty((rows, hidden), dtype=torch.float8_e4m3fn, device=x.device)
     scales = torch.empty((rows, hidden // 32), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         status = lib.dpep_mx_quant(_ptr(x), rows, hidden, _ptr(codes), _ptr(scales), _stream(x.device))
     _lib.check(status, "mx_quant")
     return codes, scales
@@ -278,7 +302,7 @@ def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
     out_s = torch.empty((experts, n, megamoe_prepared_scale_cols(k)), dtype=torch.uint8, device=w_packed.device)
     if out_s.numel() != lib.dpep_megamoe_prepared_scale_bytes(experts, n, k):
         raise RuntimeError("prepared scale size disagrees with the library")
-    with torch.cuda.device(w_packed.device):
+    with _on_device(w_packed.device):
         status = lib.dpep_megamoe_prepare_weights(
             _ptr(w_packed), _ptr(w_scales), experts, n, k, int(bool(gate_up)), _ptr(out_w), _ptr(out_s),
             _stream(w_packed.device),
@@ -308,7 +332,7 @@ def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s
     _require("s2", s2, torch.uint8, (num_local, hidden, megamoe_prepared_scale_cols(intermediate)), dev)
     _require("y", y, torch.bfloat16, (tokens, hidden), dev)
     _require("expert_token_nums", expert_token_nums, torch.int32, (num_local,), dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         status = lib.dpep_megamoe_forward(
             ws.handle, _ptr(x_codes), _ptr(x_scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(w1), _ptr(s1), _ptr(w2),
             _ptr(s2), tokens, hidden, intermediate, topk, num_experts, expert_begin, num_local, _ptr(y),
