@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
             for (int w = 0; w < kWaves; ++w) running[w][e] += offset;
             if (blockIdx.x == 0) {
                 counts[e] = mine[j];
-                mailbox[2 + e] = static_cast<uint32_t>(mine[j]);  // pinned host memory
+                if (mailbox != nullptr) mailbox[2 + e] = static_cast<uint32_t>(mine[j]);  // pinned host memory
                 psum[e] = offset + mine[j];
                 offsets[e + 1] = offset + mine[j];
             }
@@ -204,9 +204,9 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
     }
     // The host polls the mailbox's sequence word: publish it (with the row count, one 8-byte store) after
     // every per-expert count of this workgroup has reached host memory.
-    if (blockIdx.x == 0) __threadfence_system();
+    if (blockIdx.x == 0 && mailbox != nullptr) __threadfence_system();
     __syncthreads();
-    if (blockIdx.x == 0 && tid == kThreads - 1) {
+    if (blockIdx.x == 0 && mailbox != nullptr && tid == kThreads - 1) {
         const unsigned long long word = (static_cast<unsigned long long>(sequence) << 32) | static_cast<uint32_t>(offset);
         __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), word, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
@@ -260,7 +260,7 @@ int chunk_routes(int n_routes, int padded_local)
 template <typename IdxT>
 int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int num_experts, int expert_begin,
                   int num_local, int32_t* counts, int32_t* psum, int32_t* offsets, int32_t* route_to_row,
-                  int32_t* row_to_route, int32_t* num_rows, hipStream_t stream)
+                  int32_t* row_to_route, int32_t* num_rows, bool report_to_host, hipStream_t stream)
 {
     Workspace* w = as_workspace(ws);
     DPEP_REQUIRE(w != nullptr, "layout: not a live workspace");
@@ -289,11 +289,14 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
         if (int rc = launch_status("layout_count")) return rc;
     }
     // With no routes one workgroup still publishes the all-zero counts and prefix sums.
-    w->sequence = w->sequence == 0xffffffffu ? 1u : w->sequence + 1u;  // never 0: that is "nothing launched"
-    w->mailbox_local = num_local;
+    if (report_to_host) {
+        w->sequence = w->sequence == 0xffffffffu ? 1u : w->sequence + 1u;  // never 0: that is "nothing launched"
+        w->mailbox_local = num_local;
+    }
     hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks > 0 ? blocks : 1), dim3(kThreads), 0, stream, idx,
                        n_routes, num_experts, expert_begin, num_local, padded, nbits, chunk, num_chunks, hist, counts,
-                       psum, offsets, num_rows, route_to_row, row_to_route, w->mailbox_device, w->sequence);
+                       psum, offsets, num_rows, route_to_row, row_to_route, report_to_host ? w->mailbox_device : nullptr,
+                       w->sequence);
     return launch_status("layout_assign");
 }
 
@@ -305,7 +308,7 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
                int32_t* row_to_route, int32_t* num_rows, hipStream_t stream)
 {
     return launch_layout<int32_t>(ws, idx, num_tokens, num_topk, num_experts, expert_begin, num_local, counts, psum,
-                                  offsets, route_to_row, row_to_route, num_rows, stream);
+                                  offsets, route_to_row, row_to_route, num_rows, /*report_to_host=*/false, stream);
 }
 
 }  // namespace dpep
@@ -324,7 +327,7 @@ int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk,
 {
     return dpep::launch_layout<int64_t>(ws, topk_idx, num_tokens, num_topk, num_experts, expert_begin, num_local,
                                         counts, psum, offsets, route_to_row, row_to_route, num_rows,
-                                        static_cast<hipStream_t>(stream));
+                                        /*report_to_host=*/true, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

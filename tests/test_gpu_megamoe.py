@@ -169,3 +169,58 @@ def test_public_api_workflow():
         buf.destroy()
     with pytest.raises(RuntimeError, match="destroyed"):
         megamoe.fp8_fp4_mega_moe(y, p1, p2, buf)
+
+
+def test_megamoe_forward_in_hip_graph(ops):
+    # The forward is five launches and no host synchronisation, so it can be captured once and replayed
+    # with new inputs in the same buffers; every replay is checked against the eager result.
+    tokens, hidden, inter, experts, local, topk = 192, 512, 512, 8, 8, 2
+    dev = "cuda"
+    problems = [_make_problem(tokens, hidden, inter, experts, 0, local, topk, seed=s) for s in (11, 12, 13)]
+    _, _, l1, l2, _, _ = problems[0]
+    w1, s1 = ops.megamoe_prepare_weights(torch.from_numpy(l1[0]).to(dev), torch.from_numpy(l1[1]).reshape(local, 2 * inter, -1).to(dev), True)
+    w2, s2 = ops.megamoe_prepare_weights(torch.from_numpy(l2[0]).to(dev), torch.from_numpy(l2[1]).reshape(local, hidden, -1).to(dev), False)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local))
+    x_codes = torch.empty((tokens, hidden), dtype=torch.uint8, device=dev)
+    x_scales = torch.empty((tokens, hidden // 32), dtype=torch.uint8, device=dev)
+    idx = torch.empty((tokens, topk), dtype=torch.int32, device=dev)
+    weights = torch.empty((tokens, topk), dtype=torch.float32, device=dev)
+    y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+
+    def load(problem):
+        codes, scales, _, _, ids, wts = problem
+        x_codes.copy_(torch.from_numpy(codes)); x_scales.copy_(torch.from_numpy(scales))
+        idx.copy_(torch.from_numpy(ids)); weights.copy_(torch.from_numpy(wts))
+
+    def forward():
+        ops.megamoe_forward(ws, x_codes.view(torch.float8_e4m3fn), x_scales, idx, weights, w1, s1, w2, s2, experts, 0, local, y, counts)
+
+    try:
+        eager = []
+        for problem in problems:
+            load(problem)
+            forward()
+            torch.cuda.synchronize()
+            eager.append((y.clone(), counts.clone()))
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            forward()  # warm-up on the capture stream
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            forward()
+        for turn in range(2):
+            for problem, (want_y, want_counts) in zip(problems, eager):
+                load(problem)
+                y.zero_()
+                torch.cuda.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(counts, want_counts)
+                assert torch.equal(y.view(torch.int16), want_y.view(torch.int16)), f"replay {turn} differs from eager"
+    finally:
+        torch.cuda.synchronize()
+        ws.destroy()
