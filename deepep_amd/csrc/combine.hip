@@ -28,7 +28,8 @@ template <int kWeights>
 __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ row_weights, const int* __restrict__ route_to_row,
     int num_topk, int vec_per_row, int vec_per_part, int parts, u32x4* __restrict__ out,
-    const float* __restrict__ return_in, float* __restrict__ return_out)
+    const float* __restrict__ return_in, float* __restrict__ return_out, const int* __restrict__ shared_first_row,
+    int num_shared, int num_tokens)
 {
     __shared__ int rows[DPEP_MAX_TOPK + kBatch];
     __shared__ float wts[DPEP_MAX_TOPK + kBatch];
@@ -42,10 +43,16 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
             wts[threadIdx.x] = row >= 0 ? row_weights[static_cast<size_t>(token) * num_topk + threadIdx.x] : 0.0f;
         if (part == 0 && return_out != nullptr && threadIdx.x < num_topk)
             return_out[static_cast<size_t>(token) * num_topk + threadIdx.x] = row >= 0 ? return_in[row] : 0.0f;
+        // Shared experts (MegaMoE): slot K + j is row first + j * B + token with weight 1, summed after the routes.
+        if (kWeights == 2 && threadIdx.x >= num_topk && threadIdx.x < num_topk + num_shared) {
+            rows[threadIdx.x] = shared_first_row[0] + (threadIdx.x - num_topk) * num_tokens + token;
+            wts[threadIdx.x] = 1.0f;
+        }
     }
+    const int num_slots = num_topk + (kWeights == 2 ? num_shared : 0);
     // Tokens without any row (the common case of a sparse receive share) are plain zero fill.  Streaming
     // stores: cached ones would push the rows read next, and the caller's other data, out of the caches.
-    const bool any_row = __syncthreads_or(threadIdx.x < num_topk && rows[threadIdx.x] >= 0) != 0;
+    const bool any_row = __syncthreads_or(threadIdx.x < num_slots && rows[threadIdx.x] >= 0) != 0;
     const int v_begin = part * vec_per_part;
     const int v_end = min(v_begin + vec_per_part, vec_per_row);
     if (!any_row) {
@@ -58,7 +65,7 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-        for (int s0 = 0; s0 < num_topk; s0 += kBatch) {
+        for (int s0 = 0; s0 < num_slots; s0 += kBatch) {
             u32x4 val[kBatch];
 #pragma unroll
             for (int j = 0; j < kBatch; ++j) {
@@ -116,22 +123,25 @@ CombineGrid combine_grid(int num_tokens, int num_rows, int vec)
 
 template <int kWeights>
 void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, const float* weights, const int32_t* route_to_row,
-                    int num_topk, int vec, void* out, const float* return_in, float* return_out)
+                    int num_topk, int vec, void* out, const float* return_in, float* return_out,
+                    const int32_t* shared_first_row = nullptr, int num_shared = 0, int num_tokens = 0)
 {
     hipLaunchKernelGGL(combine_kernel<kWeights>, dim3(g.blocks), dim3(g.threads), 0, stream, static_cast<const u32x4*>(y),
                        weights, route_to_row, num_topk, vec, g.per_part, g.parts, static_cast<u32x4*>(out), return_in,
-                       return_out);
+                       return_out, shared_first_row, num_shared, num_tokens);
 }
 
 }  // namespace
 
 // Route-weighted reduce used by the MegaMoE forward: out[t] = bf16( sum_s w[t,s] * float(y[row(t,s)]) ).
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
-                   int num_rows_hint, int hidden, void* out, hipStream_t stream)
+                   int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
+                   hipStream_t stream)
 {
     const int vec = hidden / 8;
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
-    launch_combine<2>(g, stream, y, route_weights, route_to_row, num_topk, vec, out, nullptr, nullptr);
+    launch_combine<2>(g, stream, y, route_weights, route_to_row, num_topk, vec, out, nullptr, nullptr, shared_first_row,
+                      num_shared, num_tokens);
     return launch_status("combine_routes");
 }
 

@@ -21,7 +21,8 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
                int num_local, int32_t* counts, int32_t* psum, int32_t* offsets, int32_t* route_to_row,
                int32_t* row_to_route, int32_t* num_rows, hipStream_t stream);
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
-                   int num_rows_hint, int hidden, void* out, hipStream_t stream);
+                   int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
+                   hipStream_t stream);
 
 namespace {
 
@@ -193,6 +194,9 @@ struct GemmParams {
     int num_local;
     const uint8_t* w;          // prepared fragments, expert stride N*K/2
     const uint8_t* ws;         // prepared scales, expert stride N*K/32
+    int num_routed;            // experts >= num_routed are shared experts with weights of their own:
+    const uint8_t* w_shared;   //   expert e reads w_shared / ws_shared at index e - num_routed
+    const uint8_t* ws_shared;
     int n, k;
     uint8_t* act_codes;        // first GEMM: [rows, N/2] e4m3
     uint8_t* act_scales;       //             [rows, N/64] e8m0
@@ -378,7 +382,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             const int src = kGather ? index[r] / p.topk : info.row0 + r;
             sa_src = p.a_scales + static_cast<size_t>(src) * scale_bytes;
         }
-        b_base = p.w + static_cast<size_t>(info.expert) * p.n * (p.k / 2) +
+        const bool shared = info.expert >= p.num_routed;
+        const size_t weight_index = shared ? info.expert - p.num_routed : info.expert;
+        b_base = (shared ? p.w_shared : p.w) + weight_index * p.n * (p.k / 2) +
                  static_cast<size_t>(info.nt) * (2 * kCT) * ksteps * 1024;
         // fragment q = copy*4 + wave of the 16 (column tile, k step) fragments of one k tile
 #pragma unroll
@@ -386,7 +392,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             const int q = j * 4 + wave;
             b_off[j] = static_cast<uint32_t>(((q >> 1) * ksteps + (q & 1)) * 1024 + lane * 16);
         }
-        sb_src = p.ws + (static_cast<size_t>(info.expert) * n_tiles + info.nt) * spans * Cfg::kColScaleSlot + tid * 16;
+        sb_src = (shared ? p.ws_shared : p.ws) + (weight_index * n_tiles + info.nt) * spans * Cfg::kColScaleSlot + tid * 16;
     };
     auto aim_index_prefetch = [&](const TileInfo& info) {
         if (kGather) index_src = p.row_to_route + info.row0 + min(tid, info.valid - 1);
@@ -707,6 +713,20 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     DPEP_STAMP(6);
 }
 
+// Shared experts take every token: their rows follow the routed ones, expert-major, token order.
+// offsets[num_routed + 1 + s] = R + (s + 1) * B and row_to_route[R + s * B + t] = t * topk (so that the gather's
+// route / topk is t), with R read from the device.
+__global__ __launch_bounds__(256) void shared_rows_kernel(const int* __restrict__ num_rows, int num_tokens, int num_topk,
+                                                          int num_routed, int num_shared, int* __restrict__ offsets,
+                                                          int* __restrict__ row_to_route)
+{
+    const int first = num_rows[0];
+    const long long id = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id < num_shared) offsets[num_routed + 1 + id] = first + static_cast<int>(id + 1) * num_tokens;
+    if (id < static_cast<long long>(num_shared) * num_tokens)
+        row_to_route[first + id] = static_cast<int>(id % num_tokens) * num_topk;
+}
+
 int check_gemm(const char* what, int n, int k, int num_local)
 {
     DPEP_REQUIRE(num_local >= 1 && num_local <= kMaxMoeExperts, "%s: number of local experts %d outside [1, %d]", what,
@@ -838,17 +858,18 @@ struct MegaLayout {
     size_t hist, meta, route_to_row, row_to_route, act_codes, act_scales, out2, total;
 };
 
-static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int intermediate, int num_local)
+static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int intermediate, int num_local, int num_shared)
 {
     auto up = [](size_t v) { return (v + 255) / 256 * 256; };
     const size_t routes = static_cast<size_t>(num_tokens) * num_topk;
-    const size_t max_rows = static_cast<size_t>(num_tokens) * (num_topk < num_local ? num_topk : num_local);
+    const size_t shared_rows = static_cast<size_t>(num_tokens) * num_shared;
+    const size_t max_rows = static_cast<size_t>(num_tokens) * (num_topk < num_local ? num_topk : num_local) + shared_rows;
     MegaLayout l;
     size_t at = 0;
     l.hist = at;         at += up(dpep_layout_workspace_bytes(num_tokens, num_topk, num_local));
-    l.meta = at;         at += up((3 * static_cast<size_t>(num_local) + 2) * 4);
+    l.meta = at;         at += up((3 * static_cast<size_t>(num_local) + num_shared + 2) * 4);
     l.route_to_row = at; at += up(routes * 4);
-    l.row_to_route = at; at += up(routes * 4);
+    l.row_to_route = at; at += up((routes + shared_rows) * 4);
     l.act_codes = at;    at += up(max_rows * intermediate);
     l.act_scales = at;   at += up(max_rows * (intermediate / 32));
     l.out2 = at;         at += up(max_rows * hidden * 2);
@@ -856,17 +877,19 @@ static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int inte
     return l;
 }
 
-size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, int intermediate, int num_local)
+size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, int intermediate, int num_local,
+                                    int num_shared)
 {
-    if (num_tokens < 1 || num_topk < 1 || hidden < 1 || intermediate < 1 || num_local < 1) return 0;
-    return mega_layout(num_tokens, num_topk, hidden, intermediate, num_local).total;
+    if (num_tokens < 1 || num_topk < 1 || hidden < 1 || intermediate < 1 || num_local < 1 || num_shared < 0) return 0;
+    return mega_layout(num_tokens, num_topk, hidden, intermediate, num_local, num_shared).total;
 }
 
 int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales, const int32_t* topk_idx,
                          const float* topk_weights, const uint8_t* w1, const uint8_t* s1, const uint8_t* w2,
-                         const uint8_t* s2, int num_tokens, int hidden, int intermediate, int num_topk,
-                         int num_experts, int expert_begin, int num_local, void* y, int32_t* expert_token_nums,
-                         void* stream)
+                         const uint8_t* s2, const uint8_t* shared_w1, const uint8_t* shared_s1,
+                         const uint8_t* shared_w2, const uint8_t* shared_s2, int num_shared, int num_tokens, int hidden,
+                         int intermediate, int num_topk, int num_experts, int expert_begin, int num_local, void* y,
+                         int32_t* expert_token_nums, void* stream)
 {
     using namespace dpep;
     Workspace* w = as_workspace(ws);
@@ -876,45 +899,63 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     DPEP_REQUIRE(hidden % 256 == 0 && intermediate % 256 == 0 && hidden >= 512 && intermediate >= 512,
                  "megamoe_forward: hidden=%d and intermediate=%d must be multiples of 256, at least 512", hidden,
                  intermediate);
-    DPEP_REQUIRE(num_local >= 1 && num_local <= 128 && expert_begin >= 0 &&
-                     expert_begin + num_local <= num_experts,
+    DPEP_REQUIRE(num_local >= 1 && expert_begin >= 0 && expert_begin + num_local <= num_experts,
                  "megamoe_forward: bad expert range E=%d begin=%d L=%d", num_experts, expert_begin, num_local);
+    DPEP_REQUIRE(num_shared >= 0 && num_shared <= 8 && num_topk + num_shared <= DPEP_MAX_TOPK &&
+                     num_local + num_shared <= kMaxMoeExperts,
+                 "megamoe_forward: %d shared experts with K=%d, L=%d (at most 8, K+S <= %d, L+S <= %d)", num_shared,
+                 num_topk, num_local, DPEP_MAX_TOPK, kMaxMoeExperts);
     DPEP_REQUIRE(x_codes && x_scales && topk_idx && topk_weights && w1 && s1 && w2 && s2 && y && expert_token_nums,
                  "megamoe_forward: NULL buffer");
-    DPEP_REQUIRE(aligned16(x_codes) && aligned16(w1) && aligned16(w2) && aligned16(y), "megamoe_forward: misaligned buffer");
+    DPEP_REQUIRE(num_shared == 0 || (shared_w1 && shared_s1 && shared_w2 && shared_s2 && aligned16(shared_w1) &&
+                                     aligned16(shared_w2) && aligned16(shared_s1) && aligned16(shared_s2)),
+                 "megamoe_forward: shared experts need their four prepared weight buffers, 16-byte aligned");
+    DPEP_REQUIRE(aligned16(x_codes) && aligned16(w1) && aligned16(w2) && aligned16(s1) && aligned16(s2) && aligned16(y),
+                 "megamoe_forward: misaligned buffer");
     // the GEMM's copies address activation rows with 32-bit byte offsets
-    DPEP_REQUIRE(static_cast<long long>(num_tokens) * hidden < (1LL << 32) &&
-                     static_cast<long long>(num_tokens) * (num_topk < num_local ? num_topk : num_local) * intermediate < (1LL << 32),
+    const long long max_rows = static_cast<long long>(num_tokens) * ((num_topk < num_local ? num_topk : num_local) + num_shared);
+    DPEP_REQUIRE(static_cast<long long>(num_tokens) * hidden < (1LL << 32) && max_rows * intermediate < (1LL << 32),
                  "megamoe_forward: activation tensors of B=%d tokens exceed 4 GiB", num_tokens);
-    const MegaLayout l = mega_layout(num_tokens, num_topk, hidden, intermediate, num_local);
+    const MegaLayout l = mega_layout(num_tokens, num_topk, hidden, intermediate, num_local, num_shared);
     DPEP_REQUIRE(l.total <= w->bytes, "megamoe_forward: workspace too small (%zu needed, %zu available)", l.total, w->bytes);
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint8_t* base = static_cast<uint8_t*>(w->base);
     int32_t* meta = reinterpret_cast<int32_t*>(base + l.meta);
     int32_t* psum = meta;
-    int32_t* offsets = meta + num_local;
-    int32_t* num_rows = meta + 2 * num_local + 1;
+    int32_t* offsets = meta + num_local;                          // [L + S + 1]
+    int32_t* num_rows = meta + 2 * num_local + num_shared + 1;    // rows of the routed experts
     int32_t* route_to_row = reinterpret_cast<int32_t*>(base + l.route_to_row);
     int32_t* row_to_route = reinterpret_cast<int32_t*>(base + l.row_to_route);
     if (int rc = layout_i32(ws, topk_idx, num_tokens, num_topk, num_experts, expert_begin, num_local, expert_token_nums,
                             psum, offsets, route_to_row, row_to_route, num_rows, s))
         return rc;
+    if (num_shared > 0) {
+        const long long shared_rows = static_cast<long long>(num_tokens) * num_shared;
+        hipLaunchKernelGGL(shared_rows_kernel, dim3(static_cast<unsigned>((shared_rows + 255) / 256)), dim3(256), 0, s,
+                           num_rows, num_tokens, num_topk, num_local, num_shared, offsets, row_to_route);
+        if (int rc = launch_status("shared_rows")) return rc;
+    }
     GemmParams g1{};
     g1.a_codes = static_cast<const uint8_t*>(x_codes);
     g1.a_scales = x_scales;
     g1.row_to_route = row_to_route;
     g1.topk = num_topk;
     g1.offsets = offsets;
-    g1.num_local = num_local;
+    g1.num_local = num_local + num_shared;
+    g1.num_routed = num_local;
     g1.w = w1;
     g1.ws = s1;
+    g1.w_shared = shared_w1;
+    g1.ws_shared = shared_s1;
     g1.n = 2 * intermediate;
     g1.k = hidden;
     g1.act_codes = base + l.act_codes;
     g1.act_scales = base + l.act_scales;
-    // Expected rows (the true counts stay on the device): tokens * topk / experts per expert.
-    const long long expected_rows = static_cast<long long>(num_tokens) * num_topk * num_local / num_experts;
-    const int per_expert = static_cast<int>((expected_rows + num_local - 1) / num_local);
+    // Expected rows (the true counts stay on the device): tokens * topk / experts per routed expert, every
+    // token for a shared one.
+    const long long expected_routed = static_cast<long long>(num_tokens) * num_topk * num_local / num_experts;
+    const long long expected_rows = expected_routed + static_cast<long long>(num_tokens) * num_shared;
+    const int per_expert = static_cast<int>((expected_rows + g1.num_local - 1) / g1.num_local);
     if (int rc = launch_gemm1(g1, per_expert, s)) return rc;
     GemmParams g2{};
     g2.a_codes = base + l.act_codes;
@@ -922,15 +963,19 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g2.row_to_route = nullptr;
     g2.topk = 1;
     g2.offsets = offsets;
-    g2.num_local = num_local;
+    g2.num_local = num_local + num_shared;
+    g2.num_routed = num_local;
     g2.w = w2;
     g2.ws = s2;
+    g2.w_shared = shared_w2;
+    g2.ws_shared = shared_s2;
     g2.n = hidden;
     g2.k = intermediate;
     g2.out = reinterpret_cast<uint16_t*>(base + l.out2);
     if (int rc = launch_gemm2(g2, per_expert, s)) return rc;
     return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,
-                          static_cast<int>(expected_rows), hidden, y, s);
+                          static_cast<int>(expected_rows),
+                          hidden, y, num_shared > 0 ? num_rows : nullptr, num_shared, s);
 }
 
 }  // extern "C"

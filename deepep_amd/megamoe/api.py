@@ -8,8 +8,9 @@ transform_weights_for_mega_moe :311-379, mega_moe :382-413, fp8_fp4_mega_moe :52
     ``num_experts / world_size`` experts and its inputs hold the flattened tokens of all source ranks
     (capacity ``world_size * num_max_tokens_per_rank`` rows).  The reference needs 2..128 real ranks;
   * prepared weights are this library's fragment order (``dpep_megamoe_prepare_weights``), not Ascend NZ;
-  * shared experts and FP8xFP8 weights are not built; hidden and intermediate_hidden must be multiples
-    of 256 with intermediate_hidden >= 512 (the reference: multiples of 64 and 128, from 256).
+  * FP8xFP8 weights are not built; hidden and intermediate_hidden must be multiples of 256 with
+    intermediate_hidden >= 512 (the reference: multiples of 64 and 128, from 256);
+  * shared experts run as extra experts that take every token (weight 1, added after the routed ones).
 """
 
 from __future__ import annotations
@@ -105,8 +106,8 @@ class SymmBuffer:
             raise ValueError("Only SwiGLU with FP8xFP4/FP8xFP8 is implemented; no BF16xBF16")
         if mma_type != "fp8xfp4":
             raise NotImplementedError("This build implements FP8xFP4 (W4A8) weights only")
-        if num_shared_experts:
-            raise NotImplementedError("Shared experts are not built yet")
+        if num_topk + num_shared_experts > 32:
+            raise ValueError("num_topk + num_shared_experts must not exceed 32 in this build")
         if num_experts % size or num_experts // size > 128:
             raise ValueError("Experts must divide EP, with at most 128 local experts")
         if ranks_per_node and size % ranks_per_node:
@@ -152,7 +153,8 @@ class SymmBuffer:
         if self._workspace is not None:
             self._workspace.destroy()
             self._workspace = None
-        need = ops.megamoe_workspace_bytes(bs, self.num_topk, self.hidden, self.intermediate_hidden, self.num_local_experts)
+        need = ops.megamoe_workspace_bytes(bs, self.num_topk, self.hidden, self.intermediate_hidden, self.num_local_experts,
+                                           self.num_shared_experts)
         self._workspace = ops.Workspace(need, self._device)
         self._plan_bs = bs
 
@@ -221,8 +223,7 @@ def transform_weights_for_mega_moe(l1_weights, l2_weights, activation: str = "sw
     """
     if activation != "swiglu":
         raise NotImplementedError("Only SwiGLU is supported")
-    if shared:
-        raise NotImplementedError("Shared experts are not built yet")
+    # shared=True: the weights of shared experts; this build lays them out exactly like routed ones.
     prepared = []
     for name, value, gate_up in (("l1_weights", l1_weights, True), ("l2_weights", l2_weights, False)):
         weight, scale = _pair(value, name)
@@ -267,8 +268,8 @@ def _run(x, topk_idx, topk_weights, l1_weights, l2_weights, sym_buffer, *, share
     if not isinstance(sym_buffer, SymmBuffer):
         raise TypeError("sym_buffer must be this installation's MegaMoE SymmBuffer")
     data, scales = _pair(x, "x") if isinstance(x, tuple) else (x, None)
-    if shared_l1_weights is not None or shared_l2_weights is not None:
-        raise NotImplementedError("Shared experts are not built yet")
+    if (shared_l1_weights is None) != (shared_l2_weights is None):
+        raise ValueError("Supply both shared weight pairs, or neither")
     if timer is not None:
         raise RuntimeError("W4A8 timer requires DEEPEP_MEGAMOE_TIMER=ON (device timers are not built; use rocprofv3)")
     b = sym_buffer
@@ -282,6 +283,15 @@ def _run(x, topk_idx, topk_weights, l1_weights, l2_weights, sym_buffer, *, share
         raise ValueError("l1_weights / l2_weights are swapped")
     w1, s1 = l1_weights.checked()
     w2, s2 = l2_weights.checked()
+    shared = None
+    if shared_l1_weights is not None:
+        if not isinstance(shared_l1_weights, _PreparedPair) or not isinstance(shared_l2_weights, _PreparedPair):
+            raise ValueError("Shared weights must come from transform_weights_for_mega_moe(..., shared=True)")
+        if not shared_l1_weights.gate_up or shared_l2_weights.gate_up:
+            raise ValueError("shared_l1_weights / shared_l2_weights are swapped")
+        shared = (*shared_l1_weights.checked(), *shared_l2_weights.checked())
+    if (shared[0].shape[0] if shared is not None else 0) != sym_buffer.num_shared_experts:
+        raise ValueError("Shared expert count does not match the buffer configuration")
     if data.ndim != 2 or not 0 < data.shape[0] <= b.capacity_tokens or data.shape[1] != b.hidden:
         raise ValueError("x must be nonempty [BS,H] within the buffer capacity")
     if data.device != b._device:
@@ -295,7 +305,7 @@ def _run(x, topk_idx, topk_weights, l1_weights, l2_weights, sym_buffer, *, share
         raise TypeError("x must be BF16, or an (FP8 E4M3, E8M0) pair")
     if scales is not None and (data.dtype != torch.float8_e4m3fn or scales.dtype not in (torch.float8_e8m0fnu, torch.uint8)):
         raise TypeError("x pair must be (FP8 E4M3 [BS,H], E8M0 [BS,H/32])")
-    tensors = [t for t in (data, scales, topk_idx, topk_weights, w1, s1, w2, s2) if t is not None]
+    tensors = [t for t in (data, scales, topk_idx, topk_weights, w1, s1, w2, s2, *(shared or ())) if t is not None]
     if any(t.requires_grad for t in tensors) or (out is not None and out.requires_grad):
         raise NotImplementedError("MegaMoE is inference-only")
     if out is not None:
@@ -330,6 +340,7 @@ def _run(x, topk_idx, topk_weights, l1_weights, l2_weights, sym_buffer, *, share
             ops.megamoe_forward(
                 b._workspace, data.contiguous(), scales.contiguous(), topk_idx.contiguous(), topk_weights.contiguous(),
                 w1, s1, w2, s2, b.num_experts, b.group.rank() * b.num_local_experts, b.num_local_experts, y, counts,
+                shared=shared,
             )
             if cumulative_stats is not None:
                 cumulative_stats.add_(counts)

@@ -278,8 +278,8 @@ def mx_quant(x):
     return codes, scales
 
 
-def megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local) -> int:
-    return int(_lib.load().dpep_megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local))
+def megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local, num_shared: int = 0) -> int:
+    return int(_lib.load().dpep_megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local, num_shared))
 
 
 def megamoe_prepared_scale_cols(k: int) -> int:
@@ -312,8 +312,10 @@ def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
 
 
 def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s2, num_experts, expert_begin,
-                    num_local, y, expert_token_nums):
-    """Fused W4A8 forward of one rank's local experts; writes y [B,H] BF16 and expert_token_nums [L] int32."""
+                    num_local, y, expert_token_nums, shared=None):
+    """Fused W4A8 forward of one rank's local experts; writes y [B,H] BF16 and expert_token_nums [L] int32.
+
+    ``shared`` = (w1, s1, w2, s2) prepared weights of S shared experts, which every token passes through."""
     lib = _lib.load()
     dev = ws.device
     _require("x_codes", x_codes, torch.float8_e4m3fn, device=dev)
@@ -332,11 +334,21 @@ def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s
     _require("s2", s2, torch.uint8, (num_local, hidden, megamoe_prepared_scale_cols(intermediate)), dev)
     _require("y", y, torch.bfloat16, (tokens, hidden), dev)
     _require("expert_token_nums", expert_token_nums, torch.int32, (num_local,), dev)
+    num_shared = 0
+    sw1 = ss1 = sw2 = ss2 = None
+    if shared is not None:
+        sw1, ss1, sw2, ss2 = shared
+        _require("shared w1", sw1, torch.uint8, device=dev)
+        num_shared = sw1.shape[0]
+        _require("shared w1", sw1, torch.uint8, (num_shared, 2 * intermediate, hidden // 2), dev)
+        _require("shared s1", ss1, torch.uint8, (num_shared, 2 * intermediate, megamoe_prepared_scale_cols(hidden)), dev)
+        _require("shared w2", sw2, torch.uint8, (num_shared, hidden, intermediate // 2), dev)
+        _require("shared s2", ss2, torch.uint8, (num_shared, hidden, megamoe_prepared_scale_cols(intermediate)), dev)
     with _on_device(dev):
         status = lib.dpep_megamoe_forward(
             ws.handle, _ptr(x_codes), _ptr(x_scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(w1), _ptr(s1), _ptr(w2),
-            _ptr(s2), tokens, hidden, intermediate, topk, num_experts, expert_begin, num_local, _ptr(y),
-            _ptr(expert_token_nums), _stream(dev),
+            _ptr(s2), _ptr(sw1), _ptr(ss1), _ptr(sw2), _ptr(ss2), num_shared, tokens, hidden, intermediate, topk,
+            num_experts, expert_begin, num_local, _ptr(y), _ptr(expert_token_nums), _stream(dev),
         )
     _lib.check(status, "megamoe_forward")
     return y, expert_token_nums

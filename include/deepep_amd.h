@@ -110,8 +110,10 @@ int dpep_combine(const void* y, const float* row_weights, const int32_t* route_t
  *   x bf16 [B,H], H % 32 == 0 -> codes e4m3 [B,H], scales e8m0 [B,H/32] */
 int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* scales, void* stream);
 
-/* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480). */
-size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, int intermediate, int num_local);
+/* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480).
+ * num_shared = number of shared experts (0..8) whose rows (every token, each) are held next to the routed ones. */
+size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, int intermediate, int num_local,
+                                    int num_shared);
 
 /* Bytes of the prepared scale buffer of one weight tensor: the scales are stored in spans of four k tiles
  * (k = 512), the last span padded, so this equals L*N*K/32 when K % 512 == 0 and is larger otherwise.
@@ -134,12 +136,16 @@ int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scale
  *   x_codes e4m3 [B,H], x_scales e8m0 [B,H/32], topk_idx int32 [B,K] (distinct, in [0,E)), topk_weights fp32 [B,K]
  *   w1/s1: prepared GMM1 weights [L,2I,H/2] and scales; w2/s2: prepared GMM2 weights [L,H,I/2] and scales
  *   (scale sizes: dpep_megamoe_prepared_scale_bytes)
- *   y bf16 [B,H]; expert_token_nums int32 [L] */
+ *   shared_w1/s1/w2/s2: the same for num_shared shared experts ([S,2I,H/2] ...; sw1/sw2/ss1/ss2 of
+ *   mega_moe_kernel_do), NULL when num_shared == 0.  A shared expert processes every token and its output is
+ *   added with weight 1 after the routed experts' (golden.py:160-164).
+ *   y bf16 [B,H]; expert_token_nums int32 [L] (routed experts only) */
 int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales, const int32_t* topk_idx,
                          const float* topk_weights, const uint8_t* w1, const uint8_t* s1, const uint8_t* w2,
-                         const uint8_t* s2, int num_tokens, int hidden, int intermediate, int num_topk,
-                         int num_experts, int expert_begin, int num_local, void* y, int32_t* expert_token_nums,
-                         void* stream);
+                         const uint8_t* s2, const uint8_t* shared_w1, const uint8_t* shared_s1,
+                         const uint8_t* shared_w2, const uint8_t* shared_s2, int num_shared, int num_tokens, int hidden,
+                         int intermediate, int num_topk, int num_experts, int expert_begin, int num_local, void* y,
+                         int32_t* expert_token_nums, void* stream);
 
 #ifdef __cplusplus
 }

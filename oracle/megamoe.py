@@ -133,9 +133,10 @@ def expert_forward(x, w1, w2):
     return round_bf16(qa @ np.asarray(w2, dtype=np.float32).T)
 
 
-def local_reference(x, indices, weights, l1, l2, first_expert=0):
+def local_reference(x, indices, weights, l1, l2, first_expert=0, shared_l1=None, shared_l2=None):
     """fp32 sum over local experts (expert order) of expert_forward(x[token]) * w[token, slot]
-    (reference.py:92-100); the caller rounds to BF16 at the end (golden.py:121-201)."""
+    (reference.py:92-100); the caller rounds to BF16 at the end (golden.py:121-201).
+    Shared experts follow the routed ones: every token, no route weight (golden.py:160-173)."""
     x = np.asarray(x, dtype=np.float32)
     indices = np.asarray(indices)
     result = np.zeros_like(x, dtype=np.float32)
@@ -144,6 +145,9 @@ def local_reference(x, indices, weights, l1, l2, first_expert=0):
         if token.size:
             out = expert_forward(x[token], l1[local], l2[local])
             np.add.at(result, token, out * np.asarray(weights, dtype=np.float32)[token, slot, None])
+    if shared_l1 is not None:
+        for expert in range(len(shared_l1)):
+            result += expert_forward(x, shared_l1[expert], shared_l2[expert])
     return result
 
 

@@ -105,6 +105,51 @@ def test_megamoe_forward_matches_oracle(ops, tokens, hidden, inter, experts, beg
     assert not got[untouched].any()  # tokens without a local expert receive zeros
 
 
+@pytest.mark.parametrize("tokens,hidden,inter,experts,begin,local,topk,shared", [
+    (100, 512, 512, 8, 0, 8, 2, 1),     # one shared expert beside 8 routed ones
+    (257, 768, 512, 6, 2, 2, 3, 2),     # two shared experts, partial local range, more than one row tile each
+])
+def test_megamoe_forward_with_shared_experts(ops, tokens, hidden, inter, experts, begin, local, topk, shared):
+    # shared experts take every token with weight 1 after the routed experts
+    # (experiments/megamoe/python/deep_ep_experimental/megamoe/golden.py:160-173)
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=3)
+    rng = np.random.default_rng(99)
+    sp1, ss1 = mm.quantize_weight_mxfp4((rng.normal(size=(shared, 2 * inter, hidden)) * 0.02).astype(np.float32))
+    sp2, ss2 = mm.quantize_weight_mxfp4((rng.normal(size=(shared, hidden, inter)) * 0.02).astype(np.float32))
+    dev = "cuda"
+    w1, s1 = ops.megamoe_prepare_weights(torch.from_numpy(l1[0]).to(dev), torch.from_numpy(l1[1]).reshape(local, 2 * inter, -1).to(dev), True)
+    w2, s2 = ops.megamoe_prepare_weights(torch.from_numpy(l2[0]).to(dev), torch.from_numpy(l2[1]).reshape(local, hidden, -1).to(dev), False)
+    sw1, sws1 = ops.megamoe_prepare_weights(torch.from_numpy(sp1).to(dev), torch.from_numpy(ss1).reshape(shared, 2 * inter, -1).to(dev), True)
+    sw2, sws2 = ops.megamoe_prepare_weights(torch.from_numpy(sp2).to(dev), torch.from_numpy(ss2).reshape(shared, hidden, -1).to(dev), False)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local, shared))
+    y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+    try:
+        ops.megamoe_forward(
+            ws, torch.from_numpy(x_codes).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(x_scales).to(dev),
+            torch.from_numpy(idx).to(dev), torch.from_numpy(weights).to(dev), w1, s1, w2, s2, experts, begin, local, y,
+            counts, shared=(sw1, sws1, sw2, sws2),
+        )
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+    finally:
+        ws.destroy()
+    xq = mm.mx_dequantize(x_codes, x_scales)
+    want = mm.round_bf16(mm.local_reference(xq, idx, weights, mm.unpack_weight(*l1), mm.unpack_weight(*l2), begin,
+                                            mm.unpack_weight(sp1, ss1), mm.unpack_weight(sp2, ss2)))
+    np.testing.assert_array_equal(counts.cpu().numpy(), np.bincount(idx.ravel(), minlength=experts)[begin : begin + local])
+    assert np.isfinite(got).all()
+    err = mm.relative_frobenius(got, want)
+    assert err <= 2e-2, err
+    # the shared part alone must be there for tokens without any local route
+    untouched = ~((idx >= begin) & (idx < begin + local)).any(axis=1)
+    if untouched.any():
+        only_shared = mm.round_bf16(mm.local_reference(xq[untouched], np.full((int(untouched.sum()), topk), -1), weights[untouched],
+                                                       mm.unpack_weight(*l1), mm.unpack_weight(*l2), begin,
+                                                       mm.unpack_weight(sp1, ss1), mm.unpack_weight(sp2, ss2)))
+        assert mm.relative_frobenius(got[untouched], only_shared) <= 2e-2
+
+
 def test_megamoe_forward_rank_share_shape(ops):
     # one EP rank's share at reduced token count: H=7168, I=2048, 6 local experts of 384, top-8
     tokens, hidden, inter, experts, local, topk = 2048, 7168, 2048, 384, 6, 8
@@ -224,3 +269,35 @@ def test_megamoe_forward_in_hip_graph(ops):
     finally:
         torch.cuda.synchronize()
         ws.destroy()
+
+
+def test_public_api_shared_experts():
+    # SymmBuffer(num_shared_experts=S) + transform_weights_for_mega_moe(..., shared=True) + shared_l*_weights
+    from deepep_amd import megamoe
+
+    tokens, hidden, inter, experts, topk, shared = 33, 1024, 512, 4, 2, 1
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, experts, topk, seed=8)
+    rng = np.random.default_rng(5)
+    sp1, ss1 = mm.quantize_weight_mxfp4((rng.normal(size=(shared, 2 * inter, hidden)) * 0.02).astype(np.float32))
+    sp2, ss2 = mm.quantize_weight_mxfp4((rng.normal(size=(shared, hidden, inter)) * 0.02).astype(np.float32))
+    buf = megamoe.SymmBuffer(None, experts, tokens, topk, hidden, inter, num_shared_experts=shared)
+    try:
+        p1, p2 = megamoe.transform_weights_for_mega_moe(
+            (torch.from_numpy(l1[0]).cuda(), torch.from_numpy(l1[1]).cuda()), (torch.from_numpy(l2[0]).cuda(), torch.from_numpy(l2[1]).cuda()))
+        q1, q2 = megamoe.transform_weights_for_mega_moe(
+            (torch.from_numpy(sp1).cuda(), torch.from_numpy(ss1).cuda()), (torch.from_numpy(sp2).cuda(), torch.from_numpy(ss2).cuda()),
+            shared=True)
+        x = (torch.from_numpy(x_codes).cuda().view(torch.float8_e4m3fn), torch.from_numpy(x_scales).cuda())
+        ids, wts = torch.from_numpy(idx).cuda(), torch.from_numpy(weights).cuda()
+        with pytest.raises(ValueError, match="Shared expert count"):
+            megamoe.mega_moe(x, ids, wts, p1, p2, buf)
+        with pytest.raises(ValueError, match="both shared"):
+            megamoe.mega_moe(x, ids, wts, p1, p2, buf, shared_l1_weights=q1)
+        y, counts = megamoe.mega_moe(x, ids, wts, p1, p2, buf, shared_l1_weights=q1, shared_l2_weights=q2)
+        assert counts.cpu().tolist() == np.bincount(idx.ravel(), minlength=experts).tolist()
+        xq = mm.mx_dequantize(x_codes, x_scales)
+        want = mm.round_bf16(mm.local_reference(xq, idx, weights, mm.unpack_weight(*l1), mm.unpack_weight(*l2), 0,
+                                                mm.unpack_weight(sp1, ss1), mm.unpack_weight(sp2, ss2)))
+        assert mm.relative_frobenius(y.float().cpu().numpy(), want) <= 2e-2
+    finally:
+        buf.destroy()

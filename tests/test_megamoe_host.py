@@ -28,8 +28,8 @@ def test_symm_buffer_argument_gates():
         args.update(kwargs)
         with pytest.raises(ValueError):
             SymmBuffer(**args)
-    with pytest.raises(NotImplementedError):
-        SymmBuffer(None, 4, 17, 2, 1024, 512, num_shared_experts=1)
+    with pytest.raises(ValueError):
+        SymmBuffer(None, 4, 17, 2, 1024, 512, num_shared_experts=9)
     with pytest.raises(TypeError):
         SymmBuffer(object(), 4, 17, 2, 1024, 512)
     with pytest.raises(ValueError):

@@ -68,6 +68,25 @@ def test_decomposition_and_single_expert():  # :57-71
     np.testing.assert_allclose(full[2:3], mm.expert_forward(x[2:3], w1[0], w2[0]))
 
 
+def test_shared_experts_are_dense_unweighted_terms():
+    # golden.py:160-173: a shared expert takes every token, no route weight, after the routed experts; so the
+    # result equals the routed part plus a one-expert "route everything with weight 1" problem per shared expert
+    rng = np.random.default_rng(11)
+    x = rng.normal(size=(5, 32)).astype(np.float32) * 0.1
+    w1 = rng.normal(size=(3, 64, 32)).astype(np.float32) * 0.1
+    w2 = rng.normal(size=(3, 32, 32)).astype(np.float32) * 0.1
+    s1 = rng.normal(size=(2, 64, 32)).astype(np.float32) * 0.1
+    s2 = rng.normal(size=(2, 32, 32)).astype(np.float32) * 0.1
+    ids = rng.integers(0, 3, size=(5, 1))
+    weights = rng.random((5, 1)).astype(np.float32)
+    routed = mm.local_reference(x, ids, weights, w1, w2, 0)
+    full = mm.local_reference(x, ids, weights, w1, w2, 0, s1, s2)
+    dense = sum(mm.local_reference(x, np.zeros((5, 1), int), np.ones((5, 1), np.float32), s1[e : e + 1], s2[e : e + 1], 0)
+                for e in range(2))
+    np.testing.assert_allclose(full, routed + dense, atol=1e-7)
+    assert np.abs(dense).max() > 0
+
+
 def test_route_weight_does_not_commute_with_quantization():  # :79-88
     rng = np.random.default_rng(31)
     act = rng.normal(size=(8, 64)).astype(np.float32)
