@@ -70,6 +70,8 @@ def check(status: int, what: str) -> None:
     if status == 0:
         return
     message = load().dpep_last_error().decode("utf-8", "replace")
+    if not message.startswith(what):
+        message = f"{what}: {message}"
     if status == -1:
-        raise ValueError(f"{what}: {message}")
-    raise NativeError(f"{what}: {message}")
+        raise ValueError(message)
+    raise NativeError(message)

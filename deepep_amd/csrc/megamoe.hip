@@ -899,8 +899,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     DPEP_REQUIRE(hidden % 256 == 0 && intermediate % 256 == 0 && hidden >= 512 && intermediate >= 512,
                  "megamoe_forward: hidden=%d and intermediate=%d must be multiples of 256, at least 512", hidden,
                  intermediate);
-    DPEP_REQUIRE(num_local >= 1 && expert_begin >= 0 && expert_begin + num_local <= num_experts,
-                 "megamoe_forward: bad expert range E=%d begin=%d L=%d", num_experts, expert_begin, num_local);
+    DPEP_REQUIRE(num_local >= 1 && num_local <= kMaxMoeExperts && expert_begin >= 0 &&
+                     expert_begin + num_local <= num_experts,
+                 "megamoe_forward: bad expert range E=%d begin=%d L=%d (at most %d local experts)", num_experts,
+                 expert_begin, num_local, kMaxMoeExperts);
     DPEP_REQUIRE(num_shared >= 0 && num_shared <= 8 && num_topk + num_shared <= DPEP_MAX_TOPK &&
                      num_local + num_shared <= kMaxMoeExperts,
                  "megamoe_forward: %d shared experts with K=%d, L=%d (at most 8, K+S <= %d, L+S <= %d)", num_shared,
