@@ -164,11 +164,15 @@ def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows:
     scale_cols = 0
     out_scales = None
     if scales is not None:
-        _require("scales", scales, torch.float32, device=dev)
+        # FP32 scales, or int32 words holding four packed E8M0 bytes (the low-latency scale format,
+        # docs/elastic.md:97): either way 4-byte words that are moved bit for bit
+        if not isinstance(scales, torch.Tensor) or scales.dtype not in (torch.float32, torch.int32):
+            raise ValueError("scales must be FP32 or packed int32")
+        _require("scales", scales, scales.dtype, device=dev)
         if scales.ndim != 2 or scales.shape[0] != tokens:
             raise ValueError("scales must be [T, C]")
         scale_cols = scales.shape[1]
-        out_scales = torch.empty((num_rows, scale_cols), dtype=torch.float32, device=dev)
+        out_scales = torch.empty((num_rows, scale_cols), dtype=scales.dtype, device=dev)
     out_weights = None
     if topk_weights is not None:
         _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)

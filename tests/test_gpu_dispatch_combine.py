@@ -256,3 +256,20 @@ def test_argument_errors(ops, ws):
         ops.dispatch_quant_fp8(x, None, lay["route_to_row"], lay["row_to_route"], 8)  # H % 128
     with pytest.raises(ValueError):
         ops.combine(torch.zeros((8, 12), dtype=torch.bfloat16).cuda(), lay["route_to_row"])  # H % 8
+
+
+def test_dispatch_moves_packed_int32_scales_and_fp16_payload(ops, ws):
+    # low-latency formats pass through unchanged: FP16 payload rows and int32 words of four packed E8M0 bytes
+    rng = np.random.default_rng(3)
+    tokens, topk, experts, hidden = 64, 4, 16, 512
+    idx_np = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)])
+    lay = ops.layout(ws, torch.from_numpy(idx_np).cuda(), experts)
+    _, rows = ops.layout_wait(ws)
+    want = olayout.layout(idx_np, experts)
+    x = torch.from_numpy(rng.normal(size=(tokens, hidden)).astype(np.float16)).cuda()
+    packed = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=(tokens, hidden // 128), dtype=np.int64).astype(np.int32)).cuda()
+    out, out_scales, _ = ops.dispatch_copy(x, packed, None, lay["route_to_row"], lay["row_to_route"], rows)
+    token_of_row = want["row_to_route"] // topk
+    assert out.dtype == torch.float16 and out_scales.dtype == torch.int32
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint16), x.cpu().numpy().view(np.uint16)[token_of_row])
+    np.testing.assert_array_equal(out_scales.cpu().numpy(), packed.cpu().numpy()[token_of_row])
