@@ -164,7 +164,7 @@ constexpr int kStagingRowStride = 80;  // 32 BF16 + 16 B pad: conflict-free 16-b
 template <int RT, bool kGather>
 struct GemmCfg {
     static constexpr int kBM = 64 * RT;
-    static constexpr int kStages = RT == 2 ? 4 : 3;
+    static constexpr int kStages = RT == 1 ? 5 : RT == 2 ? 4 : 3;
     // Copies run a full ring ahead: a stage is refilled in the very item that consumes it, right after the
     // barrier that follows the last LDS read of it.
     static constexpr int kAhead = kStages;
@@ -265,7 +265,10 @@ __device__ __forceinline__ void wait_copies_then_barrier()
 // which is what lets the copies and the barrier be placed between individual MFMAs (builtin MFMAs are pure
 // and the compiler gathers them into bursts).  kSecond selects scale bytes 2|3 of A and byte 1 of B.
 // The compiler cannot see an MFMA in here, so the code that reads an accumulator afterwards has to
-// provide the wait states itself (settle_accumulators).
+// provide the wait states itself (settle_accumulators).  For the same reason these statements must stay in
+// straight-line code: with a branch around one the register allocator splits the accumulator's live range
+// and copies it out of the AGPRs right behind the instruction, before its last passes have written
+// (measured: accumulator registers 10-15 of every tile stale).
 template <bool kSecond>
 __device__ __forceinline__ void mfma_fp8_fp4(v16f& acc, const v8i& a, const u32x4& b, int scale_a, int scale_b)
 {
@@ -657,12 +660,13 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             // fragments (whose registers the first k step has released).
             shift_scales(parity);
             constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
-            static_assert((kGroups + 1) / 2 < kMfmas / 2, "the second k step's fragments leave LDS before the barrier");
+            // enough read groups per MFMA that the second k step's fragments have all left LDS before the barrier
+            constexpr int kReadsPerMfma = (kGroups + kMfmas / 2 - 1) / (kMfmas / 2);
 #pragma unroll
             for (int n = 0; n < kMfmas; ++n) {
                 mfma_one(0, parity, n);
 #pragma unroll
-                for (int group = 2 * n; group < 2 * n + 2; ++group)
+                for (int group = kReadsPerMfma * n; group < kReadsPerMfma * (n + 1); ++group)
                     if (group < kGroups) read_group(stage_now, 1, group);
                 if (n == kMfmas / 2 - 1) {
                     // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies
@@ -760,7 +764,7 @@ int launch_gemm_rt(const GemmParams& p, hipStream_t stream, const char* what)
     return launch_status(what);
 }
 
-// Row-tile height: the cheaper of 128 / 192 rows, whose tile count fits one round of workgroups, judged
+// Row-tile height: the cheapest of 64 / 128 / 192 rows, whose tile count fits one round of workgroups, judged
 // from the expected rows per expert (the true counts stay on the device).
 template <bool kGateUp>
 int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t stream, const char* what)
@@ -769,12 +773,15 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
     const int n_tiles = p.n / kBN;
     int best = 2;
     double best_cost = 1e30;
-    for (int rt = 2; rt <= 3; ++rt) {
+    for (int rt = 1; rt <= 3; ++rt) {
         const int bm = 64 * rt;
         const int m_tiles = (expected_rows_per_expert + bm - 1) / bm;
         const long long tiles = static_cast<long long>(p.num_local) * (m_tiles > 0 ? m_tiles : 1) * n_tiles;
         const long long rounds = (tiles + cus - 1) / cus;
-        const double cost = static_cast<double>(rounds) * rt;  // time of a tile grows with its height
+        // The time of a tile grows with its height, on top of a part that does not (its weight tile has to be
+        // fetched whatever the height, and there are the prologue and epilogue): the 64-row tile pays off only
+        // when the experts have few rows (decode), where the GEMM is bound by streaming the weights.
+        const double cost = static_cast<double>(rounds) * (rt + 0.5);
         if (cost < best_cost - 1e-9) {
             best_cost = cost;
             best = rt;
@@ -783,6 +790,7 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
 #ifdef DPEP_TUNE_GEMM_RT
     best = DPEP_TUNE_GEMM_RT;
 #endif
+    if (best == 1) return launch_gemm_rt<1, kGateUp>(p, stream, what);
     if (best == 2) return launch_gemm_rt<2, kGateUp>(p, stream, what);
     return launch_gemm_rt<3, kGateUp>(p, stream, what);
 }
