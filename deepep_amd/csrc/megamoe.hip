@@ -703,6 +703,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         if (kt == ktiles) {
             DPEP_STAMP(4);
             settle_accumulators();
+            // tie every accumulator to a statement behind the wait, so that no read of it can be moved above
+#pragma unroll
+            for (int i = 0; i < RT; ++i)
+#pragma unroll
+                for (int c = 0; c < kCT; ++c) asm volatile("" : "+a"(acc[i][c]));
             epilogue(info);
             DPEP_STAMP(5);
             clear_acc();
