@@ -84,8 +84,9 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const u32x4* __restrict__
 }
 
 // =====================================================================================================
-// Weight re-layout: raw [L][N][K/2] + [L][N][K/32]  ->  per (column tile of 32, k step of 64) one
-// contiguous 1 KiB block holding every lane's 16-byte B fragment; scales as 2 bytes per lane per k=128.
+// Weight re-layout: raw [L][N][K/2] + [L][N][K/32]  ->  1 KiB blocks holding every lane's 16-byte B fragment of
+// one (column tile of 32, k step of 64), ordered [expert][256 columns][k tile of 128][column tile][k step] so
+// that a workgroup's 16 KiB per item are contiguous; scales as 2 bytes per lane per k=128.
 // =====================================================================================================
 __device__ __forceinline__ int source_row(int physical_col, int n, int gate_up)
 {
@@ -102,14 +103,17 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
                                                               long long packed_chunks, long long scale_pairs)
 {
     const long long id = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const int ksteps = k / 64, ktiles = k / 128, ctiles = n / 32;
-    if (id < packed_chunks) {  // one 16-byte fragment
-        const int lane = id & 63;
-        long long rest = id >> 6;
-        const int ks = rest % ksteps;
-        rest /= ksteps;
-        const int c = rest % ctiles;
-        const long long e = rest / ctiles;
+    const int ktiles = k / 128;
+    if (id < packed_chunks) {
+        // one 16-byte fragment; order [expert][block of 8 column tiles][k tile][column tile][k step][lane]: the
+        // 16 KiB a workgroup copies per item are contiguous and its items follow each other in memory
+        const int lane = id & 63, q = (id >> 6) & 15;
+        long long rest = id >> 10;
+        const int kt = rest % ktiles;
+        rest /= ktiles;
+        const int nb = rest % (n / 256);
+        const long long e = rest / (n / 256);
+        const int c = nb * 8 + (q >> 1), ks = kt * 2 + (q & 1);
         const int row = source_row(c * 32 + (lane & 31), n, gate_up);
         const uint8_t* src = w + (e * n + row) * (k / 2) + ks * 32 + (lane >> 5) * 16;
         reinterpret_cast<u32x4*>(w_out)[id] = *reinterpret_cast<const u32x4*>(src);
@@ -311,7 +315,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     const int wm = wave >> 1, wn = wave & 1;
     const int g = lane >> 5, lr = lane & 31;
     const int n_tiles = p.n / kBN;
-    const int ksteps = p.k / 64, ktiles = p.k / kBK;
+    const int ktiles = p.k / kBK;
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
     const uint32_t lds_index = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&tile_index[0][0]));
 
@@ -388,12 +392,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         const bool shared = info.expert >= p.num_routed;
         const size_t weight_index = shared ? info.expert - p.num_routed : info.expert;
         b_base = (shared ? p.w_shared : p.w) + weight_index * p.n * (p.k / 2) +
-                 static_cast<size_t>(info.nt) * (2 * kCT) * ksteps * 1024;
+                 static_cast<size_t>(info.nt) * ktiles * 16384;
         // fragment q = copy*4 + wave of the 16 (column tile, k step) fragments of one k tile
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int q = j * 4 + wave;
-            b_off[j] = static_cast<uint32_t>(((q >> 1) * ksteps + (q & 1)) * 1024 + lane * 16);
+            b_off[j] = static_cast<uint32_t>(q * 1024 + lane * 16);
         }
         sb_src = (shared ? p.ws_shared : p.ws) + (weight_index * n_tiles + info.nt) * spans * Cfg::kColScaleSlot + tid * 16;
     };
@@ -416,7 +420,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         if (c < 2 * RT)
             copy16_to_lds(p.a_codes + static_cast<size_t>(copy_kt) * kBK, a_off[c], stage + Cfg::kOffA + c * 4096 + wave * 1024);
         else
-            copy16_to_lds(b_base + static_cast<size_t>(copy_kt) * 2048, b_off[c - 2 * RT],
+            copy16_to_lds(b_base + static_cast<size_t>(copy_kt) * 16384, b_off[c - 2 * RT],
                           stage + Cfg::kOffB + ((c - 2 * RT) * 4 + wave) * 1024);
     };
     // Every fourth item starts a new span: a 16-byte window of row scales per row (clamped so that it never
