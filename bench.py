@@ -193,9 +193,12 @@ def main():
     ws = ops.Workspace(max(ops.layout_workspace_bytes(tokens, topk, experts), 1 << 20))
 
     def step():
+        # as ElasticBuffer.dispatch does when every expert is local: the payload kernel is queued behind the layout
+        # into outputs of T*K rows, and the host synchronisation that yields R (to narrow them) runs meanwhile
         lay = ops.layout(ws, idxd, experts)
-        _, rows = ops.layout_wait(ws)  # the host synchronisation a fresh dispatch needs to size its outputs
-        recv = ops.dispatch_quant_fp8(xd, wd, lay["route_to_row"], lay["row_to_route"], rows)
+        full = ops.dispatch_quant_fp8(xd, wd, lay["route_to_row"], lay["row_to_route"], None)
+        _, rows = ops.layout_wait(ws)
+        recv = tuple(t[:rows] for t in full)
         out = ops.combine(gd[:rows], lay["route_to_row"])
         return rows, recv, out
 

@@ -231,9 +231,10 @@ int check_common(const char* what, int num_tokens, int num_topk, int num_rows, c
 {
     DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "%s: bad T=%d K=%d", what, num_tokens,
                  num_topk);
-    DPEP_REQUIRE(num_rows >= 0 && static_cast<long long>(num_rows) <= static_cast<long long>(num_tokens) * num_topk,
-                 "%s: num_rows=%d outside [0, T*K]", what, num_rows);
-    DPEP_REQUIRE(num_rows == 0 || (route_to_row != nullptr && row_to_route != nullptr), "%s: NULL routing maps", what);
+    DPEP_REQUIRE(num_rows >= -1 && static_cast<long long>(num_rows) <= static_cast<long long>(num_tokens) * num_topk,
+                 "%s: num_rows=%d outside [0, T*K] (or -1: not known yet)", what, num_rows);
+    DPEP_REQUIRE(num_rows == 0 || route_to_row != nullptr, "%s: NULL routing maps", what);
+    DPEP_REQUIRE(num_rows <= 0 || row_to_route != nullptr, "%s: NULL routing maps", what);
     return DPEP_OK;
 }
 
@@ -253,11 +254,12 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
     DPEP_REQUIRE((scales == nullptr) == (out_scales == nullptr), "dispatch_copy: scales and out_scales go together");
     DPEP_REQUIRE(scales == nullptr || scale_cols > 0, "dispatch_copy: scale_cols must be positive with scales");
     DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "dispatch_copy: weights and out_weights go together");
-    if (num_rows == 0) return DPEP_OK;
+    if (num_rows == 0 || num_tokens == 0) return DPEP_OK;
     DPEP_REQUIRE(x != nullptr && out != nullptr && aligned16(x) && aligned16(out), "dispatch_copy: x/out must be 16-byte aligned");
     const int vec = row_bytes / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
+    // the token-major grid does not depend on R, so a launch that does not know R yet takes it
+    if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
         const Split sp = choose_split(num_tokens, vec, 1);
         hipLaunchKernelGGL(dispatch_copy_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
                            static_cast<const u32x4*>(x), scales, topk_weights, route_to_row, num_topk, vec, sp.per_part,
@@ -280,11 +282,12 @@ int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int3
     DPEP_REQUIRE(hidden > 0 && hidden % 128 == 0 && hidden / 128 <= kMaxScaleCols,
                  "dispatch_quant_fp8: hidden=%d must be a positive multiple of 128, at most %d", hidden, 128 * kMaxScaleCols);
     DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "dispatch_quant_fp8: weights and out_weights go together");
-    if (num_rows == 0) return DPEP_OK;
+    if (num_rows == 0 || num_tokens == 0) return DPEP_OK;
     DPEP_REQUIRE(x && out && out_scales && aligned16(x) && aligned16(out), "dispatch_quant_fp8: x/out must be 16-byte aligned");
     const int units = hidden / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
+    // the token-major grid does not depend on R, so a launch that does not know R yet takes it
+    if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
         const Split sp = choose_split(num_tokens, units, 8);
         hipLaunchKernelGGL(dispatch_quant_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
                            static_cast<const u32x4*>(x), topk_weights, route_to_row, num_topk, units, sp.per_part,

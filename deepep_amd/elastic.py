@@ -500,18 +500,29 @@ class ElasticBuffer:
                 producer = EventHandle()
                 with gpu_api().stream(runtime.stream):
                     producer.current_stream_wait()
+
+                    def payload(rows):
+                        if fuse_quant:
+                            return native.dispatch_quant_fp8(hidden, topk_weights, route_to_row, row_to_route, rows)
+                        return native.dispatch_copy(hidden, scales, topk_weights, route_to_row, row_to_route, rows)
+
                     if handle is None:
-                        handle = self._notify(hidden, topk_idx, num_experts, capacity, do_handle_copy)
-                    rows = handle.num_expanded_tokens
-                    row_to_route = handle._row_to_route_full
-                    if fuse_quant:
-                        out, out_scales, out_weights = native.dispatch_quant_fp8(
-                            hidden, topk_weights, handle.route_to_row, row_to_route, rows
-                        )
+                        plan, indices = self._notify_launch(topk_idx, num_experts, do_handle_copy)
+                        route_to_row, row_to_route = plan["route_to_row"], plan["row_to_route"]
+                        # Where most routes stay on this rank, outputs allocated for all T*K routes cost little, and
+                        # the payload kernel can be queued right behind the layout: the host reads R while both
+                        # run and narrows the outputs, instead of leaving the GPU idle between the two.
+                        early = 2 * (num_experts // world) >= num_experts
+                        full = payload(None) if early else None
+                        handle = self._notify_finish(hidden, plan, indices, num_experts, capacity)
+                        rows = handle.num_expanded_tokens
+                        if early:
+                            out, out_scales, out_weights = (None if t is None else t[:rows] for t in full)
+                        else:
+                            out, out_scales, out_weights = payload(rows)
                     else:
-                        out, out_scales, out_weights = native.dispatch_copy(
-                            hidden, scales, topk_weights, handle.route_to_row, row_to_route, rows
-                        )
+                        route_to_row, row_to_route = handle.route_to_row, handle._row_to_route_full
+                        out, out_scales, out_weights = payload(handle.num_expanded_tokens)
                     retained = (hidden, scales, topk_weights, out, out_scales, out_weights, handle.topk_idx) + tuple(
                         getattr(handle, name) for name in _ROUTING
                     )
@@ -529,20 +540,24 @@ class ElasticBuffer:
                 runtime.notify_failed = True
                 raise
 
-    def _notify(self, hidden, topk_idx, num_experts, capacity, do_handle_copy) -> EPHandle:
-        """Routing layout + the one host read-back (counts, prefix, R) that sizes the outputs."""
+    def _notify_launch(self, topk_idx, num_experts, do_handle_copy):
+        """Queues the routing layout; returns its device outputs and the routing tensor it read."""
         runtime = self._runtime
-        native = runtime.native
-        tokens, width = hidden.shape
-        topk = topk_idx.shape[1]
         local = num_experts // runtime.world_size
-        begin = runtime.rank * local
         # Persistent routing keeps version counters even when the caller runs in inference mode.
         with torch.inference_mode(False), torch.no_grad():
             indices = topk_idx.clone() if do_handle_copy else topk_idx
-            plan = native.layout(runtime.workspace, indices, num_experts, begin, local)
-            # The single host synchronisation: the kernel reports counts and R through pinned host memory.
-            counts, rows = native.layout_wait(runtime.workspace, local, 100.0)  # num_gpu_timeout_secs
+            plan = runtime.native.layout(runtime.workspace, indices, num_experts, runtime.rank * local, local)
+        return plan, indices
+
+    def _notify_finish(self, hidden, plan, indices, num_experts, capacity) -> EPHandle:
+        """The one host read-back (counts, R) that sizes the outputs, and the handle built from it."""
+        runtime = self._runtime
+        tokens, width = hidden.shape
+        topk = indices.shape[1]
+        local = num_experts // runtime.world_size
+        # The single host synchronisation: the kernel reports counts and R through pinned host memory.
+        counts, rows = runtime.native.layout_wait(runtime.workspace, local, 100.0)  # num_gpu_timeout_secs
         handle = EPHandle(
             True, num_experts, 1, capacity, 64, indices, None, rows, counts, None, plan["psum"], plan["counts"], None,
             None, None, None,

@@ -144,8 +144,11 @@ def layout_wait(ws: Workspace, num_local: Optional[int] = None, timeout_s: float
     return counts, int(rows.value)
 
 
-def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows: int):
-    """out[row] = x[token(row)] (+ scale rows, + per-row weights).  x is BF16 [T,H] or FP8 [T,H]."""
+def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows: Optional[int]):
+    """out[row] = x[token(row)] (+ scale rows, + per-row weights).  x is BF16 [T,H] or FP8 [T,H].
+
+    ``num_rows=None``: R is not known on the host yet (no ``layout_wait``): the outputs are allocated with T*K rows,
+    of which the first R are written; the caller narrows them once it has R."""
     lib = _lib.load()
     if not isinstance(x, torch.Tensor) or x.dtype not in (torch.bfloat16, torch.float8_e4m3fn, torch.float16):
         raise ValueError("x must be a BF16, FP16 or FP8 E4M3FN tensor")
@@ -161,6 +164,7 @@ def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows:
     row_bytes = hidden * x.element_size()
     if row_bytes % 16:
         raise ValueError("hidden row size must be a multiple of 16 bytes")
+    num_rows, known_rows = (tokens * topk, -1) if num_rows is None else (num_rows, num_rows)
     scale_cols = 0
     out_scales = None
     if scales is not None:
@@ -180,15 +184,15 @@ def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows:
     out = torch.empty((num_rows, hidden), dtype=x.dtype, device=dev)
     with _on_device(dev):
         status = lib.dpep_dispatch_copy(
-            _ptr(x), _ptr(scales), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, num_rows,
+            _ptr(x), _ptr(scales), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, known_rows,
             row_bytes, scale_cols, _ptr(out), _ptr(out_scales), _ptr(out_weights), _stream(dev),
         )
     _lib.check(status, "dispatch_copy")
     return out, out_scales, out_weights
 
 
-def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: int):
-    """Fused per-128 FP8 quantisation + expand-permute of BF16 x [T,H]."""
+def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: Optional[int]):
+    """Fused per-128 FP8 quantisation + expand-permute of BF16 x [T,H]; ``num_rows=None`` as in ``dispatch_copy``."""
     lib = _lib.load()
     _require("x", x, torch.bfloat16)
     if x.ndim != 2:
@@ -201,6 +205,7 @@ def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: in
     topk = route_to_row.shape[1]
     _require("route_to_row", route_to_row, torch.int32, (tokens, topk), dev)
     _require("row_to_route", row_to_route, torch.int32, device=dev)
+    num_rows, known_rows = (tokens * topk, -1) if num_rows is None else (num_rows, num_rows)
     out_weights = None
     if topk_weights is not None:
         _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)
@@ -209,7 +214,7 @@ def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: in
     out_scales = torch.empty((num_rows, hidden // 128), dtype=torch.float32, device=dev)
     with _on_device(dev):
         status = lib.dpep_dispatch_quant_fp8(
-            _ptr(x), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, num_rows, hidden,
+            _ptr(x), _ptr(topk_weights), _ptr(route_to_row), _ptr(row_to_route), tokens, topk, known_rows, hidden,
             _ptr(out), _ptr(out_scales), _ptr(out_weights), _stream(dev),
         )
     _lib.check(status, "dispatch_quant_fp8")

@@ -75,7 +75,10 @@ int dpep_layout_wait(void* ws, int32_t* counts_host, int num_local, int32_t* num
  *   row_bytes     bytes per payload row (BF16: 2H, FP8: H); must be a multiple of 16
  *   scales        optional fp32 [T, scale_cols] side rows moved with the payload (FP8 per-128 scales)
  *   topk_weights  optional fp32 [T,K]; out_weights[row] = topk_weights[t,s]
- *   num_rows      R (host value read back from dpep_layout) */
+ *   num_rows      R (host value from dpep_layout_wait), or -1 when the host does not know R yet: the launch then
+ *                 does not depend on R, out / out_scales / out_weights must hold T*K rows and the first R are
+ *                 written.  A caller that allocates at capacity can thus queue layout and dispatch back to back
+ *                 and read R (to narrow its outputs) while they run. */
 int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_weights,
                        const int32_t* route_to_row, const int32_t* row_to_route, int num_tokens,
                        int num_topk, int num_rows, int row_bytes, int scale_cols, void* out,
@@ -84,7 +87,8 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
 /* Fused per-128-element FP8 e4m3fn quantisation + expand-permute: the reference's caller-side
  * per_token_cast_to_fp8 (deep_ep/utils/math.py:45-61) followed by the FP8 dispatch above, in one pass.
  *   x             bf16 [T,H], H % 128 == 0
- *   out           fp8  [R,H]; out_scales fp32 [R, H/128] */
+ *   out           fp8  [R,H]; out_scales fp32 [R, H/128]
+ *   num_rows      R or -1, as for dpep_dispatch_copy */
 int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int32_t* route_to_row,
                             const int32_t* row_to_route, int num_tokens, int num_topk, int num_rows,
                             int hidden, void* out, float* out_scales, float* out_weights, void* stream);

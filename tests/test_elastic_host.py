@@ -51,10 +51,19 @@ class FakeNative:
         if self.fail_next:
             raise RuntimeError(self.fail_next)
         self.calls["dispatch_copy"] += 1
+        # rows=None: R not known to the caller yet; outputs hold T*K rows, the tail is left as filler
+        pad = 0 if rows is not None else route_to_row.numel() - self.last_layout[1]
+        self.calls["dispatch_at_capacity"] += rows is None
+        rows = self.last_layout[1] if rows is None else rows
         route = row_to_route[:rows].long()
         token = route // route_to_row.shape[1]
-        out = x.view(torch.uint8 if x.element_size() == 1 else torch.int16)[token].view(x.dtype)
-        return out, None if scales is None else scales[token], None if w is None else w.reshape(-1)[route]
+
+        def padded(t):
+            return None if t is None else torch.cat([t, torch.full((pad,) + t.shape[1:], 77).to(t.dtype)])
+
+        out = x.view(torch.uint8 if x.element_size() == 1 else torch.int16)[token]
+        return (padded(out).view(x.dtype), padded(None if scales is None else scales[token]),
+                padded(None if w is None else w.reshape(-1)[route]))
 
     def dispatch_quant_fp8(self, x, w, route_to_row, row_to_route, rows):
         self.calls["dispatch_quant_fp8"] += 1
@@ -116,6 +125,9 @@ def test_fresh_dispatch_combine_and_cached_dispatch(host):
     want = olayout.layout(idx.numpy(), 8)
     assert none is None and isinstance(ev, event.EventOverlap)
     assert handle.num_expanded_tokens == want["num_rows"] == recv.shape[0]
+    # every expert is local: the payload was queued before the host knew R, into outputs of T*K rows, then narrowed
+    assert calls["dispatch_at_capacity"] == 1 and want["num_rows"] < idx.numel()
+    assert recv.untyped_storage().nbytes() == idx.numel() * 128 * 2 and recv.is_contiguous()
     assert handle.num_recv_tokens_per_expert_list == want["counts"].tolist()
     assert handle.psum_num_recv_tokens_per_expert.tolist() == want["psum"].tolist()
     assert handle.num_unaligned_recv_tokens_per_expert.tolist() == want["counts"].tolist()
@@ -140,7 +152,7 @@ def test_fresh_dispatch_combine_and_cached_dispatch(host):
 
 
 def test_rank_share_selects_local_experts(host):
-    make, _ = host
+    make, calls = host
     buffer, _ = make(world=4, rank=2)
     x, idx, w = _inputs(tokens=16, experts=8, topk=3)
     recv, _, recv_w, handle, _ = buffer.dispatch(x, topk_idx=idx, topk_weights=w, num_experts=8)
@@ -148,6 +160,8 @@ def test_rank_share_selects_local_experts(host):
     assert handle.num_recv_tokens_per_expert_list == want["counts"].tolist()
     assert handle.weight_return_meta.tolist() == want["row_to_route"].tolist()
     assert recv.shape[0] == want["num_rows"]
+    # a quarter of the experts is local: outputs are sized after the host has read R
+    assert calls["dispatch_at_capacity"] == 0 and recv.untyped_storage().nbytes() == want["num_rows"] * 128 * 2
 
 
 def test_fp8_tuple_and_fused_quant(host):

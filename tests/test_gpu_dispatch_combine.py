@@ -273,3 +273,27 @@ def test_dispatch_moves_packed_int32_scales_and_fp16_payload(ops, ws):
     assert out.dtype == torch.float16 and out_scales.dtype == torch.int32
     np.testing.assert_array_equal(out.cpu().numpy().view(np.uint16), x.cpu().numpy().view(np.uint16)[token_of_row])
     np.testing.assert_array_equal(out_scales.cpu().numpy(), packed.cpu().numpy()[token_of_row])
+
+
+@pytest.mark.parametrize("name,tokens", [("C1", None), ("C2", None), ("C3", 700), ("C4", 2048)])
+def test_dispatch_before_the_host_knows_the_row_count(ops, ws, name, tokens):
+    """num_rows=None: layout and payload kernels queued back to back into outputs of T*K rows; the first R rows
+    equal those of a dispatch sized after the read-back, for the BF16 copy and the fused FP8 path, in dense and
+    rank-share routing alike."""
+    x, idx, w, cfg = cases.make_inputs(name, tokens=tokens)
+    xd, wd = x.cuda(), w.cuda()
+    lay = ops.layout(ws, idx.cuda(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    early = ops.dispatch_copy(xd, None, wd, lay["route_to_row"], lay["row_to_route"], None)
+    early_q = ops.dispatch_quant_fp8(xd, wd, lay["route_to_row"], lay["row_to_route"], None)
+    _, rows = ops.layout_wait(ws)
+    assert early[0].shape[0] == early_q[0].shape[0] == idx.numel() and early[1] is None
+    late = ops.dispatch_copy(xd, None, wd, lay["route_to_row"], lay["row_to_route"], rows)
+    late_q = ops.dispatch_quant_fp8(xd, wd, lay["route_to_row"], lay["row_to_route"], rows)
+    want = olayout.layout(idx.numpy(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    assert rows == want["num_rows"]
+    np.testing.assert_array_equal(bf16_bits(early[0][:rows]), olayout.expand_rows(bf16_bits(x), want["row_to_route"], cfg["topk"]))
+    np.testing.assert_array_equal(bf16_bits(early[0][:rows]), bf16_bits(late[0]))
+    np.testing.assert_array_equal(f32_bits(early[2][:rows]), f32_bits(late[2]))
+    np.testing.assert_array_equal(fp8_bits(early_q[0][:rows]), fp8_bits(late_q[0]))
+    np.testing.assert_array_equal(f32_bits(early_q[1][:rows]), f32_bits(late_q[1]))
+    np.testing.assert_array_equal(f32_bits(early_q[2][:rows]), f32_bits(late_q[2]))
