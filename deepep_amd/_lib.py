@@ -23,6 +23,7 @@ SIGNATURES = {
     "dpep_workspace_create": (_I, (_Z, ctypes.POINTER(_P))),
     "dpep_workspace_destroy": (_I, (_P,)),
     "dpep_workspace_capacity": (_I, (_P, ctypes.POINTER(_Z))),
+    "dpep_workspace_tune": (_I, (_P, ctypes.c_char_p, ctypes.c_longlong)),
     "dpep_layout_workspace_bytes": (_Z, (_I, _I, _I)),
     "dpep_layout": (_I, (_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P)),
     "dpep_layout_wait": (_I, (_P, _P, _I, ctypes.POINTER(ctypes.c_int32), ctypes.c_longlong)),

@@ -42,8 +42,17 @@ struct Workspace {
     uint32_t* mailbox_device;  // the same memory as the kernels address it
     uint32_t sequence;         // of the most recent layout launch
     int mailbox_local;         // its number of local experts
+    // One-launch layout: its barrier between workgroups (device memory, zero between launches), the bound of the
+    // barrier's wait in 100 MHz ticks, and two switches for tests (take two launches instead; expect more
+    // arrivals than there are workgroups, so that the wait runs out).
+    void* barrier;
+    long long barrier_ticks;
+    int barrier_extra_arrivals;
+    int layout_one_launch;
 };
-constexpr int kMailboxWords = 2 + DPEP_MAX_LOCAL_EXPERTS;
+constexpr int kMailboxTimeout = 2 + DPEP_MAX_LOCAL_EXPERTS;  // word a layout kernel sets when its barrier wait ran out
+constexpr int kMailboxWords = 3 + DPEP_MAX_LOCAL_EXPERTS;
+constexpr long long kLayoutBarrierTicks = 200000000;  // 2 s
 constexpr uint32_t kWorkspaceMagic = 0x44504550u;  // "DPEP"
 Workspace* as_workspace(void* ws);
 

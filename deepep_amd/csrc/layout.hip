@@ -1,16 +1,23 @@
 // Routing layout for one rank: per-expert counts, prefix sums and the stable expert-major
-// permutation of the T*K routes (a stable counting sort), without atomics that would reorder rows.
+// permutation of the T*K routes (a stable counting sort); no atomic decides the order of rows.
 //
 // Observable contract (reference: tests/utils/reference.py:39-73, tests/clos/common.py:248-287,
 // tests/elastic/test_dispatch.py:538-548): rows are ordered (local expert, token, slot); every valid
 // slot gets its own row (duplicates included); invalid ids produce no row.
 //
 // Decomposition: the flat route stream is cut into chunks, one wavefront each, four per workgroup.
-//   count  : each wave histograms its chunk                    -> hist[chunk][expert]   (<= 64 KiB, L2-resident)
-//   assign : each workgroup sums the histogram columns (all chunks -> expert totals and their exclusive
-//            scan; chunks before each of its waves -> that wave's base), then every wave replays its
-//            chunk in order.  The rank of a route among equal experts inside a 64-route step comes from
-//            ballot/popcount, the carry between steps lives in LDS.  There is no separate scan launch.
+//   count  : each wave histograms its chunk in LDS (atomic adds: a count does not depend on order)
+//            -> wave_hist[chunk][expert] and the workgroup's sum block_hist[workgroup][expert]
+//   assign : each workgroup sums block_hist over the workgroups (expert totals and their exclusive scan; the
+//            workgroups before it -> its own base) and adds its waves' rows, then every wave replays its chunk in
+//            order.  Inside a 64-route step the lanes with the same expert find each other through a 64-bit
+//            mask per expert in LDS (each lane ORs its bit in, then all read the mask back): a route's row is
+//            its expert's next free row plus the number of lower lanes in the mask.  The carry between steps
+//            lives in LDS.  There is no separate scan launch.
+// Inputs whose chunks fit a wave's registers (at most kKeep steps of 64 routes) take ONE launch: the workgroups
+// (at most 65, far fewer than there are CUs, so all are resident together) count, meet at a barrier in device
+// memory, and assign from the ids they still hold.  The barrier's wait is bounded; a wait that runs out is
+// recorded in the workspace's mailbox and fails the next call on that workspace.  Larger inputs take two launches.
 #include "common.h"
 
 namespace dpep {
@@ -19,8 +26,10 @@ namespace {
 constexpr int kWaves = 4;             // wavefronts (= chunks) per workgroup
 constexpr int kThreads = kWaves * kWave;
 constexpr int kHistInts = 16384;      // chunks * padded experts never exceeds this
+constexpr int kBlockHistInts = kHistInts / kWaves + DPEP_MAX_LOCAL_EXPERTS;  // workgroups * experts, rounded up
 constexpr int kMinChunk = 256;        // routes per wavefront, lower bound (multiple of 64)
-constexpr int kPrefetch = 8;          // 64-route steps whose ids are fetched before the ordered replay
+constexpr int kPrefetch = 8;          // 64-route steps whose ids are fetched at once
+constexpr int kKeep = 16;             // 64-route steps of a chunk that the one-launch kernel holds in registers
 constexpr int kColumnBatch = 16;      // histogram loads in flight per thread
 
 __device__ __forceinline__ uint64_t lanes_below()
@@ -28,139 +37,230 @@ __device__ __forceinline__ uint64_t lanes_below()
     return (1ull << (threadIdx.x & 63)) - 1ull;
 }
 
-// Mask of lanes in this wave whose (valid) expert equals mine.  nbits = bits needed for L-1.
-__device__ __forceinline__ uint64_t match_expert(int e, bool valid, int nbits)
+// Orders this wave's LDS accesses before the call against those after it, for all its lanes.
+__device__ __forceinline__ void wave_sync()
 {
-    uint64_t mask = __ballot(valid);
-    for (int b = 0; b < nbits; ++b) {
-        const bool bit = (e >> b) & 1;
-        const uint64_t vote = __ballot(valid && bit);
-        mask &= bit ? vote : ~vote;
-    }
-    return valid ? mask : 0ull;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <typename IdxT>
-__device__ __forceinline__ int local_expert(const IdxT* __restrict__ idx, int route, int end, int num_experts,
-                                            int expert_begin, int num_local)
+// Local expert of a raw id, -1 if the route is past `end` or its expert is not one of this rank's.
+__device__ __forceinline__ int local_expert(long long e, int route, int end, int num_experts, int expert_begin,
+                                            int num_local)
 {
-    if (route >= end) return -1;
-    const long long e = static_cast<long long>(idx[route]);
-    if (e < 0 || e >= num_experts) return -1;
     const long long local = e - expert_begin;
-    return (local >= 0 && local < num_local) ? static_cast<int>(local) : -1;
+    const bool valid = route < end && e >= 0 && e < num_experts && local >= 0 && local < num_local;
+    return valid ? static_cast<int>(local) : -1;
+}
+
+// Local experts of kSteps consecutive 64-route steps from `base` on.  All loads are issued before the first is
+// used (a route past the end reads the last id instead of branching around the load), so that the wave pays
+// one memory latency for the batch, not one per step.  Needs n_routes > 0.
+template <int kSteps, typename IdxT>
+__device__ __forceinline__ void fetch_experts(int (&experts)[kSteps], const IdxT* __restrict__ idx, int base, int end,
+                                              int n_routes, int num_experts, int expert_begin, int num_local)
+{
+    const int lane = threadIdx.x & 63;
+    IdxT raw[kSteps];
+#pragma unroll
+    for (int i = 0; i < kSteps; ++i) raw[i] = idx[min(base + i * kWave + lane, n_routes - 1)];
+#pragma unroll
+    for (int i = 0; i < kSteps; ++i)
+        experts[i] = local_expert(static_cast<long long>(raw[i]), base + i * kWave + lane, end, num_experts, expert_begin,
+                                  num_local);
+}
+
+// LDS of one workgroup.  running[w][e]: wave w's histogram, later its next free row of expert e; match[w][e]: bit
+// per lane of wave w whose route in the current step goes to expert e (all zero between steps); totals[e]: rows
+// of expert e.
+struct LayoutLds {
+    int totals[DPEP_MAX_LOCAL_EXPERTS];
+    int running[kWaves][DPEP_MAX_LOCAL_EXPERTS];
+    unsigned long long match[kWaves][DPEP_MAX_LOCAL_EXPERTS];
+    int partial[kThreads * 2];
+    int wave_sums[kWaves];
+};
+
+// kCoherent: the access goes past the caches (in the one-launch kernel other CUs read what this one has just written).
+template <bool kCoherent>
+__device__ __forceinline__ void store_int(int* dst, int value)
+{
+    if (kCoherent) __hip_atomic_store(dst, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *dst = value;
+}
+template <bool kCoherent>
+__device__ __forceinline__ int load_int(const int* src)
+{
+    return kCoherent ? __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *src;
+}
+
+__device__ __forceinline__ void clear_wave_lds(LayoutLds& lds, int num_local)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int e = lane; e < num_local; e += kWave) {
+        lds.running[wave][e] = 0;
+        lds.match[wave][e] = 0ull;
+    }
+    wave_sync();
+}
+
+__device__ __forceinline__ void count_step(int e, int* __restrict__ mine)
+{
+    if (e >= 0) __hip_atomic_fetch_add(mine + e, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+}
+
+// The waves' histograms (lds.running) out to wave_hist, and their sum to block_hist.  Called by all threads.
+template <bool kCoherent>
+__device__ __forceinline__ void publish_histograms(LayoutLds& lds, int num_local, int num_chunks,
+                                                   int* __restrict__ wave_hist, int* __restrict__ block_hist)
+{
+    __syncthreads();
+    for (int e = threadIdx.x; e < num_local; e += kThreads) {
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const int g = blockIdx.x * kWaves + w;
+            const int count = lds.running[w][e];
+            sum += count;
+            if (g < num_chunks) store_int<kCoherent>(wave_hist + static_cast<size_t>(g) * num_local + e, count);
+        }
+        store_int<kCoherent>(block_hist + static_cast<size_t>(blockIdx.x) * num_local + e, sum);
+    }
+}
+
+// One 64-route step of the ordered replay.
+__device__ __forceinline__ void assign_step(int e, int route, int end, unsigned long long* __restrict__ match,
+                                            int* __restrict__ next_row, int* __restrict__ route_to_row,
+                                            int* __restrict__ row_to_route)
+{
+    if (e >= 0)
+        __hip_atomic_fetch_or(match + e, 1ull << (threadIdx.x & 63), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    wave_sync();
+    int row = -1, ahead = 0, group = 0;
+    if (e >= 0) {
+        const unsigned long long mask = match[e];
+        ahead = __popcll(mask & lanes_below());
+        group = __popcll(mask);
+        row = next_row[e] + ahead;
+    }
+    wave_sync();  // every lane has read its expert's mask and next row before the first lane of the group moves them
+    if (e >= 0 && ahead == 0) {
+        next_row[e] = row + group;
+        match[e] = 0ull;
+    }
+    wave_sync();
+    if (route < end) {
+        route_to_row[route] = row;
+        if (row >= 0) row_to_route[row] = route;
+    }
 }
 
 template <typename IdxT>
 __global__ __launch_bounds__(kThreads) void layout_count_kernel(const IdxT* __restrict__ idx, int n_routes,
                                                                 int num_experts, int expert_begin, int num_local,
-                                                                int nbits, int chunk, int num_chunks,
-                                                                int* __restrict__ hist)
+                                                                int chunk, int num_chunks, int* __restrict__ wave_hist,
+                                                                int* __restrict__ block_hist)
 {
-    extern __shared__ int lds[];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __shared__ LayoutLds lds;
+    const int wave = threadIdx.x >> 6;
     const int g = blockIdx.x * kWaves + wave;
-    if (g >= num_chunks) return;
-    int* mine = lds + wave * num_local;
-    for (int e = lane; e < num_local; e += kWave) mine[e] = 0;
-    __builtin_amdgcn_wave_barrier();
-    const int begin = g * chunk;
-    const int end = min(begin + chunk, n_routes);
+    const int begin = g < num_chunks ? g * chunk : 0;
+    const int end = g < num_chunks ? min(begin + chunk, n_routes) : 0;
+    clear_wave_lds(lds, num_local);
     for (int base = begin; base < end; base += kPrefetch * kWave) {
         int experts[kPrefetch];
+        fetch_experts(experts, idx, base, end, n_routes, num_experts, expert_begin, num_local);
 #pragma unroll
-        for (int i = 0; i < kPrefetch; ++i)
-            experts[i] = local_expert(idx, base + i * kWave + lane, end, num_experts, expert_begin, num_local);
-#pragma unroll
-        for (int i = 0; i < kPrefetch; ++i) {
-            const int e = experts[i];
-            const uint64_t mask = match_expert(e, e >= 0, nbits);
-            if (e >= 0 && (mask & lanes_below()) == 0) mine[e] += __popcll(mask);
-            __builtin_amdgcn_wave_barrier();
-        }
+        for (int i = 0; i < kPrefetch; ++i) count_step(experts[i], lds.running[wave]);
     }
-    int* out = hist + static_cast<size_t>(g) * num_local;
-    for (int e = lane; e < num_local; e += kWave) out[e] = mine[e];
+    publish_histograms<false>(lds, num_local, num_chunks, wave_hist, block_hist);
 }
 
-// Column sums of hist for one expert over the chunks {first, first+stride, ...}: the total, and for
-// each wave w of this workgroup the part that lies in chunks before chunk0 + w.
+// For one expert, over the workgroups {first, first+stride, ...}: the sum of all block_hist rows and of those
+// of workgroups before this one.
 struct ColumnSums {
     int total;
-    int before[kWaves];
+    int before;
 };
 
-__device__ __forceinline__ ColumnSums column_sums(const int* __restrict__ hist, int num_local, int e, int first,
-                                                  int stride, int num_chunks, int chunk0)
+template <bool kCoherent>
+__device__ __forceinline__ ColumnSums column_sums(const int* __restrict__ block_hist, int num_local, int e, int first,
+                                                  int stride, int num_blocks)
 {
-    ColumnSums sums;
-    sums.total = 0;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) sums.before[w] = 0;
-    for (int c0 = first; c0 < num_chunks; c0 += kColumnBatch * stride) {
+    ColumnSums sums = {0, 0};
+    for (int b0 = first; b0 < num_blocks; b0 += kColumnBatch * stride) {
         int v[kColumnBatch];
 #pragma unroll
         for (int j = 0; j < kColumnBatch; ++j) {
-            const int c = c0 + j * stride;
-            v[j] = c < num_chunks ? hist[static_cast<size_t>(c) * num_local + e] : 0;
+            const int b = b0 + j * stride;
+            v[j] = b < num_blocks ? load_int<kCoherent>(block_hist + static_cast<size_t>(b) * num_local + e) : 0;
         }
 #pragma unroll
         for (int j = 0; j < kColumnBatch; ++j) {
-            const int c = c0 + j * stride;
             sums.total += v[j];
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) sums.before[w] += c < chunk0 + w ? v[j] : 0;
+            sums.before += b0 + j * stride < static_cast<int>(blockIdx.x) ? v[j] : 0;
         }
     }
     return sums;
 }
 
-template <typename IdxT>
-__global__ __launch_bounds__(kThreads) void layout_assign_kernel(
-    const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int padded_local,
-    int nbits, int chunk, int num_chunks, const int* __restrict__ hist, int* __restrict__ counts,
-    int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows, int* __restrict__ route_to_row,
-    int* __restrict__ row_to_route, uint32_t* __restrict__ mailbox, uint32_t sequence)
+// From the histograms to every wave's first row per expert (lds.running).  The launch's last workgroup owns no
+// chunk: it is the reporter, which writes the per-expert outputs and reports to the host, so that the wait for the
+// host stores (a PCIe round trip) delays no workgroup that still has routes to assign.  Called by all threads.
+// num_blocks = workgroups that own chunks.  kCoherent: the histograms were written by other CUs of this launch.
+template <bool kCoherent>
+__device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restrict__ wave_hist,
+                                             const int* __restrict__ block_hist, int num_local, int padded_local,
+                                             int num_chunks, int num_blocks, int* __restrict__ counts,
+                                             int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows,
+                                             uint32_t* __restrict__ mailbox, uint32_t sequence)
 {
-    // totals[e]: rows of expert e (later its exclusive offset); running[w][e]: next row of expert e for wave w.
-    __shared__ int totals[DPEP_MAX_LOCAL_EXPERTS];
-    __shared__ int running[kWaves][DPEP_MAX_LOCAL_EXPERTS];
-    __shared__ int partial[kThreads * (kWaves + 1)];
-    __shared__ int wave_sums[kWaves];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int chunk0 = blockIdx.x * kWaves;
-
+    const bool reporter = blockIdx.x == gridDim.x - 1;
+    // This workgroup's own rows are asked for before the column sums, so that all loads are in flight together.
+    auto own_rows = [&](int e, int (&own)[kWaves]) {
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const int g = blockIdx.x * kWaves + w;
+            own[w] = g < num_chunks ? load_int<kCoherent>(wave_hist + static_cast<size_t>(g) * num_local + e) : 0;
+        }
+    };
+    auto finish = [&](int e, int total, int before, const int (&own)[kWaves]) {  // the waves one after the other
+        lds.totals[e] = total;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            lds.running[w][e] = before;
+            before += own[w];
+        }
+    };
     if (padded_local >= kThreads) {
         for (int e = tid; e < num_local; e += kThreads) {
-            const ColumnSums sums = column_sums(hist, num_local, e, 0, 1, num_chunks, chunk0);
-            totals[e] = sums.total;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) running[w][e] = sums.before[w];
+            int own[kWaves];
+            own_rows(e, own);
+            const ColumnSums sums = column_sums<kCoherent>(block_hist, num_local, e, 0, 1, num_blocks);
+            finish(e, sums.total, sums.before, own);
         }
     } else {
-        // Few experts: split the chunks over `parts` thread groups (at most 16), then reduce through LDS.
+        // Few experts: split the workgroups' rows over `parts` thread groups (at most 16), then reduce through LDS.
         int parts = kThreads / padded_local;
         if (parts > 16) parts = 16;
         const int p = tid / padded_local, e = tid % padded_local;
-        const bool active = p < parts && e < num_local;
-        if (active) {
-            const ColumnSums sums = column_sums(hist, num_local, e, p, parts, num_chunks, chunk0);
-            partial[tid * (kWaves + 1)] = sums.total;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) partial[tid * (kWaves + 1) + 1 + w] = sums.before[w];
+        int own[kWaves] = {0, 0, 0, 0};
+        if (tid < num_local) own_rows(tid, own);
+        if (p < parts && e < num_local) {
+            const ColumnSums sums = column_sums<kCoherent>(block_hist, num_local, e, p, parts, num_blocks);
+            lds.partial[tid * 2] = sums.total;
+            lds.partial[tid * 2 + 1] = sums.before;
         }
         __syncthreads();
         if (tid < num_local) {
-            int total = 0, before[kWaves] = {0, 0, 0, 0};
+            int total = 0, before = 0;
             for (int q = 0; q < parts; ++q) {
-                const int* src = partial + (q * padded_local + tid) * (kWaves + 1);
-                total += src[0];
-#pragma unroll
-                for (int w = 0; w < kWaves; ++w) before[w] += src[1 + w];
+                total += lds.partial[(q * padded_local + tid) * 2];
+                before += lds.partial[(q * padded_local + tid) * 2 + 1];
             }
-            totals[tid] = total;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) running[w][tid] = before[w];
+            finish(tid, total, before, own);
         }
     }
     __syncthreads();
@@ -170,7 +270,7 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int e = tid * 4 + j;
-        mine[j] = e < num_local ? totals[e] : 0;
+        mine[j] = e < num_local ? lds.totals[e] : 0;
         local_sum += mine[j];
     }
     int incl = local_sum;
@@ -179,65 +279,162 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
         const int up = __shfl_up(incl, d);
         if (lane >= d) incl += up;
     }
-    if (lane == kWave - 1) wave_sums[wave] = incl;
+    if (lane == kWave - 1) lds.wave_sums[wave] = incl;
     __syncthreads();
     int offset = incl - local_sum;
-    for (int w = 0; w < wave; ++w) offset += wave_sums[w];
+    for (int w = 0; w < wave; ++w) offset += lds.wave_sums[w];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int e = tid * 4 + j;
         if (e < num_local) {
 #pragma unroll
-            for (int w = 0; w < kWaves; ++w) running[w][e] += offset;
-            if (blockIdx.x == 0) {
+            for (int w = 0; w < kWaves; ++w) lds.running[w][e] += offset;
+            if (reporter) {
                 counts[e] = mine[j];
-                if (mailbox != nullptr) mailbox[2 + e] = static_cast<uint32_t>(mine[j]);  // pinned host memory
+                if (mailbox != nullptr)  // pinned host memory, written through every cache
+                    __hip_atomic_store(mailbox + 2 + e, static_cast<uint32_t>(mine[j]), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_SYSTEM);
                 psum[e] = offset + mine[j];
                 offsets[e + 1] = offset + mine[j];
             }
         }
         offset += mine[j];
     }
-    if (blockIdx.x == 0 && tid == kThreads - 1) {
+    if (reporter && tid == kThreads - 1) {
         offsets[0] = 0;
         num_rows[0] = offset;
     }
     // The host polls the mailbox's sequence word: publish it (with the row count, one 8-byte store) after
-    // every per-expert count of this workgroup has reached host memory.
-    if (blockIdx.x == 0 && mailbox != nullptr) __threadfence_system();
+    // every per-expert count of this workgroup has reached host memory.  The counts went out as write-through
+    // stores, so each thread only has to wait until its own are acknowledged: no cache needs writing back, which
+    // is what a system-scope release fence would spend microseconds on after a kernel that left the L2 dirty.
+    if (reporter && mailbox != nullptr) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (blockIdx.x == 0 && mailbox != nullptr && tid == kThreads - 1) {
+    if (reporter && mailbox != nullptr && tid == kThreads - 1) {
         const unsigned long long word = (static_cast<unsigned long long>(sequence) << 32) | static_cast<uint32_t>(offset);
-        __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), word, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
+}
 
-    const int g = chunk0 + wave;
-    if (g >= num_chunks) return;
-    int* next_row = running[wave];
-    const int begin = g * chunk;
-    const int end = min(begin + chunk, n_routes);
+template <typename IdxT>
+__global__ __launch_bounds__(kThreads) void layout_assign_kernel(
+    const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int padded_local,
+    int chunk, int num_chunks, const int* __restrict__ wave_hist, const int* __restrict__ block_hist,
+    int* __restrict__ counts, int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows,
+    int* __restrict__ route_to_row, int* __restrict__ row_to_route, uint32_t* __restrict__ mailbox, uint32_t sequence)
+{
+    __shared__ LayoutLds lds;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int g = blockIdx.x * kWaves + wave;
+    const int begin = g < num_chunks ? g * chunk : 0;
+    const int end = g < num_chunks ? min(begin + chunk, n_routes) : 0;
+    int experts[kPrefetch];  // the first ids travel while the histograms are summed
+    if (begin < end) fetch_experts(experts, idx, begin, end, n_routes, num_experts, expert_begin, num_local);
+    clear_wave_lds(lds, num_local);
+    __syncthreads();  // expert_bases writes the rows of all waves
+    expert_bases<false>(lds, wave_hist, block_hist, num_local, padded_local, num_chunks, gridDim.x - 1, counts, psum,
+                        offsets, num_rows, mailbox, sequence);
     for (int base = begin; base < end; base += kPrefetch * kWave) {
-        int experts[kPrefetch];
+        if (base != begin) fetch_experts(experts, idx, base, end, n_routes, num_experts, expert_begin, num_local);
 #pragma unroll
         for (int i = 0; i < kPrefetch; ++i)
-            experts[i] = local_expert(idx, base + i * kWave + lane, end, num_experts, expert_begin, num_local);
-#pragma unroll
-        for (int i = 0; i < kPrefetch; ++i) {
-            const int route = base + i * kWave + lane;
-            const int e = experts[i];
-            const uint64_t mask = match_expert(e, e >= 0, nbits);
-            const int ahead = __popcll(mask & lanes_below());
-            int row = -1;
-            if (e >= 0) row = next_row[e] + ahead;
-            __builtin_amdgcn_wave_barrier();
-            if (e >= 0 && ahead == 0) next_row[e] = row + __popcll(mask);
-            __builtin_amdgcn_wave_barrier();
-            if (route < end) {
-                route_to_row[route] = row;
-                if (row >= 0) row_to_route[row] = route;
+            assign_step(experts[i], base + i * kWave + lane, end, lds.match[wave], lds.running[wave], route_to_row,
+                        row_to_route);
+    }
+}
+
+// Barrier of the one-launch kernel, in device memory, all zero between launches.
+struct GridBarrier {
+    unsigned arrived;
+    unsigned departed;
+};
+
+// All threads call it.  Returns false if the wait ran out (the other workgroups did not all arrive in time).
+// What the workgroups exchange (the histograms) is written and read with device-scope accesses that go past
+// the per-CU and per-XCD caches, so the barrier only has to order them: every thread waits until its own stores are
+// acknowledged before its workgroup's arrival is counted.  Acquire/release fences here would write back and
+// invalidate whole caches, which costs more than the launch this barrier saves.
+__device__ __forceinline__ bool grid_arrive_and_wait(GridBarrier* bar, unsigned needed, long long limit_ticks, int* verdict)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned seen = __hip_atomic_fetch_add(&bar->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+        const long long start = wall_clock64();
+        bool in_time = true;
+        while (seen < needed) {
+            __builtin_amdgcn_s_sleep(1);
+            if (wall_clock64() - start > limit_ticks) {
+                in_time = false;
+                break;
             }
+            seen = __hip_atomic_load(&bar->arrived, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        *verdict = in_time;
+    }
+    __syncthreads();
+    return *verdict != 0;
+}
+
+// The last workgroup to leave clears the barrier for the next launch: by then none is waiting on it any more.
+__device__ __forceinline__ void grid_depart(GridBarrier* bar)
+{
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned left = __hip_atomic_fetch_add(&bar->departed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == gridDim.x - 1) {
+            __hip_atomic_store(&bar->arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&bar->departed, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
+}
+
+#ifdef DPEP_DEBUG_TIMING
+__device__ unsigned long long g_layout_times[8];
+#define DPEP_LAYOUT_STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) g_layout_times[i] = wall_clock64(); } while (0)
+#else
+#define DPEP_LAYOUT_STAMP(i) do { } while (0)
+#endif
+
+// Count, barrier, assign in one launch; every wave keeps the ids of its chunk (at most kKeep steps) in registers.
+// `needed` is the number of workgroups (the reporter included), `limit_ticks` the bound of the wait (100 MHz ticks).
+template <typename IdxT>
+__global__ __launch_bounds__(kThreads) void layout_fused_kernel(
+    const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int padded_local,
+    int chunk, int num_chunks, int* __restrict__ wave_hist, int* __restrict__ block_hist, int* __restrict__ counts,
+    int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows, int* __restrict__ route_to_row,
+    int* __restrict__ row_to_route, uint32_t* __restrict__ mailbox, uint32_t sequence, GridBarrier* __restrict__ bar,
+    unsigned needed, long long limit_ticks, uint32_t* __restrict__ timeouts)
+{
+    __shared__ LayoutLds lds;
+    __shared__ int verdict;
+    DPEP_LAYOUT_STAMP(0);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int g = blockIdx.x * kWaves + wave;
+    const int begin = g < num_chunks ? g * chunk : 0;
+    const int end = g < num_chunks ? min(begin + chunk, n_routes) : 0;
+    int experts[kKeep];
+    fetch_experts(experts, idx, begin, end, n_routes, num_experts, expert_begin, num_local);
+    clear_wave_lds(lds, num_local);
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) count_step(experts[i], lds.running[wave]);
+    DPEP_LAYOUT_STAMP(1);
+    publish_histograms<true>(lds, num_local, num_chunks, wave_hist, block_hist);
+    DPEP_LAYOUT_STAMP(2);
+    if (!grid_arrive_and_wait(bar, needed, limit_ticks, &verdict) && threadIdx.x == 0)
+        __hip_atomic_store(timeouts, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);  // this launch's results are not valid
+    DPEP_LAYOUT_STAMP(3);
+    expert_bases<true>(lds, wave_hist, block_hist, num_local, padded_local, num_chunks, gridDim.x - 1, counts, psum, offsets,
+                       num_rows, mailbox, sequence);
+    DPEP_LAYOUT_STAMP(4);
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i)
+        if (begin + i * kWave < end)
+            assign_step(experts[i], begin + i * kWave + lane, end, lds.match[wave], lds.running[wave], route_to_row,
+                        row_to_route);
+    DPEP_LAYOUT_STAMP(5);
+    grid_depart(bar);
+    DPEP_LAYOUT_STAMP(6);
 }
 
 int padded_experts(int num_local)
@@ -275,28 +472,38 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
     DPEP_REQUIRE(n_routes == 0 || (idx && route_to_row && row_to_route), "layout: NULL routing buffer");
     const size_t need = dpep_layout_workspace_bytes(num_tokens, num_topk, num_local);
     DPEP_REQUIRE(need <= w->bytes, "layout: workspace too small (%zu needed, %zu available)", need, w->bytes);
+    if (w->mailbox_host[kMailboxTimeout] != 0)
+        return fail(DPEP_ERUNTIME, "layout: an earlier layout kernel on this workspace ran out of time at its barrier; "
+                                   "its results were not valid and the workspace must be replaced");
     const int padded = padded_experts(num_local);
     const int chunk = chunk_routes(n_routes, padded);
     const int num_chunks = (n_routes + chunk - 1) / chunk;
-    int nbits = 0;
-    while ((1 << nbits) < num_local) ++nbits;
-    int* hist = static_cast<int*>(w->base);
+    int* wave_hist = static_cast<int*>(w->base);
+    int* block_hist = wave_hist + kHistInts;
     const int blocks = (num_chunks + kWaves - 1) / kWaves;
-    if (blocks > 0) {
-        hipLaunchKernelGGL(layout_count_kernel<IdxT>, dim3(blocks), dim3(kThreads),
-                           static_cast<size_t>(kWaves) * num_local * sizeof(int), stream, idx, n_routes, num_experts,
-                           expert_begin, num_local, nbits, chunk, num_chunks, hist);
-        if (int rc = launch_status("layout_count")) return rc;
-    }
-    // With no routes one workgroup still publishes the all-zero counts and prefix sums.
     if (report_to_host) {
         w->sequence = w->sequence == 0xffffffffu ? 1u : w->sequence + 1u;  // never 0: that is "nothing launched"
         w->mailbox_local = num_local;
     }
-    hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks > 0 ? blocks : 1), dim3(kThreads), 0, stream, idx,
-                       n_routes, num_experts, expert_begin, num_local, padded, nbits, chunk, num_chunks, hist, counts,
-                       psum, offsets, num_rows, route_to_row, row_to_route, report_to_host ? w->mailbox_device : nullptr,
-                       w->sequence);
+    uint32_t* mailbox = report_to_host ? w->mailbox_device : nullptr;
+    if (blocks > 0 && chunk <= kKeep * kWave && w->layout_one_launch) {
+        hipLaunchKernelGGL(layout_fused_kernel<IdxT>, dim3(blocks + 1), dim3(kThreads), 0, stream, idx, n_routes, num_experts,
+                           expert_begin, num_local, padded, chunk, num_chunks, wave_hist, block_hist, counts, psum, offsets,
+                           num_rows, route_to_row, row_to_route, mailbox, w->sequence,
+                           static_cast<GridBarrier*>(w->barrier), static_cast<unsigned>(blocks + 1 + w->barrier_extra_arrivals),
+                           w->barrier_ticks, w->mailbox_device + kMailboxTimeout);
+        return launch_status("layout_fused");
+    }
+    if (blocks > 0) {
+        hipLaunchKernelGGL(layout_count_kernel<IdxT>, dim3(blocks), dim3(kThreads), 0, stream, idx, n_routes, num_experts,
+                           expert_begin, num_local, chunk, num_chunks, wave_hist, block_hist);
+        if (int rc = launch_status("layout_count")) return rc;
+    }
+    // One workgroup more than there are chunks to assign: the reporter (with no routes, it alone publishes the
+    // all-zero counts and prefix sums).
+    hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks + 1), dim3(kThreads), 0, stream, idx,
+                       n_routes, num_experts, expert_begin, num_local, padded, chunk, num_chunks, wave_hist, block_hist, counts,
+                       psum, offsets, num_rows, route_to_row, row_to_route, mailbox, w->sequence);
     return launch_status("layout_assign");
 }
 
@@ -315,10 +522,17 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
 
 extern "C" {
 
+#ifdef DPEP_DEBUG_TIMING
+int dpep_debug_layout_times(unsigned long long* host8)
+{
+    return hipMemcpyFromSymbol(host8, HIP_SYMBOL(dpep::g_layout_times), 8 * sizeof(unsigned long long)) == hipSuccess ? 0 : -2;
+}
+#endif
+
 size_t dpep_layout_workspace_bytes(int num_tokens, int num_topk, int num_local_experts)
 {
     if (num_tokens < 0 || num_topk < 1 || num_local_experts < 1) return 0;
-    return static_cast<size_t>(dpep::kHistInts) * sizeof(int);
+    return static_cast<size_t>(dpep::kHistInts + dpep::kBlockHistInts) * sizeof(int);
 }
 
 int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk, int num_experts, int expert_begin,

@@ -40,7 +40,12 @@ int dpep_workspace_create(size_t bytes, void** ws)
     DPEP_REQUIRE(bytes > 0, "workspace_create: bytes must be positive");
     *ws = nullptr;
     void* base = nullptr;
-    DPEP_HIP(hipMalloc(&base, bytes));
+    const size_t barrier_at = (bytes + 255) / 256 * 256;  // the layout's barrier words follow the caller's bytes
+    DPEP_HIP(hipMalloc(&base, barrier_at + 256));
+    if (hipError_t cleared = hipMemset(static_cast<char*>(base) + barrier_at, 0, 256); cleared != hipSuccess) {
+        (void)hipFree(base);
+        return dpep::fail(DPEP_ERUNTIME, "workspace_create: %s", hipGetErrorString(cleared));
+    }
     dpep::Workspace* w = static_cast<dpep::Workspace*>(malloc(sizeof(dpep::Workspace)));
     if (w == nullptr) {
         (void)hipFree(base);
@@ -64,6 +69,10 @@ int dpep_workspace_create(size_t bytes, void** ws)
     w->mailbox_device = static_cast<uint32_t*>(mailbox_device);
     w->sequence = 0;
     w->mailbox_local = 0;
+    w->barrier = static_cast<char*>(base) + barrier_at;
+    w->barrier_ticks = dpep::kLayoutBarrierTicks;
+    w->barrier_extra_arrivals = 0;
+    w->layout_one_launch = 1;
     *ws = w;
     return DPEP_OK;
 }
@@ -103,9 +112,30 @@ int dpep_layout_wait(void* ws, int32_t* counts_host, int num_local, int32_t* num
         __builtin_ia32_pause();
     }
     __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    if (box[dpep::kMailboxTimeout] != 0)
+        return dpep::fail(DPEP_ERUNTIME, "layout_wait: the layout kernel ran out of time at its barrier between "
+                                         "workgroups; its results are not valid and the workspace must be replaced");
     *num_rows_host = static_cast<int32_t>(box[0]);
     if (counts_host != nullptr)
         for (int e = 0; e < num_local; ++e) counts_host[e] = static_cast<int32_t>(box[2 + e]);
+    return DPEP_OK;
+}
+
+int dpep_workspace_tune(void* ws, const char* key, long long value)
+{
+    dpep::Workspace* w = dpep::as_workspace(ws);
+    DPEP_REQUIRE(w != nullptr && key != nullptr, "workspace_tune: not a live workspace");
+    if (strcmp(key, "layout_one_launch") == 0) {
+        w->layout_one_launch = value != 0;
+    } else if (strcmp(key, "layout_barrier_ticks") == 0) {
+        DPEP_REQUIRE(value > 0, "workspace_tune: layout_barrier_ticks must be positive");
+        w->barrier_ticks = value;
+    } else if (strcmp(key, "layout_barrier_extra_arrivals") == 0) {
+        DPEP_REQUIRE(value >= 0 && value <= 1, "workspace_tune: layout_barrier_extra_arrivals is 0 or 1");
+        w->barrier_extra_arrivals = static_cast<int>(value);
+    } else {
+        return dpep::fail(DPEP_EINVAL, "workspace_tune: unknown key '%s'", key);
+    }
     return DPEP_OK;
 }
 

@@ -87,6 +87,10 @@ class Workspace:
     def closed(self) -> bool:
         return self._handle is None
 
+    def tune(self, key: str, value: int) -> None:
+        """Test and diagnosis switches of the native workspace (``dpep_workspace_tune``)."""
+        _lib.check(self._lib.dpep_workspace_tune(self.handle, key.encode(), int(value)), "workspace_tune")
+
     def destroy(self) -> None:
         if self._handle is not None:
             handle, self._handle = self._handle, None

@@ -39,6 +39,14 @@ int dpep_version(void);
 int dpep_workspace_create(size_t bytes, void** ws);
 int dpep_workspace_destroy(void* ws);
 int dpep_workspace_capacity(void* ws, size_t* bytes);
+/* Switches of a workspace for tests and diagnosis; no counterpart in the reference.  Keys:
+ *   "layout_one_launch"             0: dpep_layout always takes two launches (count, assign); 1 (default): one
+ *                                   launch with a barrier between its workgroups where the input is small enough
+ *   "layout_barrier_ticks"          bound of that barrier's wait in 10 ns ticks (default 2 s)
+ *   "layout_barrier_extra_arrivals" 1: the barrier expects one workgroup more than there are, so that its wait
+ *                                   runs out (exercises the error path: dpep_layout_wait and every later layout
+ *                                   on the workspace then fail with DPEP_ERUNTIME) */
+int dpep_workspace_tune(void* ws, const char* key, long long value);
 /* Scratch bytes dpep_layout needs for T*K routes and L local experts
  * (notify_layout() workspace_bytes, csrc/ops/notify.cpp:98-110). */
 size_t dpep_layout_workspace_bytes(int num_tokens, int num_topk, int num_local_experts);

@@ -60,14 +60,42 @@ LAYOUT_SHAPES = [
     (16384, 8, 384, 0, 6),
     (16384, 8, 384, 378, 6),
     (5000, 6, 7, 2, 3),
+    (16384, 8, 256, 0, 256),  # chunks too long for the one-launch kernel's registers: always two launches
 ]
 
 
+@pytest.mark.parametrize("one_launch", [True, False])
 @pytest.mark.parametrize("tokens,topk,experts,begin,local", LAYOUT_SHAPES)
-def test_layout_matches_oracle(ops, ws, tokens, topk, experts, begin, local):
+def test_layout_matches_oracle(ops, ws, tokens, topk, experts, begin, local, one_launch):
+    """Both forms of the layout (one launch with a barrier between workgroups; count and assign launches)."""
     rng = np.random.default_rng(tokens * 31 + topk)
     idx = rng.integers(-1, experts + 1, size=(tokens, topk))  # includes -1 and == E (both invalid)
-    _check_layout(ops, ws, idx, experts, begin, local)
+    ws.tune("layout_one_launch", one_launch)
+    try:
+        _check_layout(ops, ws, idx, experts, begin, local)
+        _check_layout(ops, ws, idx[::-1].copy(), experts, begin, local)  # the barrier is clear again for the next launch
+    finally:
+        ws.tune("layout_one_launch", 1)
+
+
+def test_layout_barrier_wait_that_runs_out_is_reported(ops):
+    """The barrier's wait is bounded: told to expect one workgroup more than the launch has, with a bound of
+    100 us, every workgroup gives up, the kernel ends normally, and the host gets an error instead of results."""
+    workspace = ops.Workspace(1 << 20)
+    try:
+        idx = torch.randint(0, 16, (512, 4), device="cuda")
+        workspace.tune("layout_barrier_extra_arrivals", 1)
+        workspace.tune("layout_barrier_ticks", 10_000)
+        ops.layout(workspace, idx, 16)
+        with pytest.raises(RuntimeError, match="barrier"):
+            ops.layout_wait(workspace)
+        torch.cuda.synchronize()
+        with pytest.raises(RuntimeError, match="barrier"):  # the workspace stays marked
+            ops.layout(workspace, idx, 16)
+        with pytest.raises(ValueError, match="unknown key"):
+            workspace.tune("no_such_switch", 1)
+    finally:
+        workspace.destroy()
 
 
 def test_layout_skew_duplicates_and_masks(ops, ws):
