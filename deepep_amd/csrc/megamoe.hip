@@ -262,6 +262,8 @@ __device__ __forceinline__ void copy4_to_lds_unless(const void* src, uint32_t ld
 template <int kOutstanding>
 __device__ __forceinline__ void wait_copies_then_barrier()
 {
+    // (Never weaken this for a timing experiment: the gather indices of the next tile travel through LDS too, so a
+    // wave that runs ahead of a copy reads a stale index and fetches from a wild address.)
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
