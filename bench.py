@@ -279,7 +279,7 @@ def main():
             "bytes_per_step": moved,
         },
         "roofline": {
-            "kernel": "combine_kernel<0>",
+            "kernel": "combine_kernel<0, false>",
             "bound": "hbm",
             "achieved": dominant["GBps"],
             "peak": HBM_PEAK_GBS,

@@ -24,7 +24,8 @@ constexpr int kMaxThreads = DPEP_TUNE_MAX_THREADS;
 constexpr int kBatch = 8;  // rows fetched per thread before the dependent adds start
 
 // kWeights: 0 = plain sum, 1 = weight per expert row (w[row]), 2 = weight per route (w[t*K + s]).
-template <int kWeights>
+// kHalf: rows and output are IEEE half instead of BF16.
+template <int kWeights, bool kHalf = false>
 __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ row_weights, const int* __restrict__ route_to_row,
     int num_topk, int vec_per_row, int vec_per_part, int parts, u32x4* __restrict__ out,
@@ -78,8 +79,8 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
                 const float w = kWeights != 0 ? wts[s0 + j] : 1.0f;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float lo = bf16_to_f32(val[j][i] & 0xffffu);
-                    float hi = bf16_to_f32(val[j][i] >> 16);
+                    float lo = kHalf ? f16_to_f32(val[j][i] & 0xffffu) : bf16_to_f32(val[j][i] & 0xffffu);
+                    float hi = kHalf ? f16_to_f32(val[j][i] >> 16) : bf16_to_f32(val[j][i] >> 16);
                     if (kWeights != 0) {
                         lo = __fmul_rn(lo, w);
                         hi = __fmul_rn(hi, w);
@@ -91,7 +92,8 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
         }
         u32x4 packed;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) packed[i] = pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
+        for (int i = 0; i < 4; ++i)
+            packed[i] = kHalf ? pack_f16x2(acc[2 * i], acc[2 * i + 1]) : pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
         store16_nt(out + static_cast<size_t>(token) * vec_per_row + v, packed);
     }
 }
@@ -121,12 +123,12 @@ CombineGrid combine_grid(int num_tokens, int num_rows, int vec)
     return g;
 }
 
-template <int kWeights>
+template <int kWeights, bool kHalf = false>
 void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, const float* weights, const int32_t* route_to_row,
                     int num_topk, int vec, void* out, const float* return_in, float* return_out,
                     const int32_t* shared_first_row = nullptr, int num_shared = 0, int num_tokens = 0)
 {
-    hipLaunchKernelGGL(combine_kernel<kWeights>, dim3(g.blocks), dim3(g.threads), 0, stream, static_cast<const u32x4*>(y),
+    hipLaunchKernelGGL((combine_kernel<kWeights, kHalf>), dim3(g.blocks), dim3(g.threads), 0, stream, static_cast<const u32x4*>(y),
                        weights, route_to_row, num_topk, vec, g.per_part, g.parts, static_cast<u32x4*>(out), return_in,
                        return_out, shared_first_row, num_shared, num_tokens);
 }
@@ -147,29 +149,49 @@ int combine_routes(const void* y, const float* route_weights, const int32_t* rou
 
 }  // namespace dpep
 
+namespace dpep {
+namespace {
+
+template <bool kHalf>
+int combine_entry(const char* what, const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens,
+                  int num_topk, int num_rows, int hidden, void* out, const float* return_in, float* return_out, void* stream)
+{
+    DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "%s: bad T=%d K=%d", what, num_tokens,
+                 num_topk);
+    DPEP_REQUIRE(num_rows >= 0 && static_cast<long long>(num_rows) <= static_cast<long long>(num_tokens) * num_topk,
+                 "%s: num_rows=%d outside [0, T*K]", what, num_rows);
+    DPEP_REQUIRE(hidden > 0 && hidden % 8 == 0, "%s: hidden=%d must be a positive multiple of 8", what, hidden);
+    DPEP_REQUIRE((return_in == nullptr) == (return_out == nullptr), "%s: return_in and return_out go together", what);
+    if (num_tokens == 0) return DPEP_OK;
+    DPEP_REQUIRE(route_to_row != nullptr && out != nullptr && aligned16(out), "%s: NULL or misaligned buffer", what);
+    DPEP_REQUIRE(num_rows == 0 || (y != nullptr && aligned16(y)), "%s: y must be 16-byte aligned", what);
+    const int vec = hidden / 8;
+    const CombineGrid g = combine_grid(num_tokens, num_rows, vec);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (row_weights != nullptr)
+        launch_combine<1, kHalf>(g, s, y, row_weights, route_to_row, num_topk, vec, out, return_in, return_out);
+    else
+        launch_combine<0, kHalf>(g, s, y, nullptr, route_to_row, num_topk, vec, out, return_in, return_out);
+    return launch_status(what);
+}
+
+}  // namespace
+}  // namespace dpep
+
 extern "C" {
 
 int dpep_combine(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
                  int num_rows, int hidden, void* out, const float* return_in, float* return_out, void* stream)
 {
-    using namespace dpep;
-    DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "combine: bad T=%d K=%d", num_tokens,
-                 num_topk);
-    DPEP_REQUIRE(num_rows >= 0 && static_cast<long long>(num_rows) <= static_cast<long long>(num_tokens) * num_topk,
-                 "combine: num_rows=%d outside [0, T*K]", num_rows);
-    DPEP_REQUIRE(hidden > 0 && hidden % 8 == 0, "combine: hidden=%d must be a positive multiple of 8", hidden);
-    DPEP_REQUIRE((return_in == nullptr) == (return_out == nullptr), "combine: return_in and return_out go together");
-    if (num_tokens == 0) return DPEP_OK;
-    DPEP_REQUIRE(route_to_row != nullptr && out != nullptr && aligned16(out), "combine: NULL or misaligned buffer");
-    DPEP_REQUIRE(num_rows == 0 || (y != nullptr && aligned16(y)), "combine: y must be 16-byte aligned");
-    const int vec = hidden / 8;
-    const CombineGrid g = combine_grid(num_tokens, num_rows, vec);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (row_weights != nullptr)
-        launch_combine<1>(g, s, y, row_weights, route_to_row, num_topk, vec, out, return_in, return_out);
-    else
-        launch_combine<0>(g, s, y, nullptr, route_to_row, num_topk, vec, out, return_in, return_out);
-    return launch_status("combine");
+    return dpep::combine_entry<false>("combine", y, row_weights, route_to_row, num_tokens, num_topk, num_rows, hidden, out,
+                                      return_in, return_out, stream);
+}
+
+int dpep_combine_fp16(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
+                      int num_rows, int hidden, void* out, const float* return_in, float* return_out, void* stream)
+{
+    return dpep::combine_entry<true>("combine_fp16", y, row_weights, route_to_row, num_tokens, num_topk, num_rows, hidden,
+                                     out, return_in, return_out, stream);
 }
 
 }  // extern "C"

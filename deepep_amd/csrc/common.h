@@ -72,6 +72,18 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 }
 __device__ __forceinline__ uint32_t f32_to_bf16(float v) { return pack_bf16x2(v, 0.0f) & 0xffffu; }
 
+// The same pair of helpers for IEEE half (low-latency payloads): exact widening, round-to-nearest-even narrowing.
+typedef _Float16 dpep_f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float f16_to_f32(uint32_t bits16)
+{
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16)));
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
+{
+    const dpep_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, dpep_f16x2));
+}
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 

@@ -32,6 +32,10 @@ MAX_HIDDEN = 7168
 MAX_TOPK = 16
 MAX_EXPERTS = 1024
 MIN_WORKSPACE_BYTES = 2 << 20
+WORKSPACE_ALLOCATION_CAP = 64 << 20
+LOW_LATENCY_WORKSPACE_BYTES = 8 << 30
+LOW_LATENCY_WORLD_SIZES = (16, 32, 64, 128, 256)
+LOW_LATENCY_MAX_TOKENS = 256
 # Routing tensors whose (data_ptr, version) are pinned at dispatch and re-checked by every later
 # cached dispatch and combine.
 _ROUTING = ("topk_idx", "route_to_row", "weight_return_meta", "expert_totals", "psum_num_recv_tokens_per_expert")
@@ -103,6 +107,8 @@ class EPHandle:
         self.expert_totals = None         # int32 [L]: rows per local expert
         self.expert_offsets = None        # int32 [L+1]: exclusive prefix
         self.source_weights = None        # fp32 [R]: saved route weights (low-latency style handles)
+        self.send_counts = None           # int32 [E]: low-latency handles; its last entry is R
+        self.expert_recv_counts = None
         self.rank = None
         self.world_size = None
         self.num_tokens = None
@@ -136,7 +142,9 @@ class _Runtime:
         self.notify_lock = threading.RLock()
         self.notify_failed = False
         self.notify_inflight = None
-        self.workspace = native.Workspace(num_bytes, self.torch_device)
+        # `capacity` is what the caller asked for (the low-latency path insists on exactly 8 GiB, as the reference
+        # does); the HBM actually taken is bounded by what the single-GPU kernels use, the layout scratch.
+        self.workspace = native.Workspace(min(num_bytes, WORKSPACE_ALLOCATION_CAP), self.torch_device)
         self.stream = gpu_api().Stream(device=self.torch_device)
         self.closed = False
 
@@ -398,6 +406,45 @@ class ElasticBuffer:
             raise ValueError("Dispatch requires combine_only=False when constructing ElasticBuffer")
         if isinstance(handle, EPHandle) and handle.is_low_latency:
             raise NotImplementedError("Cached dispatch is not supported for LL handles")
+        if handle is None:
+            # Path selection as in the reference (elastic.py:710-746): small batches on EP16+ with weights and
+            # default options prefer the low-latency path, decided from host metadata only.
+            first = x[0] if isinstance(x, tuple) and len(x) == 2 else x
+            if isinstance(first, torch.Tensor) and first.ndim == 2:
+                capacity = (
+                    (self.num_max_tokens_per_rank or -(-first.shape[0] // runtime.world_size))
+                    if num_max_tokens_per_rank is None
+                    else num_max_tokens_per_rank
+                )
+                within_bound = type(capacity) is int and (
+                    not self.num_max_tokens_per_rank or capacity <= self.num_max_tokens_per_rank
+                )
+                ll_options = (
+                    within_bound
+                    and type(do_handle_copy) is bool
+                    and (do_cpu_sync is None or type(do_cpu_sync) is bool)
+                    and (do_expand is None or do_expand is True)
+                    and (expert_alignment is None or type(expert_alignment) is int and expert_alignment == 1)
+                    and type(num_sms) is int
+                    and num_sms == 0
+                    and type(num_qps) is int
+                    and num_qps == 0
+                    and cumulative_local_expert_recv_stats is None
+                    and previous_event is None
+                    and previous_event_before_epilogue is None
+                    and async_with_compute_stream is False
+                    and allocate_on_comm_stream is False
+                    and do_zero_padding is False
+                    and use_tma_aligned_col_major_sf is False
+                )
+                plan = self._low_latency_plan(x, topk_idx, topk_weights, num_experts, capacity) if ll_options else None
+                if plan is not None:
+                    if runtime.capacity != LOW_LATENCY_WORKSPACE_BYTES:
+                        raise ValueError(
+                            "LL dispatch requires Buffer(num_bytes=8589934592), exactly 8 GiB; "
+                            f"got {runtime.capacity} bytes for EP{runtime.world_size}"
+                        )
+                    return self._dispatch_low_latency(x, topk_idx, topk_weights, num_experts, capacity, do_handle_copy, plan)
         with runtime.notify_lock:
             if runtime.notify_failed:
                 raise RuntimeError("A previous communication launch failed; restart the distributed job")
@@ -540,6 +587,157 @@ class ElasticBuffer:
                 runtime.notify_failed = True
                 raise
 
+    def _low_latency_plan(self, x, topk_idx, topk_weights, num_experts, capacity):
+        """Host-metadata check that selects the low-latency path (elastic.py:401-450); never reads routes.
+        Returns the capacity layout's row count, or None when the call is not a low-latency one."""
+        runtime = self._runtime
+        hidden, scales = x if isinstance(x, tuple) and len(x) == 2 else (x, None)
+        if not isinstance(hidden, torch.Tensor) or hidden.ndim != 2:
+            return None
+        tokens, width = hidden.shape
+        per_rank = -(-tokens // runtime.world_size)
+        if (
+            type(capacity) is not int
+            or not 0 < per_rank <= capacity <= LOW_LATENCY_MAX_TOKENS
+            or runtime.world_size not in LOW_LATENCY_WORLD_SIZES
+            or topk_weights is None
+        ):
+            return None
+        if hidden.dtype not in (torch.bfloat16, torch.float16, torch.float8_e4m3fn):
+            return None
+        if self.use_fp8_dispatch and hidden.dtype != torch.float8_e4m3fn:
+            return None  # quantising inside the dispatch kernel is a high-throughput feature of this build
+        if not isinstance(topk_idx, torch.Tensor) or topk_idx.ndim != 2:
+            return None
+        topk = topk_idx.shape[1]
+        if type(num_experts) is not int or num_experts < runtime.world_size or num_experts % runtime.world_size:
+            return None
+        if (self.hidden and width != self.hidden) or (self.num_topk and topk != self.num_topk):
+            return None
+        if width <= 0 or (width * hidden.element_size()) % 16 or not 1 <= topk <= 32 or num_experts > MAX_EXPERTS:
+            return None
+        if hidden.dtype == torch.float8_e4m3fn:
+            if (
+                not isinstance(scales, torch.Tensor)
+                or scales.dtype not in (torch.int32, torch.float32)
+                or tuple(scales.shape) != (tokens, (width + 127) // 128)
+            ):
+                return None
+        elif scales is not None:
+            return None
+        for value, dtype, shape in (
+            (hidden, hidden.dtype, (tokens, width)),
+            (topk_idx, torch.int64, (tokens, topk)),
+            (topk_weights, torch.float32, (tokens, topk)),
+        ):
+            if not self._check_tensor(value, dtype, shape):
+                return None
+        if scales is not None and not self._check_tensor(scales, scales.dtype):
+            return None
+        return {"capacity_rows": runtime.world_size * capacity * min(topk, num_experts // runtime.world_size)}
+
+    def _dispatch_low_latency(self, x, topk_idx, topk_weights, num_experts, capacity, do_handle_copy, plan):
+        """Low-latency dispatch (elastic.py:453-564; docs/elastic.md:85-125) for one rank's share: the capacity
+        layout ``[C,H]`` with ``C = P*M*min(K, E/P)``, whose first R rows are the valid ones (expert-major), no host
+        synchronisation, payload and scales moved bit for bit (BF16, FP16, or FP8 with FP32 / packed-E8M0 int32
+        scales), and the route weights kept in the handle for the combine instead of being returned."""
+        runtime = self._runtime
+        native = runtime.native
+        hidden, scales = x if isinstance(x, tuple) else (x, None)
+        tokens, width = hidden.shape
+        topk = topk_idx.shape[1]
+        world = runtime.world_size
+        local = num_experts // world
+        begin = runtime.rank * local
+        rows = plan["capacity_rows"]
+        with runtime.notify_lock:
+            if runtime.notify_failed:
+                raise RuntimeError("A previous communication launch failed; restart the distributed job")
+            try:
+                producer = EventHandle()
+                with gpu_api().stream(runtime.stream):
+                    producer.current_stream_wait()
+                    with torch.inference_mode(False), torch.no_grad():
+                        indices = topk_idx.clone() if do_handle_copy else topk_idx
+                        layout = native.layout(runtime.workspace, indices, num_experts, begin, local)
+                    # The payload kernel does not depend on R: it is queued right behind the layout.  (Experts
+                    # repeated within a token are outside the low-latency contract; their surplus rows fall
+                    # beyond C and are dropped from the returned view, never written out of bounds.)
+                    out, out_scales, row_weights = (
+                        None if t is None else t[:rows]
+                        for t in native.dispatch_copy(
+                            hidden, scales, topk_weights, layout["route_to_row"], layout["row_to_route"], None,
+                            capacity_rows=rows,
+                        )
+                    )
+                    # send_counts[e]: rows of experts 0..e on this rank (inclusive), so that its last entry is R
+                    send_counts = torch.zeros((num_experts,), dtype=torch.int32, device=hidden.device)
+                    send_counts[begin : begin + local] = layout["psum"]
+                    send_counts[begin + local :] = layout["num_rows"]
+                    handle = EPHandle(
+                        True, num_experts, 1, capacity, 0, indices, world * capacity, rows, [], None, None, None, None,
+                        None, None, None, is_low_latency=True,
+                    )
+                    handle.route_to_row = layout["route_to_row"]
+                    handle.source_weights = row_weights
+                    handle.send_counts = send_counts
+                    handle.expert_recv_counts = None
+                    handle.metadata_only = False
+                    handle._buffer_token = self._handle_token
+                    handle.rank, handle.world_size = runtime.rank, world
+                    handle.num_tokens, handle.num_topk, handle.hidden = tokens, topk, width
+                    retained = (hidden, scales, topk_weights, indices, out, out_scales, row_weights, send_counts,
+                                layout["route_to_row"], layout["row_to_route"], layout["meta"])
+                    event = EventOverlap._from_resources(EventHandle(), retained)
+                event.current_stream_wait(release_handle=True)
+                runtime.notify_inflight = None
+                return (out, out_scales) if scales is not None else out, None, None, handle, event
+            except Exception:
+                runtime.notify_failed = True
+                raise
+
+    def _combine_low_latency(self, x, handle, topk_weights, bias, num_sms, num_qps, previous_event,
+                             previous_event_before_epilogue, async_with_compute_stream, allocate_on_comm_stream):
+        """Low-latency combine (elastic.py:566-646): weights come from the handle, output has x's dtype."""
+        runtime = self._runtime
+        if handle._buffer_token is not self._handle_token or handle.metadata_only:
+            raise ValueError("LL handle must come from this buffer's payload dispatch")
+        if topk_weights is not None or bias is not None:
+            raise NotImplementedError("LL combine takes its weights from the handle and does not support bias")
+        if (
+            type(num_sms) is not int
+            or num_sms != 0
+            or type(num_qps) is not int
+            or num_qps != 0
+            or previous_event is not None
+            or previous_event_before_epilogue is not None
+            or async_with_compute_stream is not False
+            or allocate_on_comm_stream is not False
+        ):
+            raise NotImplementedError("LL combine supports default scheduling and stream options only")
+        if not (
+            isinstance(x, torch.Tensor)
+            and x.dtype in (torch.bfloat16, torch.float16)
+            and self._check_tensor(x, x.dtype, (handle.num_expanded_tokens, handle.hidden))
+        ):
+            raise ValueError("LL combine requires contiguous BF16/FP16 expert output matching its handle")
+        with runtime.notify_lock:
+            if runtime.notify_failed:
+                raise RuntimeError("A previous communication launch failed; restart the distributed job")
+            try:
+                producer = EventHandle()
+                with gpu_api().stream(runtime.stream):
+                    producer.current_stream_wait()
+                    output, _ = runtime.native.combine(x, handle.route_to_row, handle.source_weights, None)
+                    retained = (x, output, handle.route_to_row, handle.source_weights, handle.topk_idx)
+                    event = EventOverlap._from_resources(EventHandle(), retained)
+                event.current_stream_wait(release_handle=True)
+                runtime.notify_inflight = None
+                return output, None, event
+            except Exception:
+                runtime.notify_failed = True
+                raise
+
     def _notify_launch(self, topk_idx, num_experts, do_handle_copy):
         """Queues the routing layout; returns its device outputs and the routing tensor it read."""
         runtime = self._runtime
@@ -597,6 +795,11 @@ class ElasticBuffer:
         runtime = self._live_runtime()
         runtime.ensure_alive()
         native = runtime.native
+        if isinstance(handle, EPHandle) and handle.is_low_latency and handle.send_counts is not None:
+            return self._combine_low_latency(
+                x, handle, topk_weights, bias, num_sms, num_qps, previous_event, previous_event_before_epilogue,
+                async_with_compute_stream, allocate_on_comm_stream,
+            )
         with runtime.notify_lock:
             if runtime.notify_failed:
                 raise RuntimeError("A previous communication launch failed; restart the distributed job")

@@ -148,11 +148,12 @@ def layout_wait(ws: Workspace, num_local: Optional[int] = None, timeout_s: float
     return counts, int(rows.value)
 
 
-def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows: Optional[int]):
+def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows: Optional[int],
+                  capacity_rows: Optional[int] = None):
     """out[row] = x[token(row)] (+ scale rows, + per-row weights).  x is BF16 [T,H] or FP8 [T,H].
 
     ``num_rows=None``: R is not known on the host yet (no ``layout_wait``): the outputs are allocated with T*K rows,
-    of which the first R are written; the caller narrows them once it has R."""
+    (at least ``capacity_rows``, if given), of which the first R are written; the caller narrows them."""
     lib = _lib.load()
     if not isinstance(x, torch.Tensor) or x.dtype not in (torch.bfloat16, torch.float8_e4m3fn, torch.float16):
         raise ValueError("x must be a BF16, FP16 or FP8 E4M3FN tensor")
@@ -168,7 +169,7 @@ def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows:
     row_bytes = hidden * x.element_size()
     if row_bytes % 16:
         raise ValueError("hidden row size must be a multiple of 16 bytes")
-    num_rows, known_rows = (tokens * topk, -1) if num_rows is None else (num_rows, num_rows)
+    num_rows, known_rows = (max(tokens * topk, capacity_rows or 0), -1) if num_rows is None else (num_rows, num_rows)
     scale_cols = 0
     out_scales = None
     if scales is not None:
@@ -241,9 +242,12 @@ def cast_to_fp8(x):
 
 
 def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
-    """out[t] = bf16( sum_s fp32(y[row(t,s)]) (* row_weights[row]) ); optional weight-return channel."""
+    """out[t] = round( sum_s fp32(y[row(t,s)]) (* row_weights[row]) ) in y's dtype (BF16 or FP16); optional
+    weight-return channel."""
     lib = _lib.load()
-    _require("y", y, torch.bfloat16)
+    if not isinstance(y, torch.Tensor) or y.dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError("y must be a BF16 or FP16 tensor")
+    _require("y", y, y.dtype)
     if y.ndim != 2:
         raise ValueError("y must be [R, H]")
     dev = y.device
@@ -261,11 +265,12 @@ def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
         _require("return_values", return_values, torch.float32, (rows,), dev)
         returned = torch.empty((tokens, topk), dtype=torch.float32, device=dev)
     if out is None:
-        out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+        out = torch.empty((tokens, hidden), dtype=y.dtype, device=dev)
     else:
-        _require("out", out, torch.bfloat16, (tokens, hidden), dev)
+        _require("out", out, y.dtype, (tokens, hidden), dev)
+    entry = lib.dpep_combine if y.dtype == torch.bfloat16 else lib.dpep_combine_fp16
     with _on_device(dev):
-        status = lib.dpep_combine(
+        status = entry(
             _ptr(y), _ptr(row_weights), _ptr(route_to_row), tokens, topk, rows, hidden, _ptr(out),
             _ptr(return_values), _ptr(returned), _stream(dev),
         )

@@ -117,6 +117,13 @@ int dpep_combine(const void* y, const float* row_weights, const int32_t* route_t
                  int num_topk, int num_rows, int hidden, void* out, const float* return_in,
                  float* return_out, void* stream);
 
+/* The same combine for IEEE half rows and output (the low-latency path accepts BF16 or FP16 expert outputs and
+ * returns the same dtype: deep_ep/backends/mesh_clos/elastic.py:596-606; oracle expected_combine,
+ * tests/elastic/test_ep_low_latency.py:449-463): fp32 accumulation in slot order, one RNE rounding to half. */
+int dpep_combine_fp16(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens,
+                      int num_topk, int num_rows, int hidden, void* out, const float* return_in,
+                      float* return_out, void* stream);
+
 /* MXFP8 activation quantiser, block 32 (quantize_input, experiments/megamoe/python/
  * deep_ep_experimental/megamoe/reference.py:44-54; device ComputeMxScale/QuantizeMxFp8Data).
  *   x bf16 [B,H], H % 32 == 0 -> codes e4m3 [B,H], scales e8m0 [B,H/32] */

@@ -72,6 +72,53 @@ CONFIGS = {
 }
 
 
+def ll_routes(world_size, tokens, topk, experts, seed):
+    """Routes of the low-latency system test (make_routes, tests/elastic/test_ep_low_latency.py:397-407): per
+    source rank and token, `topk` distinct experts drawn with random.Random(seed).sample."""
+    import random
+
+    rng = random.Random(seed)
+    return [[rng.sample(range(experts), topk) for _ in range(tokens)] for _ in range(world_size)]
+
+
+def ll_payload(sources, tokens, hidden):
+    """Payload rows of the same test (payload, :421-430): ((src*3 + tok*5 + col) % 17) - 8, with the first four
+    columns replaced by src//16, src%16, tok//16, tok%16 (small integers, exact in BF16, FP16 and FP8)."""
+    sources, tokens = np.asarray(sources, dtype=np.int64), np.asarray(tokens, dtype=np.int64)
+    values = ((sources[:, None] * 3 + tokens[:, None] * 5 + np.arange(hidden)[None, :]) % 17 - 8).astype(np.float32)
+    values[:, 0], values[:, 1] = sources // 16, sources % 16
+    values[:, 2], values[:, 3] = tokens // 16, tokens % 16
+    return values
+
+
+def ll_fp8_scale_bits(sources, tokens, hidden, packed_e8m0):
+    """Scale words of the same test (fp8_scales, :433-446), as int32 bit patterns [n, ceil(H/128)]: 0x7F7F7F7F
+    (four packed E8M0 ones) or FP32 values with bits 0x3F000001 + src*65536 + tok*128 + group."""
+    groups = (hidden + 127) // 128
+    sources, tokens = np.asarray(sources, dtype=np.int64), np.asarray(tokens, dtype=np.int64)
+    if packed_e8m0:
+        return np.full((len(sources), groups), 0x7F7F7F7F, dtype=np.int32)
+    return (0x3F000001 + sources[:, None] * 65536 + tokens[:, None] * 128 + np.arange(groups)[None, :]).astype(np.int32)
+
+
+def ll_expert_entries(routes, experts, world_size, rank):
+    """(source, token) pairs each local expert of `rank` receives, in source-major order (expert_entries, :410-418)."""
+    local = experts // world_size
+    entries = [[] for _ in range(local)]
+    for source, rows in enumerate(routes):
+        for token, selected in enumerate(rows):
+            for expert in selected:
+                if rank * local <= expert < (rank + 1) * local:
+                    entries[expert - rank * local].append((source, token))
+    return entries
+
+
+def ll_expert_map(values_f32, expert):
+    """What the test's stand-in expert computes before rounding to its output dtype (prepare_experts, :466-479):
+    x * ((e % 4 + 1) / 4) + (e % 3 - 1) / 8, in fp32."""
+    return (values_f32 * np.float32((expert % 4 + 1) / 4) + np.float32((expert % 3 - 1) / 8)).astype(np.float32)
+
+
 def make_inputs(name, seed=0, tokens=None, hidden=None):
     """x ~ N(0,1) BF16 [T,H]; distinct top-k ids (uniform, or Zipf(1.2) popularity sampled without
     replacement); weights = softmax of N(0,1) logits, fp32.  Returns torch CPU tensors."""

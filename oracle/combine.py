@@ -6,6 +6,8 @@ Pinned by (tests/test_oracle_combine.py):
   * the weighted low-latency fixture (tests/elastic/test_ep_low_latency.py:449-479): weights (s+1)/32,
     expert map y = x*((e%4+1)/4) + (e%3-1)/8;
   * the hand case of tests/test_reference.py:61-67 (6, 9, 20 and the weight channel);
+  * the same fixture in FP16 for combine_fp16, checked against the test's own torch formula evaluated with torch
+    half tensors (what the reference's expected_combine computes);
   * an fp64 sum (1-ulp bound) and order sensitivity: a reversed-slot sum differs on a crafted input,
     so a wrong accumulation order fails.
 """
@@ -15,6 +17,28 @@ from __future__ import annotations
 import numpy as np
 
 from .quant import bf16_bits_to_f32, f32_to_bf16_bits
+
+
+def combine_fp16(y_f16, route_to_row, row_weights=None):
+    """The same reduce for IEEE half rows (the low-latency path takes BF16 or FP16 expert outputs and returns the
+    same dtype, deep_ep/backends/mesh_clos/elastic.py:596-606; expected_combine,
+    tests/elastic/test_ep_low_latency.py:449-463): half -> fp32 exactly, separate multiply and add in fp32, slot
+    order, one RNE rounding to half (numpy's float32 -> float16 cast).  y: float16 [R, H]; returns float16 [T, H]."""
+    y = np.asarray(y_f16, dtype=np.float16)
+    r2r = np.asarray(route_to_row, dtype=np.int64)
+    acc = np.zeros((r2r.shape[0], y.shape[1]), dtype=np.float32)
+    w = None if row_weights is None else np.asarray(row_weights, dtype=np.float32)
+    for slot in range(r2r.shape[1]):
+        rows = r2r[:, slot]
+        valid = rows >= 0
+        safe = np.where(valid, rows, 0)
+        if y.shape[0] == 0:
+            continue
+        tmp = y[safe].astype(np.float32)
+        if w is not None:
+            tmp = (tmp * w[safe][:, None]).astype(np.float32)
+        acc = np.where(valid[:, None], (acc + tmp).astype(np.float32), acc)
+    return acc.astype(np.float16)
 
 
 def combine(y_bf16_bits, route_to_row, row_weights=None):

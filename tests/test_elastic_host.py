@@ -47,12 +47,12 @@ class FakeNative:
         counts, rows = self.last_layout
         return (counts if num_local is not None else None), rows
 
-    def dispatch_copy(self, x, scales, w, route_to_row, row_to_route, rows):
+    def dispatch_copy(self, x, scales, w, route_to_row, row_to_route, rows, capacity_rows=None):
         if self.fail_next:
             raise RuntimeError(self.fail_next)
         self.calls["dispatch_copy"] += 1
-        # rows=None: R not known to the caller yet; outputs hold T*K rows, the tail is left as filler
-        pad = 0 if rows is not None else route_to_row.numel() - self.last_layout[1]
+        # rows=None: R not known to the caller yet; outputs hold T*K rows (or more), the tail is left as filler
+        pad = 0 if rows is not None else max(route_to_row.numel(), capacity_rows or 0) - self.last_layout[1]
         self.calls["dispatch_at_capacity"] += rows is None
         rows = self.last_layout[1] if rows is None else rows
         route = row_to_route[:rows].long()
@@ -72,6 +72,9 @@ class FakeNative:
 
     def combine(self, y, route_to_row, row_weights=None, return_values=None):
         self.calls["combine"] += 1
+        if y.dtype == torch.float16:
+            out = ocombine.combine_fp16(y.numpy(), route_to_row.numpy(), None if row_weights is None else row_weights.numpy())
+            return torch.from_numpy(out), None
         out = ocombine.combine(_bits(y), route_to_row.numpy(), None if row_weights is None else row_weights.numpy())
         returned = None
         if return_values is not None:
@@ -92,7 +95,7 @@ def host(monkeypatch):
     monkeypatch.setattr(event, "gpu_api", lambda: gpu)
     monkeypatch.setattr(elastic, "gpu_api", lambda: gpu)
 
-    def make(world=1, rank=0, hidden=0, topk=0, bound=0, fp8=False):
+    def make(world=1, rank=0, hidden=0, topk=0, bound=0, fp8=False, num_bytes=1 << 30):
         native = FakeNative(calls)
         buffer = elastic.ElasticBuffer.__new__(elastic.ElasticBuffer)
         buffer.hidden, buffer.num_topk, buffer.num_max_tokens_per_rank = hidden, topk, bound
@@ -100,7 +103,7 @@ def host(monkeypatch):
         buffer._handle_token = object()
         buffer._runtime = SimpleNamespace(
             native=native, device=0, torch_device=torch.device("cpu"), rank=rank, world_size=world, combine_only=False,
-            capacity=1 << 30, notify_lock=threading.RLock(), notify_failed=False, notify_inflight=None,
+            capacity=num_bytes, notify_lock=threading.RLock(), notify_failed=False, notify_inflight=None,
             workspace=object(), stream=stream, closed=False, ensure_alive=lambda: None, close=lambda: None,
         )
         return buffer, native
@@ -262,3 +265,66 @@ def test_constructor_gates():
     with pytest.raises(NotImplementedError, match="Pass num_bytes"):
         elastic.ElasticBuffer(explicitly_destroy=True)
     assert elastic.ElasticBuffer.get_buffer_size_hint(None, 4096, 7168, 8) >= 2 << 20
+
+
+def test_low_latency_path_selection_and_contract(host):
+    """Small batches on EP16+ with route weights and default options take the low-latency path
+    (deep_ep/backends/mesh_clos/elastic.py:710-746): capacity layout, weights kept in the handle, FP16 accepted."""
+    from oracle import cases
+
+    make, calls = host
+    world, rank, per_rank, hidden, experts, topk = 16, 3, 4, 64, 32, 3
+    routes = cases.ll_routes(world, per_rank, topk, experts, seed=11)
+    idx = torch.tensor([row for source in routes for row in source])
+    sources, toks = np.repeat(np.arange(world), per_rank), np.tile(np.arange(per_rank), world)
+    w = ((torch.arange(topk) + 1) / 32).repeat(world * per_rank, 1).contiguous()
+    entries = cases.ll_expert_entries(routes, experts, world, rank)
+    rows = sum(len(v) for v in entries)
+    capacity_rows = world * per_rank * min(topk, experts // world)
+    for dtype in (torch.bfloat16, torch.float16):
+        buffer, _ = make(world=world, rank=rank, num_bytes=8 << 30)
+        x = torch.from_numpy(cases.ll_payload(sources, toks, hidden)).to(dtype)
+        recv, none, recv_w, handle, ev = buffer.dispatch(x, topk_idx=idx, topk_weights=w, num_experts=experts)
+        assert none is None and recv_w is None and handle.is_low_latency and calls["dispatch_at_capacity"] >= 1
+        assert recv.shape == (capacity_rows, hidden) and recv.dtype == dtype
+        assert handle.num_expanded_tokens == capacity_rows and handle.num_recv_tokens == world * per_rank
+        assert handle.num_recv_tokens_per_expert_list == [] and handle.psum_num_recv_tokens_per_expert is None
+        assert handle.num_unaligned_recv_tokens_per_expert is None and handle.expert_recv_counts is None
+        assert int(handle.send_counts[-1]) == rows and handle.send_counts.shape == (experts,)
+        start = 0
+        for block in entries:  # expert-major blocks, (source, token) order inside (tests/elastic/test_ep_low_latency.py:518-531)
+            got = recv[start : start + len(block)].float()
+            ids = [(int(r[0]) * 16 + int(r[1]), int(r[2]) * 16 + int(r[3])) for r in got]
+            assert ids == block
+            start += len(block)
+        # combine: weights from the handle, output in the experts' dtype, (out, None, event)
+        y = recv.clone()
+        y[rows:] = 0  # the capacity tail is not input: make it harmless for the CPU stand-in
+        out, out_w, _ = buffer.combine(y, handle)
+        assert out_w is None and out.dtype == dtype and out.shape == x.shape
+        local = experts // world
+        expected = torch.zeros(x.shape)
+        for t in range(idx.shape[0]):
+            for s in range(topk):
+                if rank * local <= int(idx[t, s]) < (rank + 1) * local:
+                    expected[t] += x[t].float() * ((s + 1) / 32)
+        assert torch.equal(out, expected.to(dtype))
+        with pytest.raises(NotImplementedError, match="weights from the handle"):
+            buffer.combine(y, handle, topk_weights=torch.ones(capacity_rows))
+        with pytest.raises(NotImplementedError, match="default scheduling"):
+            buffer.combine(y, handle, num_sms=64)
+        with pytest.raises(ValueError, match="matching its handle"):
+            buffer.combine(y[:-1].contiguous(), handle)
+        with pytest.raises(NotImplementedError, match="Cached dispatch is not supported for LL"):
+            buffer.dispatch(x, handle=handle)
+    # exactly 8 GiB or an error, never a silent switch to the other path (docs/elastic.md:28)
+    small, _ = make(world=world, rank=rank)
+    with pytest.raises(ValueError, match="exactly 8 GiB"):
+        small.dispatch(x.bfloat16(), topk_idx=idx, topk_weights=w, num_experts=experts)
+    # without route weights, with more than 256 tokens per rank, or below EP16 the call is a high-throughput one
+    recv, _, recv_w, handle, _ = small.dispatch(x.bfloat16(), topk_idx=idx, num_experts=experts)
+    assert not handle.is_low_latency and recv.shape[0] == rows
+    ep8, _ = make(world=8, rank=1, num_bytes=8 << 30)
+    idx8 = idx[: 8 * per_rank].contiguous()
+    _, _, _, handle, _ = ep8.dispatch(x[: 8 * per_rank].bfloat16().contiguous(), topk_idx=idx8, topk_weights=w[: 8 * per_rank].contiguous(), num_experts=experts)
+    assert not handle.is_low_latency

@@ -325,3 +325,19 @@ def test_dispatch_before_the_host_knows_the_row_count(ops, ws, name, tokens):
     np.testing.assert_array_equal(fp8_bits(early_q[0][:rows]), fp8_bits(late_q[0]))
     np.testing.assert_array_equal(f32_bits(early_q[1][:rows]), f32_bits(late_q[1]))
     np.testing.assert_array_equal(f32_bits(early_q[2][:rows]), f32_bits(late_q[2]))
+
+
+@pytest.mark.parametrize("weighted", [False, True])
+def test_combine_fp16_matches_oracle(ops, ws, weighted):
+    """IEEE half rows and output (low-latency expert outputs may be FP16): bit-exact against the half oracle,
+    including values that round differently in half and BF16 and a sum that overflows half to infinity."""
+    x, idx, w, cfg = cases.make_inputs("C2")
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"])
+    gen = torch.Generator().manual_seed(9)
+    y = (torch.randn(rows, cfg["hidden"], generator=gen) * 3).half()
+    y[0, :8] = 60000.0  # several of these in one token overflow the half range
+    w_rows = torch.from_numpy(olayout.expand_weights(w.numpy(), want["row_to_route"]))
+    out, _ = ops.combine(y.cuda(), got["route_to_row"], w_rows.cuda() if weighted else None)
+    assert out.dtype == torch.float16
+    ref = ocombine.combine_fp16(y.numpy(), want["route_to_row"], w_rows.numpy() if weighted else None)
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16))

@@ -103,3 +103,68 @@ def test_utils_cast_roundtrip():
     back = per_token_cast_back(q, s)
     q_ref, s_ref = oquant.cast_to_fp8_torch(x)
     np.testing.assert_array_equal(bf16_bits(back), oquant.cast_back(fp8_bits(q_ref), s_ref.numpy()))
+
+
+@pytest.mark.parametrize("payload", ["bfloat16", "float16", "fp8_int32_scales", "fp8_float32_scales"])
+def test_low_latency_dispatch_combine_rank_share(payload):
+    """The reference's low-latency system test (tests/elastic/test_ep_low_latency.py: routes :397-407, payload
+    :421-430, scales :433-446, dispatch checks :482-531, stand-in experts :466-479, expected combine :449-463) for
+    one EP16 rank's share: capacity layout [C,H], rows bit-exact per expert block, weights taken from the handle."""
+    import deepep_amd
+
+    world, rank, per_rank, hidden, experts, topk = 16, 5, 24, 7168, 64, 8
+    local = experts // world
+    routes = cases.ll_routes(world, per_rank, topk, experts, seed=3)
+    idx = torch.tensor([row for source in routes for row in source])
+    sources, toks = np.repeat(np.arange(world), per_rank), np.tile(np.arange(per_rank), world)
+    values = torch.from_numpy(cases.ll_payload(sources, toks, hidden))
+    w = ((torch.arange(topk) + 1) / 32).repeat(world * per_rank, 1).contiguous()
+    fp8 = payload.startswith("fp8")
+    if fp8:
+        bits = cases.ll_fp8_scale_bits(sources, toks, hidden, packed_e8m0="int32" in payload)
+        scales = torch.from_numpy(bits) if "int32" in payload else torch.from_numpy(bits).view(torch.float32)
+        x = (values.to(torch.float8_e4m3fn).cuda(), scales.cuda())
+    else:
+        x = values.to(getattr(torch, payload)).cuda()
+    entries = cases.ll_expert_entries(routes, experts, world, rank)
+    rows = sum(len(v) for v in entries)
+    capacity_rows = world * per_rank * min(topk, local)
+    buffer = deepep_amd.ElasticBuffer(None, num_bytes=8 << 30, rank=rank, world_size=world, explicitly_destroy=True)
+    try:
+        recv, none, recv_w, handle, event = buffer.dispatch(x, topk_idx=idx.cuda(), topk_weights=w.cuda(), num_experts=experts)
+        assert none is None and recv_w is None and handle.is_low_latency
+        got = recv[0] if fp8 else recv
+        assert tuple(got.shape) == (capacity_rows, hidden) and handle.num_expanded_tokens == capacity_rows
+        assert handle.num_recv_tokens == world * per_rank and handle.num_recv_tokens_per_expert_list == []
+        assert handle.psum_num_recv_tokens_per_expert is None and handle.num_unaligned_recv_tokens_per_expert is None
+        assert int(handle.send_counts[-1].item()) == rows
+        host = got.float().cpu()
+        start = 0
+        for block in entries:
+            src, tok = zip(*block) if block else ((), ())
+            want = cases.ll_payload(src, tok, hidden) if block else np.zeros((0, hidden), np.float32)
+            np.testing.assert_array_equal(host[start : start + len(block)].numpy(), want)
+            if fp8:
+                assert recv[1].dtype == x[1].dtype and tuple(recv[1].shape) == (capacity_rows, hidden // 128)
+                got_bits = recv[1][start : start + len(block)].cpu().view(torch.int32).numpy()
+                np.testing.assert_array_equal(got_bits, cases.ll_fp8_scale_bits(src, tok, hidden, "int32" in payload)) if block else None
+            start += len(block)
+        # stand-in experts on the valid rows; the capacity tail stays whatever it is
+        expert_dtype = torch.float16 if payload == "float16" else torch.bfloat16
+        y = torch.zeros((capacity_rows, hidden), dtype=expert_dtype, device="cuda")
+        row_expert = np.concatenate([[rank * local + e] * len(block) for e, block in enumerate(entries)]).astype(np.int64)
+        mapped = np.stack([cases.ll_expert_map(host[i].numpy(), int(row_expert[i])) for i in range(rows)])
+        y[:rows] = torch.from_numpy(mapped).to(expert_dtype).cuda()
+        out, out_w, _ = buffer.combine(y, handle)
+        assert out_w is None and out.dtype == expert_dtype and tuple(out.shape) == (world * per_rank, hidden)
+        lay = olayout.layout(idx.numpy(), experts, rank * local, local)
+        slot = lay["row_to_route"] % topk
+        row_w = ((slot + 1) / 32).astype(np.float32)
+        if expert_dtype == torch.float16:
+            want_out = ocombine.combine_fp16(y[:rows].cpu().numpy(), lay["route_to_row"], row_w)
+            np.testing.assert_array_equal(out.cpu().numpy().view(np.uint16), want_out.view(np.uint16))
+        else:
+            want_out = ocombine.combine(bf16_bits(y[:rows]), lay["route_to_row"], row_w)
+            np.testing.assert_array_equal(bf16_bits(out), want_out)
+    finally:
+        buffer.destroy()

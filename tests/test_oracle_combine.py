@@ -69,6 +69,44 @@ def test_reference_weighted_low_latency_fixture():
     np.testing.assert_array_equal(combine(y, lay["route_to_row"], w_rows), expected)
 
 
+def test_low_latency_fixture_in_fp16_and_its_input_recipes():
+    """combine_fp16 against the reference test's own formula evaluated in torch half (expected_combine,
+    tests/elastic/test_ep_low_latency.py:449-463), on that test's routes and payload recipes (:397-430)."""
+    import torch
+
+    from oracle.combine import combine_fp16
+
+    world, tokens, hidden, experts, topk = 4, 5, 64, 16, 3
+    routes = cases.ll_routes(world, tokens, topk, experts, seed=7)
+    assert all(len(set(row)) == topk for rank in routes for row in rank)  # distinct experts per token
+    flat = np.asarray([row for rank in routes for row in rank])
+    sources, toks = np.repeat(np.arange(world), tokens), np.tile(np.arange(tokens), world)
+    x = cases.ll_payload(sources, toks, hidden)
+    assert x[7, :4].tolist() == [0, 1, 0, 2] and x[7, 4] == (1 * 3 + 2 * 5 + 4) % 17 - 8  # identity columns + formula
+    xt = torch.from_numpy(x).half().float()
+    expected = torch.zeros_like(xt)
+    for t in range(flat.shape[0]):
+        for s in range(topk):
+            e = int(flat[t, s])
+            expected[t] += (xt[t] * ((e % 4 + 1) / 4) + (e % 3 - 1) / 8).half().float() * ((s + 1) / 32)
+    lay = layout(flat, experts)
+    route = lay["row_to_route"]
+    e, s = flat.reshape(-1)[route], route % topk
+    rows = expand_rows(xt.numpy(), route, topk)
+    y = np.stack([cases.ll_expert_map(rows[i], int(e[i])) for i in range(len(route))]).astype(np.float16)
+    got = combine_fp16(y, lay["route_to_row"], ((s + 1) / 32).astype(np.float32))
+    np.testing.assert_array_equal(got.view(np.uint16), expected.half().numpy().view(np.uint16))
+    # what each local expert of rank 1 receives, against the layout's rows for that expert range
+    entries = cases.ll_expert_entries(routes, experts, world, 1)
+    share = layout(flat, experts, 4, 4)
+    assert [len(v) for v in entries] == share["counts"].tolist()
+    first = share["row_to_route"][: len(entries[0])] // topk
+    assert [(int(t) // tokens, int(t) % tokens) for t in first] == entries[0]
+    # scale recipes: packed E8M0 ones, or FP32 words with distinct low bits
+    assert cases.ll_fp8_scale_bits([1], [2], 256, True).tolist() == [[0x7F7F7F7F] * 2]
+    assert cases.ll_fp8_scale_bits([1], [2], 256, False).tolist() == [[0x3F000001 + 65536 + 256, 0x3F000001 + 65536 + 257]]
+
+
 def test_slot_order_and_unfused_multiply_add_are_observable():
     # 2^24 + 1 - 2^24: slot order (big, one, -big) gives 0, any other order gives 1 -> order is pinned.
     big = np.float32(2.0**24)
