@@ -478,19 +478,19 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     aim_index_prefetch(next_info);
 
     // ---- fragment addresses inside a stage ---------------------------------------------------------
-    int a_addr[RT][2][2];  // [row tile][k step][lo/hi 16 bytes]
-    int sa_addr[RT];
-#pragma unroll
-    for (int i = 0; i < RT; ++i) {
-        const int row = wm * 32 * RT + i * 32 + lr;
-        const int sw = (row >> 1) & 7;
+    // Row tile i of a lane sits 32 rows = 4096 bytes below row tile 0 and has the same swizzle (32 rows is a multiple
+    // of the swizzle period), so one set of lane addresses serves all row tiles with compile-time offsets.
+    int a_addr[2][2];  // [k step][lo/hi 16 bytes] of row tile 0
+    const int row_in_wave = wm * 32 * RT + lr;
+    {
+        const int sw = (row_in_wave >> 1) & 7;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            a_addr[i][kb][0] = Cfg::kOffA + row * kBK + (((kb * 4 + g) ^ sw) << 4);
-            a_addr[i][kb][1] = Cfg::kOffA + row * kBK + (((kb * 4 + 2 + g) ^ sw) << 4);
+            a_addr[kb][0] = Cfg::kOffA + row_in_wave * kBK + (((kb * 4 + g) ^ sw) << 4);
+            a_addr[kb][1] = Cfg::kOffA + row_in_wave * kBK + (((kb * 4 + 2 + g) ^ sw) << 4);
         }
-        sa_addr[i] = Cfg::kOffRowScales + row * 16;
     }
+    const int sa_addr = Cfg::kOffRowScales + row_in_wave * 16;  // row tile i: + i * 512
     const int b_addr = Cfg::kOffB + wn * kCT * 2048 + lane * 16;
     const int sb_addr = Cfg::kOffColScales + wn * kCT * 512 + lane * 8;
 
@@ -505,8 +505,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         const uint8_t* stage = lds + stage_index * kStageBytes;
         if (group < RT) {
             const int i = group;
-            const u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][0]);
-            const u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[i][kb][1]);
+            const u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[kb][0] + i * (32 * kBK));
+            const u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[kb][1] + i * (32 * kBK));
             afrag[kb][i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
         } else {
             const int c = group - RT;
@@ -516,7 +516,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     // row_at / col_at = byte offsets of the item's scales: ring slot + position inside the span
     auto read_scale_group = [&](int slot, int row_at, int col_at, int group) {
         if (group < RT)
-            ascale[slot][group] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + sa_addr[group] + row_at));
+            ascale[slot][group] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + sa_addr + group * 512 + row_at));
         else
             bscale[slot][group - RT] =
                 static_cast<int>(*reinterpret_cast<const uint16_t*>(lds + sb_addr + (group - RT) * 512 + col_at));
