@@ -159,7 +159,7 @@ def megamoe_bench(torch, ops, dev, iters):
         "tflops_forward": flops / us / 1e6,
         "roofline": {"bound": "mfma", "achieved": flops / us / 1e6, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
-                     "note": "whole forward (5 launches); per-kernel GEMM times are in profiles/"},
+                     "note": "whole forward (4 launches); per-kernel GEMM times are in profiles/"},
     }
 
 
