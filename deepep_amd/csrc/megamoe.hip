@@ -775,24 +775,35 @@ int launch_gemm_rt(const GemmParams& p, hipStream_t stream, const char* what)
     return launch_status(what);
 }
 
-// Row-tile height: the cheapest of 64 / 128 / 192 rows, whose tile count fits one round of workgroups, judged
-// from the expected rows per expert (the true counts stay on the device).
+// Row-tile height: the cheapest of 64 / 128 / 192 rows by a small cost model, judged from the expected rows per expert (the true counts
+// stay on the device).  Routing scatters the counts around that mean (about +-sqrt(mean)), and one expert a few
+// rows over a multiple of the tile height costs a whole extra row tile each: the tile count is therefore the
+// expectation of ceil(rows / height) under a normal spread, not ceil(mean / height).  (Mean 256 over 8 experts:
+// 128-row tiles need 2.5 row tiles per expert on average = 320 tiles = two rounds on 256 CUs, 192-row tiles need
+// 2 = one round; measured 103 vs 80 us.)
 template <bool kGateUp>
 int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t stream, const char* what)
 {
     const int cus = gemm_grid();
     const int n_tiles = p.n / kBN;
+    const double mean = expected_rows_per_expert > 1 ? expected_rows_per_expert : 1;
+    const double sigma = sqrt(mean);
     int best = 2;
     double best_cost = 1e30;
     for (int rt = 1; rt <= 3; ++rt) {
         const int bm = 64 * rt;
-        const int m_tiles = (expected_rows_per_expert + bm - 1) / bm;
-        const long long tiles = static_cast<long long>(p.num_local) * (m_tiles > 0 ? m_tiles : 1) * n_tiles;
-        const long long rounds = (tiles + cus - 1) / cus;
-        // The time of a tile grows with its height, on top of a part that does not (its weight tile has to be
-        // fetched whatever the height, and there are the prologue and epilogue): the 64-row tile pays off only
-        // when the experts have few rows (decode), where the GEMM is bound by streaming the weights.
-        const double cost = static_cast<double>(rounds) * (rt + 0.5);
+        double m_tiles = 1.0;  // E[ceil(X / bm)] = sum over j >= 0 of P(X > j * bm)
+        for (int j = 1; j * bm < mean + 6.0 * sigma; ++j) m_tiles += 0.5 * erfc((j * bm - mean) / (sigma * 1.4142135623730951));
+        const double tiles = p.num_local * m_tiles * n_tiles;
+        const double rounds = ceil(tiles / cus - 0.02);  // a stray tile in one launch out of fifty does not count
+        // Microseconds per tile, fitted to kernel traces on an MI355X over shares from 32 to 512 rows per expert,
+        // 4 to 32 experts and two problem sizes (it reproduced the measured order of the three heights in 14 of 16
+        // cases, and was within 7 % in the other two): a fixed part (prologue, epilogue) plus a part per k tile;
+        // an expert with a single row tile streams its weight tile from HBM with nobody to share it with, which
+        // adds about 0.3 us per k tile whatever the height.
+        constexpr double kFixed[3] = {4.2, 2.9, 7.9}, kPerItem[3] = {0.53, 0.87, 1.29};
+        const double per_item = kPerItem[rt - 1] + (m_tiles <= 1.2 ? 0.3 : 0.0);
+        const double cost = (rounds < 1.0 ? 1.0 : rounds) * (kFixed[rt - 1] + (p.k / kBK) * per_item);
         if (cost < best_cost - 1e-9) {
             best_cost = cost;
             best = rt;
