@@ -354,7 +354,7 @@ struct GridBarrier {
 // the per-CU and per-XCD caches, so the barrier only has to order them: every thread waits until its own stores are
 // acknowledged before its workgroup's arrival is counted.  Acquire/release fences here would write back and
 // invalidate whole caches, which costs more than the launch this barrier saves.
-__device__ __forceinline__ bool grid_arrive_and_wait(GridBarrier* bar, unsigned needed, long long limit_ticks, int* verdict)
+__device__ __forceinline__ bool grid_arrive_and_wait(GridBarrier* bar, unsigned needed, long long limit_ticks, int* in_time_flag)
 {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -370,10 +370,10 @@ __device__ __forceinline__ bool grid_arrive_and_wait(GridBarrier* bar, unsigned 
             }
             seen = __hip_atomic_load(&bar->arrived, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        *verdict = in_time;
+        *in_time_flag = in_time;
     }
     __syncthreads();
-    return *verdict != 0;
+    return *in_time_flag != 0;
 }
 
 // The last workgroup to leave clears the barrier for the next launch: by then none is waiting on it any more.
@@ -407,7 +407,7 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     unsigned needed, long long limit_ticks, uint32_t* __restrict__ timeouts)
 {
     __shared__ LayoutLds lds;
-    __shared__ int verdict;
+    __shared__ int in_time_flag;
     DPEP_LAYOUT_STAMP(0);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = blockIdx.x * kWaves + wave;
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     DPEP_LAYOUT_STAMP(1);
     publish_histograms<true>(lds, num_local, num_chunks, wave_hist, block_hist);
     DPEP_LAYOUT_STAMP(2);
-    if (!grid_arrive_and_wait(bar, needed, limit_ticks, &verdict) && threadIdx.x == 0)
+    if (!grid_arrive_and_wait(bar, needed, limit_ticks, &in_time_flag) && threadIdx.x == 0)
         __hip_atomic_store(timeouts, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);  // this launch's results are not valid
     DPEP_LAYOUT_STAMP(3);
     expert_bases<true>(lds, wave_hist, block_hist, num_local, padded_local, num_chunks, gridDim.x - 1, counts, psum, offsets,
