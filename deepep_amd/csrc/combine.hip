@@ -30,7 +30,7 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ row_weights, const int* __restrict__ route_to_row,
     int num_topk, int vec_per_row, int vec_per_part, int parts, u32x4* __restrict__ out,
     const float* __restrict__ return_in, float* __restrict__ return_out, const int* __restrict__ shared_first_row,
-    int num_shared, int num_tokens)
+    int num_shared, int num_tokens, const int* __restrict__ fill_state)
 {
     __shared__ int rows[DPEP_MAX_TOPK + kBatch];
     __shared__ float wts[DPEP_MAX_TOPK + kBatch];
@@ -57,6 +57,12 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const int v_begin = part * vec_per_part;
     const int v_end = min(v_begin + vec_per_part, vec_per_row);
     if (!any_row) {
+        // (MegaMoE) rows that idle workgroups of the first GEMM have already zeroed: filler f of n took tokens
+        // f, f + n, ... and got through fill_state[1 + f] of them
+        if (kWeights == 2 && fill_state != nullptr) {
+            const int fillers = fill_state[0];
+            if (fillers > 0 && token / fillers < fill_state[1 + token % fillers]) return;
+        }
         const u32x4 zero = {0u, 0u, 0u, 0u};
         for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x)
             store16_nt(out + static_cast<size_t>(token) * vec_per_row + v, zero);
@@ -126,11 +132,12 @@ CombineGrid combine_grid(int num_tokens, int num_rows, int vec)
 template <int kWeights, bool kHalf = false>
 void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, const float* weights, const int32_t* route_to_row,
                     int num_topk, int vec, void* out, const float* return_in, float* return_out,
-                    const int32_t* shared_first_row = nullptr, int num_shared = 0, int num_tokens = 0)
+                    const int32_t* shared_first_row = nullptr, int num_shared = 0, int num_tokens = 0,
+                    const int32_t* fill_state = nullptr)
 {
     hipLaunchKernelGGL((combine_kernel<kWeights, kHalf>), dim3(g.blocks), dim3(g.threads), 0, stream, static_cast<const u32x4*>(y),
                        weights, route_to_row, num_topk, vec, g.per_part, g.parts, static_cast<u32x4*>(out), return_in,
-                       return_out, shared_first_row, num_shared, num_tokens);
+                       return_out, shared_first_row, num_shared, num_tokens, fill_state);
 }
 
 }  // namespace
@@ -138,12 +145,12 @@ void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, con
 // Route-weighted reduce used by the MegaMoE forward: out[t] = bf16( sum_s w[t,s] * float(y[row(t,s)]) ).
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
                    int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
-                   hipStream_t stream)
+                   const int32_t* fill_state, hipStream_t stream)
 {
     const int vec = hidden / 8;
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
     launch_combine<2>(g, stream, y, route_weights, route_to_row, num_topk, vec, out, nullptr, nullptr, shared_first_row,
-                      num_shared, num_tokens);
+                      num_shared, num_tokens, fill_state);
     return launch_status("combine_routes");
 }
 

@@ -22,7 +22,7 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
                int32_t* row_to_route, int32_t* num_rows, hipStream_t stream);
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
                    int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
-                   hipStream_t stream);
+                   const int32_t* fill_state, hipStream_t stream);
 
 namespace {
 
@@ -162,6 +162,7 @@ constexpr int kBK = 128;           // k per LDS stage = two MFMA k steps
 constexpr int kCT = 4;             // 32-column MFMA tiles per wave
 constexpr int kBN = 2 * kCT * 32;  // columns per workgroup tile
 constexpr int kGemmThreads = 256;
+constexpr int kGemmWaves = kGemmThreads / 64;
 constexpr int kMaxMoeExperts = 128;
 constexpr int kStagingRowStride = 80;  // 32 BF16 + 16 B pad: conflict-free 16-byte reads
 
@@ -205,6 +206,18 @@ struct GemmParams {
     uint8_t* act_codes;        // first GEMM: [rows, N/2] e4m3
     uint8_t* act_scales;       //             [rows, N/64] e8m0
     uint16_t* out;             // second GEMM: [rows, N] bf16
+    // Zero rows of the final output.  When a launch has fewer tiles than workgroups, the workgroups left
+    // without a tile stream zeros into the output rows of the tokens that no local expert serves (most tokens of a
+    // rank's share), which the weighted reduce would otherwise have to write after the GEMMs: the stores cost the
+    // matrix pipes nothing.  Every wave of such a workgroup is a filler f and takes tokens f, f + fillers, ...
+    // until a workgroup with a tile reaches its epilogue (fill_stop); fill_state[0] = number of fillers,
+    // fill_state[1 + f] = tokens filler f got through.  All of it is null / zero in launches that do not fill.
+    u32x4* fill_out;                // [fill_tokens, fill_vec] or nullptr
+    const int* fill_route_to_row;   // [fill_tokens, fill_topk]
+    int fill_tokens, fill_vec, fill_topk;
+    int* fill_state;
+    int* fill_stop;                 // written 1 by this launch, if it fills
+    int* clear_stop;                // written 0 by this launch (the one after the filling launch)
 };
 
 // gate / (1 + exp(-gate)) * up with the hardware exponential and reciprocal (about 1 ulp each; the
@@ -338,13 +351,51 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     __syncthreads();
     const int total_tiles = tile_base[p.num_local];
 
+    if (p.clear_stop != nullptr && blockIdx.x == 0 && tid == 0)
+        __hip_atomic_store(p.clear_stop, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
     // Consecutive tile ids share weights; give each XCD (workgroups are dealt round-robin over 8 XCDs)
-    // a contiguous range of tiles so that its L2 sees each weight tile from one place.
-    const int per_xcd = (gridDim.x + 7) / 8;
+    // a contiguous range of tiles so that its L2 sees each weight tile from one place.  With fewer tiles than
+    // workgroups the ranges shrink evenly, so that every XCD keeps some workgroups without a tile: those are
+    // the fillers, and stores from all eight XCDs together run three times faster than from one or two.
+    const int slots = gridDim.x >> 3;  // workgroups per XCD
+    const bool one_round = total_tiles < static_cast<int>(gridDim.x) && (gridDim.x & 7) == 0;
+    const int per_xcd = one_round ? (total_tiles + 7) / 8 : (gridDim.x + 7) / 8;
     const int first = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    const int stride = per_xcd * 8;
-    if (first >= total_tiles) return;
-    const int my_tiles = (total_tiles - first + stride - 1) / stride;
+    const int stride = one_round ? total_tiles + 1 : per_xcd * 8;  // one round: a single tile each
+    const bool has_tile = first < total_tiles && (!one_round || static_cast<int>(blockIdx.x >> 3) < per_xcd);
+#ifdef DPEP_TUNE_NO_FILL
+    const int fillers = 0;
+#else
+    const int fillers = one_round && p.fill_out != nullptr ? (static_cast<int>(gridDim.x) - total_tiles) * kGemmWaves : 0;
+#endif
+    if (blockIdx.x == 0 && tid == 0 && p.fill_state != nullptr) p.fill_state[0] = fillers;  // workgroup 0 always has tile 0
+    if (!has_tile) {
+        if (fillers == 0) return;
+        // number of this workgroup among those without a tile: XCD by XCD, then by slot
+        int rank = 0;
+        const int xcd = blockIdx.x & 7;
+        for (int x = 0; x <= xcd; ++x) {
+            const int tiles_here = min(max(total_tiles - x * per_xcd, 0), per_xcd);
+            rank += x < xcd ? slots - tiles_here : static_cast<int>(blockIdx.x >> 3) - tiles_here;
+        }
+        const int filler = rank * kGemmWaves + wave;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        int done = 0;
+        for (int token = filler; token < p.fill_tokens; token += fillers, ++done) {
+            if (__hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+            const bool mine = lane < p.fill_topk && p.fill_route_to_row[static_cast<size_t>(token) * p.fill_topk + lane] >= 0;
+            if (__ballot(mine) != 0ull) continue;  // some local expert serves the token: the reduce writes its row
+            u32x4* row = p.fill_out + static_cast<size_t>(token) * p.fill_vec;
+            for (int v = lane; v < p.fill_vec; v += 64) store16_nt(row + v, zero);
+#ifdef DPEP_TUNE_FILL_SLEEP
+            __builtin_amdgcn_s_sleep(DPEP_TUNE_FILL_SLEEP);
+#endif
+        }
+        if (lane == 0) p.fill_state[1 + filler] = done;
+        return;
+    }
+    const int my_tiles = one_round ? 1 : (total_tiles - first + stride - 1) / stride;
 
     auto decode = [&](int tile) {
         int e = 0;
@@ -708,6 +759,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         kt += 2;
         if (kt == ktiles) {
             DPEP_STAMP(4);
+            // a few microseconds of epilogue are left: time for the fillers to finish the row they are on
+            if (fillers != 0 && tid == 0) __hip_atomic_store(p.fill_stop, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             settle_accumulators();
             // tie every accumulator to a statement behind the wait, so that no read of it can be moved above
 #pragma unroll
@@ -885,7 +938,7 @@ int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scale
 
 // Workspace carve-up shared by workspace_bytes and forward.
 struct MegaLayout {
-    size_t hist, meta, route_to_row, row_to_route, act_codes, act_scales, out2, total;
+    size_t hist, meta, fill_state, route_to_row, row_to_route, act_codes, act_scales, out2, total;
 };
 
 static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int intermediate, int num_local, int num_shared)
@@ -898,6 +951,7 @@ static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int inte
     size_t at = 0;
     l.hist = at;         at += up(dpep_layout_workspace_bytes(num_tokens, num_topk, num_local));
     l.meta = at;         at += up((3 * static_cast<size_t>(num_local) + num_shared + 2) * 4);
+    l.fill_state = at;   at += up((1 + 4096) * 4);  // fillers of the first GEMM: count + progress of each (<= 1024 CUs x 4 waves)
     l.route_to_row = at; at += up(routes * 4);
     l.row_to_route = at; at += up((routes + shared_rows) * 4);
     l.act_codes = at;    at += up(max_rows * intermediate);
@@ -988,6 +1042,20 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     const long long expected_routed = static_cast<long long>(num_tokens) * num_topk * num_local / num_experts;
     const long long expected_rows = expected_routed + static_cast<long long>(num_tokens) * num_shared;
     const int per_expert = static_cast<int>((expected_rows + g1.num_local - 1) / g1.num_local);
+    // Without shared experts most tokens of a share have no row: workgroups of the first GEMM that get no tile
+    // zero those rows of y meanwhile, and the weighted reduce skips what they got through.
+    int* fill_state = reinterpret_cast<int*>(base + l.fill_state);
+    int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->barrier) + 64);
+    const bool fill = num_shared == 0;
+    if (fill) {
+        g1.fill_out = static_cast<u32x4*>(y);
+        g1.fill_route_to_row = route_to_row;
+        g1.fill_tokens = num_tokens;
+        g1.fill_vec = hidden / 8;
+        g1.fill_topk = num_topk;
+        g1.fill_stop = fill_stop;
+    }
+    g1.fill_state = fill_state;  // written even when nothing fills (then as "no fillers")
     if (int rc = launch_gemm1(g1, per_expert, s)) return rc;
     GemmParams g2{};
     g2.a_codes = base + l.act_codes;
@@ -1004,10 +1072,11 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g2.n = hidden;
     g2.k = intermediate;
     g2.out = reinterpret_cast<uint16_t*>(base + l.out2);
+    g2.clear_stop = fill_stop;
     if (int rc = launch_gemm2(g2, per_expert, s)) return rc;
     return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,
                           static_cast<int>(expected_rows),
-                          hidden, y, num_shared > 0 ? num_rows : nullptr, num_shared, s);
+                          hidden, y, num_shared > 0 ? num_rows : nullptr, num_shared, fill ? fill_state : nullptr, s);
 }
 
 }  // extern "C"

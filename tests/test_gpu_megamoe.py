@@ -301,3 +301,40 @@ def test_public_api_shared_experts():
         assert mm.relative_frobenius(y.float().cpu().numpy(), want) <= 2e-2
     finally:
         buf.destroy()
+
+
+def test_rows_of_unserved_tokens_are_zeroed_whoever_writes_them(ops):
+    """In a rank's share most tokens reach no local expert; their rows of y must come out as zeros.  Workgroups of the
+    first GEMM that get no tile write those zeros while the others compute, and the weighted reduce writes what they
+    did not get to: the result may not depend on who wrote a row, on what y held before, or on what the previous call
+    on the workspace left behind (a call whose first GEMM fills, then one with more tiles than workgroups, which does
+    not, then the first again)."""
+    dev = "cuda"
+    shapes = [  # tokens, hidden, inter, experts, begin, local, topk
+        (1536, 512, 512, 64, 8, 2, 4),      # 2 experts x few tiles: nearly every workgroup fills
+        (6144, 512, 2048, 16, 0, 16, 8),    # every expert local: about 1500 tiles, nobody fills, no token unserved
+        (1536, 512, 512, 64, 8, 2, 4),
+    ]
+    workspace = ops.Workspace(max(ops.megamoe_workspace_bytes(t, k, h, i, l) for t, h, i, _, _, l, k in shapes))
+    try:
+        for call, (tokens, hidden, inter, experts, begin, local, topk) in enumerate(shapes):
+            x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=call % 2)
+            w1, s1 = ops.megamoe_prepare_weights(torch.from_numpy(l1[0]).to(dev), torch.from_numpy(l1[1]).reshape(local, 2 * inter, -1).to(dev), True)
+            w2, s2 = ops.megamoe_prepare_weights(torch.from_numpy(l2[0]).to(dev), torch.from_numpy(l2[1]).reshape(local, hidden, -1).to(dev), False)
+            y = torch.full((tokens, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
+            counts = torch.empty((local,), dtype=torch.int32, device=dev)
+            ops.megamoe_forward(
+                workspace, torch.from_numpy(x_codes).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(x_scales).to(dev),
+                torch.from_numpy(idx).to(dev), torch.from_numpy(weights).to(dev), w1, s1, w2, s2, experts, begin, local, y, counts,
+            )
+            torch.cuda.synchronize()
+            got = y.float().cpu().numpy()
+            served = ((idx >= begin) & (idx < begin + local)).any(axis=1)
+            assert served.sum() < tokens or local == experts
+            assert not np.isnan(got).any()
+            assert not got[~served].any()  # exact zeros, every element
+            want = _oracle(x_codes, x_scales, l1, l2, idx, weights, begin)
+            err = np.linalg.norm(got - want) / np.linalg.norm(want)
+            assert err < 2e-2, err
+    finally:
+        workspace.destroy()
