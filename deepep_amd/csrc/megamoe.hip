@@ -356,30 +356,25 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 
     // Consecutive tile ids share weights; give each XCD (workgroups are dealt round-robin over 8 XCDs)
     // a contiguous range of tiles so that its L2 sees each weight tile from one place.  With fewer tiles than
-    // workgroups the ranges shrink evenly, so that every XCD keeps some workgroups without a tile: those are
-    // the fillers, and stores from all eight XCDs together run three times faster than from one or two.
-    const int slots = gridDim.x >> 3;  // workgroups per XCD
-    const bool one_round = total_tiles < static_cast<int>(gridDim.x) && (gridDim.x & 7) == 0;
-    const int per_xcd = one_round ? (total_tiles + 7) / 8 : (gridDim.x + 7) / 8;
-    const int first = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    const int stride = one_round ? total_tiles + 1 : per_xcd * 8;  // one round: a single tile each
-    const bool has_tile = first < total_tiles && (!one_round || static_cast<int>(blockIdx.x >> 3) < per_xcd);
+    // workgroups: a launch that fills keeps the ranges whole, so that the first XCDs are full and the workgroups
+    // without a tile, the fillers, sit together on the XCDs left over (their stores then stay out of the L2s the
+    // GEMM works from: fillers on every XCD fill faster but cost the GEMM three times as much); a launch that
+    // does not fill shrinks the ranges evenly (about 4 % faster than leaving two XCDs idle).
+    const bool one_round = total_tiles < static_cast<int>(gridDim.x);
 #ifdef DPEP_TUNE_NO_FILL
     const int fillers = 0;
 #else
     const int fillers = one_round && p.fill_out != nullptr ? (static_cast<int>(gridDim.x) - total_tiles) * kGemmWaves : 0;
 #endif
+    const bool spread = one_round && fillers == 0 && (gridDim.x & 7) == 0;
+    const int per_xcd = spread ? (total_tiles + 7) / 8 : (gridDim.x + 7) / 8;
+    const int first = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    const int stride = one_round ? total_tiles + 1 : per_xcd * 8;  // one round: a single tile each
+    const bool has_tile = first < total_tiles && (!spread || static_cast<int>(blockIdx.x >> 3) < per_xcd);
     if (blockIdx.x == 0 && tid == 0 && p.fill_state != nullptr) p.fill_state[0] = fillers;  // workgroup 0 always has tile 0
     if (!has_tile) {
         if (fillers == 0) return;
-        // number of this workgroup among those without a tile: XCD by XCD, then by slot
-        int rank = 0;
-        const int xcd = blockIdx.x & 7;
-        for (int x = 0; x <= xcd; ++x) {
-            const int tiles_here = min(max(total_tiles - x * per_xcd, 0), per_xcd);
-            rank += x < xcd ? slots - tiles_here : static_cast<int>(blockIdx.x >> 3) - tiles_here;
-        }
-        const int filler = rank * kGemmWaves + wave;
+        const int filler = (first - total_tiles) * kGemmWaves + wave;
         const u32x4 zero = {0u, 0u, 0u, 0u};
         int done = 0;
         for (int token = filler; token < p.fill_tokens; token += fillers, ++done) {
@@ -388,9 +383,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             if (__ballot(mine) != 0ull) continue;  // some local expert serves the token: the reduce writes its row
             u32x4* row = p.fill_out + static_cast<size_t>(token) * p.fill_vec;
             for (int v = lane; v < p.fill_vec; v += 64) store16_nt(row + v, zero);
-#ifdef DPEP_TUNE_FILL_SLEEP
-            __builtin_amdgcn_s_sleep(DPEP_TUNE_FILL_SLEEP);
-#endif
         }
         if (lane == 0) p.fill_state[1 + filler] = done;
         return;
