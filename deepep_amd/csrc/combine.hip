@@ -104,6 +104,84 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     }
 }
 
+// Route-weighted reduce for sparse shares (most tokens own no row, none owns a shared expert's): one WAVE per
+// token, so that a token without rows costs one short-lived wave instead of a workgroup with a barrier, and four
+// times as many tokens are in flight per CU (the kernel above spends its time on the chain of dependent loads
+// each of its 16384 workgroups starts with).  Same arithmetic in the same order as combine_kernel<2>: slots
+// ascending, separate fp32 multiply and add, one RNE rounding to BF16.
+#ifndef DPEP_TUNE_SPARSE_BATCH
+#define DPEP_TUNE_SPARSE_BATCH 8
+#endif
+#ifndef DPEP_TUNE_SPARSE_WAVES
+#define DPEP_TUNE_SPARSE_WAVES 4
+#endif
+constexpr int kSparseBatch = DPEP_TUNE_SPARSE_BATCH;  // 16-byte vectors per lane in flight per slot
+constexpr int kSparseWaves = DPEP_TUNE_SPARSE_WAVES;  // tokens (= waves) per workgroup
+__global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
+    const u32x4* __restrict__ y, const float* __restrict__ route_weights, const int* __restrict__ route_to_row,
+    int num_topk, int vec_per_row, u32x4* __restrict__ out, int num_tokens, const int* __restrict__ fill_state)
+{
+    const int lane = threadIdx.x & 63;
+    const int token = blockIdx.x * kSparseWaves + (threadIdx.x >> 6);
+    if (token >= num_tokens) return;
+    int row = -1;
+    float weight = 0.0f;
+    if (lane < num_topk) {
+        row = route_to_row[static_cast<size_t>(token) * num_topk + lane];
+        weight = route_weights[static_cast<size_t>(token) * num_topk + lane];
+    }
+    const uint64_t valid = __ballot(row >= 0);
+    u32x4* dst = out + static_cast<size_t>(token) * vec_per_row;
+    if (valid == 0ull) {
+        if (fill_state != nullptr) {  // rows that idle workgroups of the first GEMM have already zeroed
+            const int fillers = fill_state[0];
+            if (fillers > 0 && token / fillers < fill_state[1 + token % fillers]) return;
+        }
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        for (int v = lane; v < vec_per_row; v += 64) store16_nt(dst + v, zero);
+        return;
+    }
+    for (int v0 = 0; v0 < vec_per_row; v0 += 64 * kSparseBatch) {
+        float acc[kSparseBatch][8];
+#pragma unroll
+        for (int b = 0; b < kSparseBatch; ++b)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[b][i] = 0.0f;
+        for (uint64_t rest = valid; rest != 0ull; rest &= rest - 1ull) {
+            const int slot = __builtin_ctzll(rest);
+            const int r = __builtin_amdgcn_readlane(row, slot);
+            const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight), slot));
+            const u32x4* src = y + static_cast<size_t>(r) * vec_per_row;
+            u32x4 val[kSparseBatch];
+#pragma unroll
+            for (int b = 0; b < kSparseBatch; ++b) {
+                const int v = v0 + b * 64 + lane;
+                if (v < vec_per_row) val[b] = load16(src + v);  // rows the second GEMM has just written: cached
+            }
+#pragma unroll
+            for (int b = 0; b < kSparseBatch; ++b) {
+                if (v0 + b * 64 + lane >= vec_per_row) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lo = __fmul_rn(bf16_to_f32(val[b][i] & 0xffffu), w);
+                    const float hi = __fmul_rn(bf16_to_f32(val[b][i] >> 16), w);
+                    acc[b][2 * i] = __fadd_rn(acc[b][2 * i], lo);
+                    acc[b][2 * i + 1] = __fadd_rn(acc[b][2 * i + 1], hi);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < kSparseBatch; ++b) {
+            const int v = v0 + b * 64 + lane;
+            if (v >= vec_per_row) continue;
+            u32x4 packed;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) packed[i] = pack_bf16x2(acc[b][2 * i], acc[b][2 * i + 1]);
+            store16_nt(dst + v, packed);
+        }
+    }
+}
+
 struct CombineGrid {
     int parts, per_part, threads, blocks;
 };
@@ -148,6 +226,12 @@ int combine_routes(const void* y, const float* route_weights, const int32_t* rou
                    const int32_t* fill_state, hipStream_t stream)
 {
     const int vec = hidden / 8;
+    if (num_shared == 0 && 2LL * num_rows_hint < num_tokens) {  // a sparse share: most tokens own no row
+        hipLaunchKernelGGL(combine_sparse_kernel, dim3((num_tokens + kSparseWaves - 1) / kSparseWaves), dim3(64 * kSparseWaves), 0, stream,
+                           static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk, vec, static_cast<u32x4*>(out),
+                           num_tokens, fill_state);
+        return launch_status("combine_routes_sparse");
+    }
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
     launch_combine<2>(g, stream, y, route_weights, route_to_row, num_topk, vec, out, nullptr, nullptr, shared_first_row,
                       num_shared, num_tokens, fill_state);

@@ -378,7 +378,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         const u32x4 zero = {0u, 0u, 0u, 0u};
         int done = 0;
         for (int token = filler; token < p.fill_tokens; token += fillers, ++done) {
+#ifndef DPEP_TUNE_FILL_NO_STOP
             if (__hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+#endif
             const bool mine = lane < p.fill_topk && p.fill_route_to_row[static_cast<size_t>(token) * p.fill_topk + lane] >= 0;
             if (__ballot(mine) != 0ull) continue;  // some local expert serves the token: the reduce writes its row
             u32x4* row = p.fill_out + static_cast<size_t>(token) * p.fill_vec;
