@@ -35,16 +35,19 @@ def algorithmic_bytes(tokens, hidden, topk, rows):
 
 
 def time_kernel(fn, iters, torch, head_start=None):
-    """Average device time of `fn` in microseconds, HIP events on the stream the kernels run on.  `head_start`: a
-    large tensor that is filled first, so that the host queues launches while the GPU is busy and a kernel shorter
-    than its Python launch path is still timed back to back."""
+    """Average device time of `fn` in microseconds, HIP events on the stream the kernels run on.  `head_start`: the
+    GPU is kept busy first (a spin kernel of about 2 ms where torch offers one, else fills of that tensor), so that
+    the host queues launches meanwhile and a kernel shorter than its Python launch path is still timed back to back."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for _ in range(3):
         fn()
     torch.cuda.synchronize()
     if head_start is not None:
-        for _ in range(8):
-            head_start.zero_()
+        if hasattr(torch.cuda, "_sleep"):
+            torch.cuda._sleep(4_000_000)  # cycles; no memory traffic that the timed kernels would have to wait out
+        else:
+            for _ in range(8):
+                head_start.zero_()
     start.record()
     for _ in range(iters):
         fn()
