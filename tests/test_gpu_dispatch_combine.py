@@ -60,6 +60,7 @@ LAYOUT_SHAPES = [
     (16384, 8, 384, 0, 6),
     (16384, 8, 384, 378, 6),
     (5000, 6, 7, 2, 3),
+    (300, 32, 1024, 0, 1024),  # the largest top-k and expert count the library takes
     (16384, 8, 256, 0, 256),  # chunks too long for the one-launch kernel's registers: always two launches
 ]
 
@@ -341,3 +342,37 @@ def test_combine_fp16_matches_oracle(ops, ws, weighted):
     assert out.dtype == torch.float16
     ref = ocombine.combine_fp16(y.numpy(), want["route_to_row"], w_rows.numpy() if weighted else None)
     np.testing.assert_array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
+def test_random_shapes_end_to_end(ops, ws):
+    """Forty seeded shapes off the beaten path (token counts that are not multiples of the 64-route step, top-k that
+    does not divide it, expert counts that are not powers of two, receive shares, masked and repeated experts):
+    layout, BF16 dispatch with weights, fused FP8 dispatch and weighted combine, each bit-exact against the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        topk = int(rng.integers(1, 17))
+        experts = int(rng.integers(topk, 600))
+        tokens = int(rng.integers(1, 2500))
+        hidden = int(rng.choice([128, 256, 384, 1024, 2048]))
+        if case % 3 == 0:  # a receive share: a contiguous range of local experts
+            local = int(rng.integers(1, experts + 1))
+            begin = int(rng.integers(0, experts - local + 1))
+        else:
+            begin, local = 0, experts
+        idx = rng.integers(-1, experts + 1, size=(tokens, topk))  # -1 and E are both "no expert"; repeats allowed
+        label = f"case {case}: T={tokens} K={topk} E={experts} begin={begin} L={local} H={hidden}"
+        got, want, rows = _check_layout(ops, ws, idx, experts, begin, local)
+        gen = torch.Generator().manual_seed(case)
+        x = torch.randn(tokens, hidden, generator=gen).bfloat16()
+        w = torch.rand(tokens, topk, generator=gen)
+        out, _, out_w = ops.dispatch_copy(x.cuda(), None, w.cuda(), got["route_to_row"], got["row_to_route"], rows)
+        np.testing.assert_array_equal(bf16_bits(out), olayout.expand_rows(bf16_bits(x), want["row_to_route"], topk), err_msg=label)
+        w_rows = olayout.expand_weights(w.numpy(), want["row_to_route"])
+        np.testing.assert_array_equal(f32_bits(out_w), w_rows.view(np.uint32), err_msg=label)
+        q_ref, s_ref = oquant.cast_to_fp8_torch(x)
+        q, s, _ = ops.dispatch_quant_fp8(x.cuda(), None, got["route_to_row"], got["row_to_route"], None)  # R not passed
+        np.testing.assert_array_equal(fp8_bits(q[:rows]), olayout.expand_rows(fp8_bits(q_ref), want["row_to_route"], topk), err_msg=label)
+        np.testing.assert_array_equal(f32_bits(s[:rows]), olayout.expand_rows(f32_bits(s_ref), want["row_to_route"], topk), err_msg=label)
+        y = torch.randn(rows, hidden, generator=gen).bfloat16()
+        combined, _ = ops.combine(y.cuda(), got["route_to_row"], torch.from_numpy(w_rows).cuda())
+        np.testing.assert_array_equal(bf16_bits(combined), ocombine.combine(bf16_bits(y), want["route_to_row"], w_rows), err_msg=label)
