@@ -45,11 +45,15 @@ struct Workspace {
     // One-launch layout: its barrier between workgroups (device memory, zero between launches), the bound of the
     // barrier's wait in 100 MHz ticks, and two switches for tests (take two launches instead; expect more
     // arrivals than there are workgroups, so that the wait runs out).
-    void* barrier;
+    void* barrier;  // kSyncBytes of device memory behind the caller's bytes, see below
     long long barrier_ticks;
     int barrier_extra_arrivals;
     int layout_one_launch;
 };
+// Small words the kernels synchronise through, zero when the workspace is created and left zero by every launch:
+// the layout's barrier at offset 0 (two counters), the MegaMoE fillers' stop flag at kSyncFillStop.
+constexpr size_t kSyncBytes = 256;
+constexpr size_t kSyncFillStop = 64;
 constexpr int kMailboxTimeout = 2 + DPEP_MAX_LOCAL_EXPERTS;  // word a layout kernel sets when its barrier wait ran out
 constexpr int kMailboxWords = 3 + DPEP_MAX_LOCAL_EXPERTS;
 constexpr long long kLayoutBarrierTicks = 200000000;  // 2 s

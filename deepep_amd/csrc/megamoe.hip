@@ -1039,7 +1039,7 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     // Without shared experts most tokens of a share have no row: workgroups of the first GEMM that get no tile
     // zero those rows of y meanwhile, and the weighted reduce skips what they got through.
     int* fill_state = reinterpret_cast<int*>(base + l.fill_state);
-    int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->barrier) + 64);
+    int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->barrier) + kSyncFillStop);
     const bool fill = num_shared == 0;
     if (fill) {
         g1.fill_out = static_cast<u32x4*>(y);

@@ -41,8 +41,8 @@ int dpep_workspace_create(size_t bytes, void** ws)
     *ws = nullptr;
     void* base = nullptr;
     const size_t barrier_at = (bytes + 255) / 256 * 256;  // the layout's barrier words follow the caller's bytes
-    DPEP_HIP(hipMalloc(&base, barrier_at + 256));
-    if (hipError_t cleared = hipMemset(static_cast<char*>(base) + barrier_at, 0, 256); cleared != hipSuccess) {
+    DPEP_HIP(hipMalloc(&base, barrier_at + dpep::kSyncBytes));
+    if (hipError_t cleared = hipMemset(static_cast<char*>(base) + barrier_at, 0, dpep::kSyncBytes); cleared != hipSuccess) {
         (void)hipFree(base);
         return dpep::fail(DPEP_ERUNTIME, "workspace_create: %s", hipGetErrorString(cleared));
     }
