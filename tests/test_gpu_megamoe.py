@@ -338,3 +338,45 @@ def test_rows_of_unserved_tokens_are_zeroed_whoever_writes_them(ops):
             assert err < 2e-2, err
     finally:
         workspace.destroy()
+
+
+def test_full_size_share_against_its_served_tokens_alone(ops):
+    """The benchmark share at full size (16384 candidate tokens, 6 of 384 experts, top-8, H=7168, I=2048), too big
+    for the CPU oracle: every token's output depends on that token alone, so the forward over all tokens must
+    reproduce, bit for bit, a forward over the served tokens only (which runs with other tile heights, no zero
+    rows and the dense reduce), rows of unserved tokens must be exact zeros, and the counts must be a bincount."""
+    dev = "cuda"
+    tokens, hidden, inter, experts, local, topk = 16384, 7168, 2048, 384, 6, 8
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    idx = torch.stack([torch.randperm(experts, generator=gen)[:topk] for _ in range(tokens)]).to(torch.int32)
+    weights = torch.rand(tokens, topk, generator=gen)
+    x = (torch.randn(tokens, hidden, generator=gen) * 0.5).bfloat16().to(dev)
+    x_codes, x_scales = ops.mx_quant(x)
+    raw1 = torch.randint(0, 256, (local, 2 * inter, hidden // 2), dtype=torch.uint8, generator=gen).to(dev)
+    raw2 = torch.randint(0, 256, (local, hidden, inter // 2), dtype=torch.uint8, generator=gen).to(dev)
+    sc1 = torch.randint(116, 120, (local, 2 * inter, hidden // 32), dtype=torch.uint8, generator=gen).to(dev)
+    sc2 = torch.randint(116, 120, (local, hidden, inter // 32), dtype=torch.uint8, generator=gen).to(dev)
+    w1, s1 = ops.megamoe_prepare_weights(raw1, sc1, True)
+    w2, s2 = ops.megamoe_prepare_weights(raw2, sc2, False)
+
+    def forward(keep):
+        n = int(keep.sum())
+        workspace = ops.Workspace(ops.megamoe_workspace_bytes(n, topk, hidden, inter, local))
+        y = torch.full((n, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
+        counts = torch.empty((local,), dtype=torch.int32, device=dev)
+        keep_dev = keep.to(dev)
+        ops.megamoe_forward(workspace, x_codes[keep_dev].contiguous(), x_scales[keep_dev].contiguous(), idx[keep].contiguous().to(dev),
+                            weights[keep].contiguous().to(dev), w1, s1, w2, s2, experts, 0, local, y, counts)
+        torch.cuda.synchronize()
+        workspace.destroy()
+        return y, counts.cpu()
+
+    served = (idx < local).any(dim=1)
+    everyone = torch.ones(tokens, dtype=torch.bool)
+    y_all, counts_all = forward(everyone)
+    y_served, counts_served = forward(served)
+    assert 1500 < int(served.sum()) < 2500
+    assert counts_all.tolist() == counts_served.tolist() == torch.bincount(idx.flatten().long(), minlength=experts)[:local].tolist()
+    assert not torch.isnan(y_all.float()).any() and not y_all[~served.to(dev)].any()
+    assert torch.equal(y_all[served.to(dev)].view(torch.int16), y_served.view(torch.int16))
+    assert y_served.float().abs().max() > 0
