@@ -252,7 +252,9 @@ int combine_entry(const char* what, const void* y, const float* row_weights, con
     DPEP_REQUIRE(num_rows >= 0 && static_cast<long long>(num_rows) <= static_cast<long long>(num_tokens) * num_topk,
                  "%s: num_rows=%d outside [0, T*K]", what, num_rows);
     DPEP_REQUIRE(hidden > 0 && hidden % 8 == 0, "%s: hidden=%d must be a positive multiple of 8", what, hidden);
-    DPEP_REQUIRE((return_in == nullptr) == (return_out == nullptr), "%s: return_in and return_out go together", what);
+    // (with no rows at all the channel's input is an empty buffer, which may well be a null pointer)
+    DPEP_REQUIRE(return_in == nullptr ? (return_out == nullptr || num_rows == 0) : return_out != nullptr,
+                 "%s: return_in and return_out go together", what);
     if (num_tokens == 0) return DPEP_OK;
     DPEP_REQUIRE(route_to_row != nullptr && out != nullptr && aligned16(out), "%s: NULL or misaligned buffer", what);
     DPEP_REQUIRE(num_rows == 0 || (y != nullptr && aligned16(y)), "%s: y must be 16-byte aligned", what);

@@ -168,3 +168,26 @@ def test_low_latency_dispatch_combine_rank_share(payload):
             np.testing.assert_array_equal(bf16_bits(out), want_out)
     finally:
         buffer.destroy()
+
+
+def test_elastic_buffer_all_routes_masked():
+    """No valid route at all: the payload kernel is queued before the host knows that R = 0; outputs are empty views,
+    the handle says zero rows everywhere, and the combine of nothing is a tensor of zeros."""
+    import deepep_amd
+
+    tokens, hidden, topk, experts = 300, 1024, 4, 16
+    x = torch.randn(tokens, hidden).bfloat16().cuda()
+    idx = torch.full((tokens, topk), -1, dtype=torch.int64).cuda()
+    w = torch.rand(tokens, topk).cuda()
+    for fp8 in (False, True):
+        buffer = deepep_amd.ElasticBuffer(None, num_max_tokens_per_rank=tokens, hidden=hidden, num_topk=topk,
+                                          use_fp8_dispatch=fp8, explicitly_destroy=True)
+        try:
+            recv, _, recv_w, handle, _ = buffer.dispatch(x, topk_idx=idx, topk_weights=w, num_experts=experts)
+            payload = recv[0] if fp8 else recv
+            assert tuple(payload.shape) == (0, hidden) and tuple(recv_w.shape) == (0,)
+            assert handle.num_expanded_tokens == 0 and handle.num_recv_tokens_per_expert_list == [0] * experts
+            out, out_w, _ = buffer.combine(torch.empty((0, hidden), dtype=torch.bfloat16, device="cuda"), handle, topk_weights=recv_w)
+            assert not out.any() and tuple(out.shape) == (tokens, hidden) and not out_w.any()
+        finally:
+            buffer.destroy()
