@@ -380,3 +380,25 @@ def test_full_size_share_against_its_served_tokens_alone(ops):
     assert not torch.isnan(y_all.float()).any() and not y_all[~served.to(dev)].any()
     assert torch.equal(y_all[served.to(dev)].view(torch.int16), y_served.view(torch.int16))
     assert y_served.float().abs().max() > 0
+
+
+def test_megamoe_forward_without_any_local_route(ops):
+    """Every token routed to experts of other ranks, and the opposite corner, one local expert taking nothing while
+    its neighbour takes everything: zero output and zero counts in the first case (the GEMM launches have no tile
+    at all), parity with the oracle in the second."""
+    dev = "cuda"
+    tokens, hidden, inter, experts, begin, local, topk = 200, 512, 512, 16, 4, 2, 2
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=3)
+    elsewhere = idx.copy()
+    elsewhere[(elsewhere >= begin) & (elsewhere < begin + local)] = 0  # expert 0 belongs to another rank
+    got, counts = _run(ops, x_codes, x_scales, l1, l2, elsewhere, weights, experts, begin, local)
+    assert not got.any() and counts.tolist() == [0, 0]
+    one_sided = idx.copy()
+    one_sided[one_sided == begin] = begin + 1  # may repeat an expert within a token: give those slots to expert 0
+    for t in range(tokens):
+        if (one_sided[t] == begin + 1).sum() > 1:
+            one_sided[t, 1] = 0
+    got, counts = _run(ops, x_codes, x_scales, l1, l2, one_sided, weights, experts, begin, local)
+    assert counts[0] == 0 and counts[1] == (one_sided == begin + 1).sum() > 0
+    want = _oracle(x_codes, x_scales, l1, l2, one_sided, weights, begin)
+    assert mm.relative_frobenius(got, want) <= 2e-2
