@@ -402,3 +402,35 @@ def test_megamoe_forward_without_any_local_route(ops):
     assert counts[0] == 0 and counts[1] == (one_sided == begin + 1).sum() > 0
     want = _oracle(x_codes, x_scales, l1, l2, one_sided, weights, begin)
     assert mm.relative_frobenius(got, want) <= 2e-2
+
+
+def test_forward_is_reproducible_whoever_zeroes_which_row(ops):
+    """How far the first GEMM's idle workgroups get with the zero rows before they are told to stop changes from run
+    to run; the output may not: fifty forwards over the same share, y poisoned before each, all bit-identical."""
+    dev = "cuda"
+    tokens, hidden, inter, experts, local, topk = 8192, 2048, 1024, 256, 4, 8
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    idx = torch.stack([torch.randperm(experts, generator=gen)[:topk] for _ in range(tokens)]).to(torch.int32).to(dev)
+    weights = torch.rand(tokens, topk, generator=gen).to(dev)
+    x_codes, x_scales = ops.mx_quant((torch.randn(tokens, hidden, generator=gen) * 0.5).bfloat16().to(dev))
+    w1, s1 = ops.megamoe_prepare_weights(torch.randint(0, 256, (local, 2 * inter, hidden // 2), dtype=torch.uint8, generator=gen).to(dev),
+                                         torch.full((local, 2 * inter, hidden // 32), 118, dtype=torch.uint8, device=dev), True)
+    w2, s2 = ops.megamoe_prepare_weights(torch.randint(0, 256, (local, hidden, inter // 2), dtype=torch.uint8, generator=gen).to(dev),
+                                         torch.full((local, hidden, inter // 32), 118, dtype=torch.uint8, device=dev), False)
+    workspace = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local))
+    y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+    served = (idx < local).any(dim=1)
+    first = None
+    try:
+        for _ in range(50):
+            y.fill_(float("nan"))
+            ops.megamoe_forward(workspace, x_codes, x_scales, idx, weights, w1, s1, w2, s2, experts, 0, local, y, counts)
+            torch.cuda.synchronize()
+            if first is None:
+                first = y.clone()
+                assert not torch.isnan(first.float()).any() and not first[~served].any() and first[served].any()
+            else:
+                assert torch.equal(y.view(torch.int16), first.view(torch.int16))
+    finally:
+        workspace.destroy()
