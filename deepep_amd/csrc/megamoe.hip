@@ -597,6 +597,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         // The staging region holds one 32 x 32 tile as BF16 rows.
 #pragma unroll
         for (int i = 0; i < RT; ++i) {
+            // The last row tile of the epilogue is about what a filler needs to finish the row it is on: tell them to
+            // stop (the first workgroup to get here does; the others are at most a few microseconds behind).
+            if (i == RT - 1 && fillers != 0 && tid == 0)
+                __hip_atomic_store(p.fill_stop, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int tile_rows = min(32, info.valid - wm * 32 * RT - 32 * i);  // may be <= 0
             const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT + 32 * i;
 #pragma unroll
@@ -753,8 +757,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         kt += 2;
         if (kt == ktiles) {
             DPEP_STAMP(4);
-            // a few microseconds of epilogue are left: time for the fillers to finish the row they are on
-            if (fillers != 0 && tid == 0) __hip_atomic_store(p.fill_stop, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             settle_accumulators();
             // tie every accumulator to a statement behind the wait, so that no read of it can be moved above
 #pragma unroll
