@@ -13,10 +13,16 @@ experiments/megamoe/tests/test_reference.py:
   * bf16 ties-to-even bit patterns (:73-76);
   * decomposition over expert subsets and the single-expert special case (:57-71);
   * route weight applied after GMM2 does not commute with quantization (:79-88);
-  * the FFN itself reduces to a library matmul on dequantized fp32 operands.
-``quantize_weight_mxfp4`` is the build's own OCP-MX weight quantizer: the reference never
-quantizes weights (reference.py:72-81 samples packed nibbles directly) — parity unpinned; it is
-judged only through the 2e-2 relative Frobenius criterion.
+  * the FFN itself reduces to a library matmul on dequantized fp32 operands;
+  * ``swiglu``: closed forms (gate 0, sigmoid(ln 3) = 3/4, saturation, the clip at 80, operand roles) and
+    torch's silu; ``expert_forward``: a hand-sized case whose every step is exact, written out in the
+    test, and the same chain spelled with torch library routines (reference.py:84-89).
+``quantize_weight_mxfp4`` is the build's own OCP-MX weight quantizer: the reference never quantizes weights
+(reference.py:72-81 samples packed nibbles directly), so it holds no vector for it.  It is pinned to the OCP MX
+v1.0 rule instead: a brute-force nearest-e2m1 search with explicit ties-to-even over block exponents, grid
+values and midpoints.  It only builds test and benchmark inputs.
+
+Test infrastructure: only tests/, the driver's smoke check and the benchmark's CPU-baseline leg use this module.
 """
 
 from __future__ import annotations
@@ -88,7 +94,8 @@ def quantize_weight_mxfp4(w):
     """Dense float32 [..., N, K] -> (packed uint8 [..., N, K/2], e8m0 uint8 [..., N, K/64, 2]).
 
     OCP MX v1.0 recipe: shared exponent = floor(log2(amax)) - 2 (e2m1 emax), elements rounded to
-    e2m1 nearest-even with saturation at 6.  The build's own helper — parity unpinned (see header).
+    e2m1 nearest-even with saturation at 6.  The build's own helper (the reference holds no weight quantizer);
+    pinned to that rule by brute force in tests/test_oracle_megamoe.py.
     """
     w = np.asarray(w, dtype=np.float32)
     k = w.shape[-1]
