@@ -49,12 +49,16 @@ struct Workspace {
     long long barrier_ticks;
     int barrier_extra_arrivals;
     int layout_one_launch;
+    uint32_t layout_launches;  // number of the most recent layout launch (never 0)
+    uint32_t timeout_seen;     // number of the last timed-out launch the host has been told about
+    int gemm_tile_rows;  // 0: the grouped GEMM chooses its tile height; 64 / 128 / 192: forced (tests)
 };
 // Small words the kernels synchronise through, zero when the workspace is created and left zero by every launch:
-// the layout's barrier at offset 0 (two counters), the MegaMoE fillers' stop flag at kSyncFillStop.
-constexpr size_t kSyncBytes = 256;
-constexpr size_t kSyncFillStop = 64;
-constexpr int kMailboxTimeout = 2 + DPEP_MAX_LOCAL_EXPERTS;  // word a layout kernel sets when its barrier wait ran out
+// the layout's barrier at offset 0 (two counters), and from kSyncArrivals on one arrival counter per workgroup of
+// the grouped GEMM (tiles whose k range several workgroups share).
+constexpr size_t kSyncBytes = 8192;
+constexpr size_t kSyncArrivals = 1024;  // int[1024] up to kSyncBytes - 3072
+constexpr int kMailboxTimeout = 2 + DPEP_MAX_LOCAL_EXPERTS;  // a layout kernel whose barrier wait ran out leaves its launch number here
 constexpr int kMailboxWords = 3 + DPEP_MAX_LOCAL_EXPERTS;
 constexpr long long kLayoutBarrierTicks = 200000000;  // 2 s
 constexpr uint32_t kWorkspaceMagic = 0x44504550u;  // "DPEP"

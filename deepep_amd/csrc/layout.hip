@@ -16,8 +16,10 @@
 //            lives in LDS.  There is no separate scan launch.
 // Inputs whose chunks fit a wave's registers (at most kKeep steps of 64 routes) take ONE launch: the workgroups
 // (at most 65, far fewer than there are CUs, so all are resident together) count, meet at a barrier in device
-// memory, and assign from the ids they still hold.  The barrier's wait is bounded; a wait that runs out is
-// recorded in the workspace's mailbox and fails the next call on that workspace.  Larger inputs take two launches.
+// memory, and assign from the ids they still hold.  The barrier's wait is bounded; a launch whose wait runs out
+// assigns nothing (its histograms may be stale): it reports no rows, marks every route as having none, and leaves
+// its number in the workspace's mailbox, where the host finds it; later layouts on that workspace take two
+// launches.  Larger inputs take two launches anyway.
 #include "common.h"
 
 namespace dpep {
@@ -214,7 +216,7 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
                                              const int* __restrict__ block_hist, int num_local, int padded_local,
                                              int num_chunks, int num_blocks, int* __restrict__ counts,
                                              int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows,
-                                             uint32_t* __restrict__ mailbox, uint32_t sequence)
+                                             uint32_t* __restrict__ mailbox, uint32_t sequence, bool valid = true)
 {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const bool reporter = blockIdx.x == gridDim.x - 1;
@@ -226,11 +228,12 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
             own[w] = g < num_chunks ? load_int<kCoherent>(wave_hist + static_cast<size_t>(g) * num_local + e) : 0;
         }
     };
+    // (valid == false: the histograms cannot be trusted, every count is reported as zero)
     auto finish = [&](int e, int total, int before, const int (&own)[kWaves]) {  // the waves one after the other
-        lds.totals[e] = total;
+        lds.totals[e] = valid ? total : 0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            lds.running[w][e] = before;
+            lds.running[w][e] = valid ? before : 0;
             before += own[w];
         }
     };
@@ -389,13 +392,6 @@ __device__ __forceinline__ void grid_depart(GridBarrier* bar)
     }
 }
 
-#ifdef DPEP_DEBUG_TIMING
-__device__ unsigned long long g_layout_times[8];
-#define DPEP_LAYOUT_STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) g_layout_times[i] = wall_clock64(); } while (0)
-#else
-#define DPEP_LAYOUT_STAMP(i) do { } while (0)
-#endif
-
 // Count, barrier, assign in one launch; every wave keeps the ids of its chunk (at most kKeep steps) in registers.
 // `needed` is the number of workgroups (the reporter included), `limit_ticks` the bound of the wait (100 MHz ticks).
 template <typename IdxT>
@@ -404,11 +400,10 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     int chunk, int num_chunks, int* __restrict__ wave_hist, int* __restrict__ block_hist, int* __restrict__ counts,
     int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows, int* __restrict__ route_to_row,
     int* __restrict__ row_to_route, uint32_t* __restrict__ mailbox, uint32_t sequence, GridBarrier* __restrict__ bar,
-    unsigned needed, long long limit_ticks, uint32_t* __restrict__ timeouts)
+    unsigned needed, long long limit_ticks, uint32_t* __restrict__ timeouts, uint32_t launch_id)
 {
     __shared__ LayoutLds lds;
     __shared__ int in_time_flag;
-    DPEP_LAYOUT_STAMP(0);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = blockIdx.x * kWaves + wave;
     const int begin = g < num_chunks ? g * chunk : 0;
@@ -418,23 +413,24 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     clear_wave_lds(lds, num_local);
 #pragma unroll
     for (int i = 0; i < kKeep; ++i) count_step(experts[i], lds.running[wave]);
-    DPEP_LAYOUT_STAMP(1);
     publish_histograms<true>(lds, num_local, num_chunks, wave_hist, block_hist);
-    DPEP_LAYOUT_STAMP(2);
-    if (!grid_arrive_and_wait(bar, needed, limit_ticks, &in_time_flag) && threadIdx.x == 0)
-        __hip_atomic_store(timeouts, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);  // this launch's results are not valid
-    DPEP_LAYOUT_STAMP(3);
+    const bool in_time = grid_arrive_and_wait(bar, needed, limit_ticks, &in_time_flag);
+    if (!in_time && threadIdx.x == 0)  // this launch's results are not valid
+        __hip_atomic_store(timeouts, launch_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     expert_bases<true>(lds, wave_hist, block_hist, num_local, padded_local, num_chunks, gridDim.x - 1, counts, psum, offsets,
-                       num_rows, mailbox, sequence);
-    DPEP_LAYOUT_STAMP(4);
+                       num_rows, mailbox, sequence, in_time);
+    if (in_time) {
 #pragma unroll
-    for (int i = 0; i < kKeep; ++i)
-        if (begin + i * kWave < end)
-            assign_step(experts[i], begin + i * kWave + lane, end, lds.match[wave], lds.running[wave], route_to_row,
-                        row_to_route);
-    DPEP_LAYOUT_STAMP(5);
+        for (int i = 0; i < kKeep; ++i)
+            if (begin + i * kWave < end)
+                assign_step(experts[i], begin + i * kWave + lane, end, lds.match[wave], lds.running[wave], route_to_row,
+                            row_to_route);
+    } else {
+        // Some workgroup's histogram may be missing or left over from an earlier launch: rows computed from it
+        // could lie anywhere.  No route gets a row (and the counts above are all zero).
+        for (int route = begin + lane; route < end; route += kWave) route_to_row[route] = -1;
+    }
     grid_depart(bar);
-    DPEP_LAYOUT_STAMP(6);
 }
 
 int padded_experts(int num_local)
@@ -472,9 +468,16 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
     DPEP_REQUIRE(n_routes == 0 || (idx && route_to_row && row_to_route), "layout: NULL routing buffer");
     const size_t need = dpep_layout_workspace_bytes(num_tokens, num_topk, num_local);
     DPEP_REQUIRE(need <= w->bytes, "layout: workspace too small (%zu needed, %zu available)", need, w->bytes);
-    if (w->mailbox_host[kMailboxTimeout] != 0)
-        return fail(DPEP_ERUNTIME, "layout: an earlier layout kernel on this workspace ran out of time at its barrier; "
-                                   "its results were not valid and the workspace must be replaced");
+    // A one-launch layout whose barrier wait ran out left its number in the mailbox.  If nobody has been told yet
+    // (the launch reported to no host wait: MegaMoE's internal layout), this call is; either way the workspace
+    // takes two launches from then on.
+    if (const uint32_t timed_out = w->mailbox_host[kMailboxTimeout]; timed_out != w->timeout_seen) {
+        w->timeout_seen = timed_out;
+        w->layout_one_launch = 0;
+        return fail(DPEP_ERUNTIME, "layout: an earlier layout kernel on this workspace ran out of time at its barrier "
+                                   "between workgroups and reported no rows; layouts on this workspace take two launches from now on");
+    }
+    w->layout_launches = w->layout_launches == 0xffffffffu ? 1u : w->layout_launches + 1u;  // never 0
     const int padded = padded_experts(num_local);
     const int chunk = chunk_routes(n_routes, padded);
     const int num_chunks = (n_routes + chunk - 1) / chunk;
@@ -491,7 +494,7 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
                            expert_begin, num_local, padded, chunk, num_chunks, wave_hist, block_hist, counts, psum, offsets,
                            num_rows, route_to_row, row_to_route, mailbox, w->sequence,
                            static_cast<GridBarrier*>(w->barrier), static_cast<unsigned>(blocks + 1 + w->barrier_extra_arrivals),
-                           w->barrier_ticks, w->mailbox_device + kMailboxTimeout);
+                           w->barrier_ticks, w->mailbox_device + kMailboxTimeout, w->layout_launches);
         return launch_status("layout_fused");
     }
     if (blocks > 0) {
@@ -521,13 +524,6 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
 }  // namespace dpep
 
 extern "C" {
-
-#ifdef DPEP_DEBUG_TIMING
-int dpep_debug_layout_times(unsigned long long* host8)
-{
-    return hipMemcpyFromSymbol(host8, HIP_SYMBOL(dpep::g_layout_times), 8 * sizeof(unsigned long long)) == hipSuccess ? 0 : -2;
-}
-#endif
 
 size_t dpep_layout_workspace_bytes(int num_tokens, int num_topk, int num_local_experts)
 {

@@ -73,6 +73,9 @@ int dpep_workspace_create(size_t bytes, void** ws)
     w->barrier_ticks = dpep::kLayoutBarrierTicks;
     w->barrier_extra_arrivals = 0;
     w->layout_one_launch = 1;
+    w->gemm_tile_rows = 0;
+    w->layout_launches = 0;
+    w->timeout_seen = 0;
     *ws = w;
     return DPEP_OK;
 }
@@ -112,9 +115,12 @@ int dpep_layout_wait(void* ws, int32_t* counts_host, int num_local, int32_t* num
         __builtin_ia32_pause();
     }
     __atomic_thread_fence(__ATOMIC_ACQUIRE);
-    if (box[dpep::kMailboxTimeout] != 0)
-        return dpep::fail(DPEP_ERUNTIME, "layout_wait: the layout kernel ran out of time at its barrier between "
-                                         "workgroups; its results are not valid and the workspace must be replaced");
+    if (const uint32_t timed_out = box[dpep::kMailboxTimeout]; timed_out != w->timeout_seen) {
+        w->timeout_seen = timed_out;
+        w->layout_one_launch = 0;
+        return dpep::fail(DPEP_ERUNTIME, "layout_wait: the layout kernel ran out of time at its barrier between workgroups "
+                                         "and reported no rows; layouts on this workspace take two launches from now on");
+    }
     *num_rows_host = static_cast<int32_t>(box[0]);
     if (counts_host != nullptr)
         for (int e = 0; e < num_local; ++e) counts_host[e] = static_cast<int32_t>(box[2 + e]);
@@ -133,6 +139,10 @@ int dpep_workspace_tune(void* ws, const char* key, long long value)
     } else if (strcmp(key, "layout_barrier_extra_arrivals") == 0) {
         DPEP_REQUIRE(value >= 0 && value <= 1, "workspace_tune: layout_barrier_extra_arrivals is 0 or 1");
         w->barrier_extra_arrivals = static_cast<int>(value);
+    } else if (strcmp(key, "gemm_tile_rows") == 0) {
+        DPEP_REQUIRE(value == 0 || value == 64 || value == 128 || value == 192,
+                     "workspace_tune: gemm_tile_rows is 0 (automatic), 64, 128 or 192");
+        w->gemm_tile_rows = static_cast<int>(value);
     } else {
         return dpep::fail(DPEP_EINVAL, "workspace_tune: unknown key '%s'", key);
     }

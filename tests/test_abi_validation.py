@@ -35,7 +35,9 @@ def test_null_workspace_and_ranges(lib):
 def test_payload_entry_points_check_arguments_first(lib):
     # (bad top-k, bad row count, unaligned rows) are reported before any pointer is followed
     assert lib.dpep_combine(None, None, None, 4, 0, 0, 128, None, None, None, None) == -1 and "K=0" in _message(lib)
-    assert lib.dpep_combine(None, None, None, 4, 2, 9, 128, None, None, None, None) == -1 and "num_rows" in _message(lib)
+    assert lib.dpep_combine(None, None, None, 4, 2, -3, 128, None, None, None, None) == -1 and "num_rows" in _message(lib)
+    # more rows than routes is fine (a capacity layout); the call then fails on the buffers it was not given
+    assert lib.dpep_combine(None, None, None, 4, 2, 9, 128, None, None, None, None) == -1 and "NULL" in _message(lib)
     assert lib.dpep_combine(None, None, None, 4, 2, 4, 12, None, None, None, None) == -1 and "hidden" in _message(lib)
     assert lib.dpep_combine(None, None, None, 0, 2, 0, 128, None, None, None, None) == 0  # nothing to do
     assert lib.dpep_dispatch_copy(None, None, None, None, None, 4, 33, 4, 256, 0, None, None, None, None) == -1

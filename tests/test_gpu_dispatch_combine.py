@@ -81,20 +81,53 @@ def test_layout_matches_oracle(ops, ws, tokens, topk, experts, begin, local, one
 
 def test_layout_barrier_wait_that_runs_out_is_reported(ops):
     """The barrier's wait is bounded: told to expect one workgroup more than the launch has, with a bound of
-    100 us, every workgroup gives up, the kernel ends normally, and the host gets an error instead of results."""
+    100 us, every workgroup gives up and the kernel ends normally.  Such a launch assigns nothing (its histograms may
+    be stale, so any row computed from them could lie anywhere): every route is left without a row, every count is
+    zero, and the host gets an error instead of results.  The workspace stays usable: later layouts take two launches."""
+    workspace = ops.Workspace(1 << 20)
+    try:
+        idx = torch.randint(0, 16, (512, 4), device="cuda")
+        want = olayout.layout(idx.cpu().numpy(), 16)
+        good = ops.layout(workspace, idx, 16)  # leaves valid histograms of this very input behind
+        ops.layout_wait(workspace)
+        workspace.tune("layout_barrier_extra_arrivals", 1)
+        workspace.tune("layout_barrier_ticks", 10_000)
+        lay = ops.layout(workspace, idx, 16)
+        with pytest.raises(RuntimeError, match="barrier"):
+            ops.layout_wait(workspace)
+        torch.cuda.synchronize()
+        assert (lay["route_to_row"] == -1).all() and not lay["counts"].any() and not lay["psum"].any()
+        assert not lay["offsets"].any() and int(lay["num_rows"].item()) == 0
+        workspace.tune("layout_barrier_extra_arrivals", 0)
+        again = ops.layout(workspace, idx, 16)  # two launches now; the earlier failure has been reported already
+        _, rows = ops.layout_wait(workspace)
+        assert rows == want["num_rows"]
+        np.testing.assert_array_equal(again["route_to_row"].cpu().numpy(), want["route_to_row"])
+        np.testing.assert_array_equal(good["route_to_row"].cpu().numpy(), want["route_to_row"])
+        with pytest.raises(ValueError, match="unknown key"):
+            workspace.tune("no_such_switch", 1)
+    finally:
+        workspace.destroy()
+
+
+def test_layout_timeout_nobody_waited_for_is_reported_by_the_next_call(ops):
+    """A launch that timed out without a host wait (the way the MegaMoE forward uses the layout): the next launch on
+    the workspace reports it, once, and the one after that works."""
     workspace = ops.Workspace(1 << 20)
     try:
         idx = torch.randint(0, 16, (512, 4), device="cuda")
         workspace.tune("layout_barrier_extra_arrivals", 1)
         workspace.tune("layout_barrier_ticks", 10_000)
         ops.layout(workspace, idx, 16)
-        with pytest.raises(RuntimeError, match="barrier"):
-            ops.layout_wait(workspace)
         torch.cuda.synchronize()
-        with pytest.raises(RuntimeError, match="barrier"):  # the workspace stays marked
+        workspace.tune("layout_barrier_extra_arrivals", 0)
+        with pytest.raises(RuntimeError, match="barrier"):
             ops.layout(workspace, idx, 16)
-        with pytest.raises(ValueError, match="unknown key"):
-            workspace.tune("no_such_switch", 1)
+        lay = ops.layout(workspace, idx, 16)
+        _, rows = ops.layout_wait(workspace)
+        want = olayout.layout(idx.cpu().numpy(), 16)
+        assert rows == want["num_rows"]
+        np.testing.assert_array_equal(lay["route_to_row"].cpu().numpy(), want["route_to_row"])
     finally:
         workspace.destroy()
 

@@ -170,6 +170,41 @@ def test_low_latency_dispatch_combine_rank_share(payload):
         buffer.destroy()
 
 
+def test_low_latency_capacity_above_the_batch():
+    """The usual decode set-up: a fixed num_max_tokens_per_rank above the actual batch and at least top-k experts per
+    rank, so that the capacity layout C = P*M*K holds more rows than the batch has routes (T*K).  Dispatch returns
+    [C,H], combine takes an expert output of C rows."""
+    import deepep_amd
+
+    world, rank, per_rank, capacity, hidden, experts, topk = 16, 3, 8, 32, 1024, 256, 8
+    local = experts // world
+    routes = cases.ll_routes(world, per_rank, topk, experts, seed=9)
+    idx = torch.tensor([row for source in routes for row in source])
+    sources, toks = np.repeat(np.arange(world), per_rank), np.tile(np.arange(per_rank), world)
+    x = torch.from_numpy(cases.ll_payload(sources, toks, hidden)).bfloat16().cuda()
+    w = torch.rand(world * per_rank, topk, generator=torch.Generator().manual_seed(2))
+    capacity_rows = world * capacity * min(topk, local)
+    assert capacity_rows > world * per_rank * topk
+    buffer = deepep_amd.ElasticBuffer(None, num_bytes=8 << 30, rank=rank, world_size=world, explicitly_destroy=True)
+    try:
+        recv, _, _, handle, _ = buffer.dispatch(x, topk_idx=idx.cuda(), topk_weights=w.cuda(), num_experts=experts,
+                                                num_max_tokens_per_rank=capacity)
+        assert handle.is_low_latency and tuple(recv.shape) == (capacity_rows, hidden)
+        lay = olayout.layout(idx.numpy(), experts, rank * local, local)
+        rows = lay["num_rows"]
+        assert 0 < rows == int(handle.send_counts[-1].item())
+        np.testing.assert_array_equal(bf16_bits(recv[:rows]), olayout.expand_rows(bf16_bits(x), lay["row_to_route"], topk))
+        y = torch.zeros((capacity_rows, hidden), dtype=torch.bfloat16, device="cuda")
+        y[:rows] = (recv[:rows].float() * 0.5 + 1.0).bfloat16()
+        y[rows:] = float("nan")  # the capacity tail is never read
+        out, _, _ = buffer.combine(y, handle)
+        row_w = olayout.expand_weights(w.numpy(), lay["row_to_route"])
+        np.testing.assert_array_equal(bf16_bits(out), ocombine.combine(bf16_bits(y[:rows]), lay["route_to_row"], row_w))
+        assert not buffer._runtime.notify_failed
+    finally:
+        buffer.destroy()
+
+
 def test_elastic_buffer_all_routes_masked():
     """No valid route at all: the payload kernel is queued before the host knows that R = 0; outputs are empty views,
     the handle says zero rows everywhere, and the combine of nothing is a tensor of zeros."""
