@@ -30,7 +30,7 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ row_weights, const int* __restrict__ route_to_row,
     int num_topk, int vec_per_row, int vec_per_part, int parts, u32x4* __restrict__ out,
     const float* __restrict__ return_in, float* __restrict__ return_out, const int* __restrict__ shared_first_row,
-    int num_shared, int num_tokens, int unserved_rows_are_zero, int num_rows)
+    int num_shared, int num_tokens, const int* __restrict__ fill_state, int num_rows)
 {
     __shared__ int rows[DPEP_MAX_TOPK + kBatch];
     __shared__ float wts[DPEP_MAX_TOPK + kBatch];
@@ -58,7 +58,12 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const int v_begin = part * vec_per_part;
     const int v_end = min(v_begin + vec_per_part, vec_per_row);
     if (!any_row) {
-        if (kWeights == 2 && unserved_rows_are_zero) return;  // (MegaMoE) the GEMM launches have zeroed the output
+        // (MegaMoE) rows that idle workgroups of the first GEMM have already zeroed: filler f of n took tokens
+        // f, f + n, ... and got through fill_state[1 + f] of them
+        if (kWeights == 2 && fill_state != nullptr) {
+            const int fillers = fill_state[0];
+            if (fillers > 0 && token / fillers < fill_state[1 + token % fillers]) return;
+        }
         const u32x4 zero = {0u, 0u, 0u, 0u};
         for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x)
             store16_nt(out + static_cast<size_t>(token) * vec_per_row + v, zero);
@@ -115,7 +120,7 @@ constexpr int kSparseBatch = DPEP_TUNE_SPARSE_BATCH;  // 16-byte vectors per lan
 constexpr int kSparseWaves = DPEP_TUNE_SPARSE_WAVES;  // tokens (= waves) per workgroup
 __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ route_weights, const int* __restrict__ route_to_row,
-    int num_topk, int vec_per_row, u32x4* __restrict__ out, int num_tokens, int unserved_rows_are_zero)
+    int num_topk, int vec_per_row, u32x4* __restrict__ out, int num_tokens, const int* __restrict__ fill_state)
 {
     const int lane = threadIdx.x & 63;
     const int token = blockIdx.x * kSparseWaves + (threadIdx.x >> 6);
@@ -129,7 +134,10 @@ __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
     const uint64_t valid = __ballot(row >= 0);
     u32x4* dst = out + static_cast<size_t>(token) * vec_per_row;
     if (valid == 0ull) {
-        if (unserved_rows_are_zero) return;  // the GEMM launches have zeroed the output
+        if (fill_state != nullptr) {  // rows that idle workgroups of the first GEMM have already zeroed
+            const int fillers = fill_state[0];
+            if (fillers > 0 && token / fillers < fill_state[1 + token % fillers]) return;
+        }
         const u32x4 zero = {0u, 0u, 0u, 0u};
         for (int v = lane; v < vec_per_row; v += 64) store16_nt(dst + v, zero);
         return;
@@ -204,11 +212,11 @@ template <int kWeights, bool kHalf = false>
 void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, const float* weights, const int32_t* route_to_row,
                     int num_topk, int vec, void* out, const float* return_in, float* return_out,
                     int num_rows, const int32_t* shared_first_row = nullptr, int num_shared = 0, int num_tokens = 0,
-                    int unserved_rows_are_zero = 0)
+                    const int32_t* fill_state = nullptr)
 {
     hipLaunchKernelGGL((combine_kernel<kWeights, kHalf>), dim3(g.blocks), dim3(g.threads), 0, stream, static_cast<const u32x4*>(y),
                        weights, route_to_row, num_topk, vec, g.per_part, g.parts, static_cast<u32x4*>(out), return_in,
-                       return_out, shared_first_row, num_shared, num_tokens, unserved_rows_are_zero, num_rows);
+                       return_out, shared_first_row, num_shared, num_tokens, fill_state, num_rows);
 }
 
 }  // namespace
@@ -216,18 +224,18 @@ void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, con
 // Route-weighted reduce used by the MegaMoE forward: out[t] = bf16( sum_s w[t,s] * float(y[row(t,s)]) ).
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
                    int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
-                   bool unserved_rows_are_zero, hipStream_t stream)
+                   const int32_t* fill_state, hipStream_t stream)
 {
     const int vec = hidden / 8;
     if (num_shared == 0 && 2LL * num_rows_hint < num_tokens) {  // a sparse share: most tokens own no row
         hipLaunchKernelGGL(combine_sparse_kernel, dim3((num_tokens + kSparseWaves - 1) / kSparseWaves), dim3(64 * kSparseWaves), 0, stream,
                            static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk, vec, static_cast<u32x4*>(out),
-                           num_tokens, unserved_rows_are_zero ? 1 : 0);
+                           num_tokens, fill_state);
         return launch_status("combine_routes_sparse");
     }
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
     launch_combine<2>(g, stream, y, route_weights, route_to_row, num_topk, vec, out, nullptr, nullptr, 0x7fffffff,
-                      shared_first_row, num_shared, num_tokens, unserved_rows_are_zero ? 1 : 0);
+                      shared_first_row, num_shared, num_tokens, fill_state);
     return launch_status("combine_routes");
 }
 

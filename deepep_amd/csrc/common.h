@@ -51,13 +51,15 @@ struct Workspace {
     int layout_one_launch;
     uint32_t layout_launches;  // number of the most recent layout launch (never 0)
     uint32_t timeout_seen;     // number of the last timed-out launch the host has been told about
+    uint32_t gemm_launches;    // number of the most recent MegaMoE forward (never 0)
+    int gemm_zero_fill;        // 1 (default): idle workgroups of the first GEMM zero rows of unserved tokens; 0: the reduce does
     int gemm_tile_rows;  // 0: the grouped GEMM chooses its tile height; 64 / 128 / 192: forced (tests)
 };
 // Small words the kernels synchronise through, zero when the workspace is created and left zero by every launch:
-// the layout's barrier at offset 0 (two counters), and from kSyncArrivals on one arrival counter per workgroup of
-// the grouped GEMM (tiles whose k range several workgroups share).
-constexpr size_t kSyncBytes = 8192;
-constexpr size_t kSyncArrivals = 1024;  // int[1024] up to kSyncBytes - 3072
+// the layout's barrier at offset 0 (two counters); the word at kSyncFillStop, through which the MegaMoE fillers are
+// told to stop, holds the number of the launch that wrote it last and needs no clearing.
+constexpr size_t kSyncBytes = 256;
+constexpr size_t kSyncFillStop = 64;
 constexpr int kMailboxTimeout = 2 + DPEP_MAX_LOCAL_EXPERTS;  // a layout kernel whose barrier wait ran out leaves its launch number here
 constexpr int kMailboxWords = 3 + DPEP_MAX_LOCAL_EXPERTS;
 constexpr long long kLayoutBarrierTicks = 200000000;  // 2 s

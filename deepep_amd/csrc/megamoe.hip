@@ -23,7 +23,7 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
                int32_t* row_to_route, int32_t* num_rows, hipStream_t stream);
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
                    int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
-                   bool unserved_rows_are_zero, hipStream_t stream);
+                   const int32_t* fill_state, hipStream_t stream);
 
 namespace {
 
@@ -147,13 +147,9 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
 // Grouped GEMM
 // =====================================================================================================
 // Workgroup = 4 waves (2 row halves x 2 column halves), tile (64*RT) rows x 256 columns, k tile 128
-// (two MFMA k steps) per LDS stage.  Workgroups are persistent (one per CU); the launch's work is ONE flat
-// stream of (tile, k tile) items, tile-major, and every workgroup takes a consecutive range of it
-// (gemm_schedule.h): asynchronous global->LDS copies run kAhead items ahead of the MFMAs and roll straight
-// into the next tile, so a tile's epilogue overlaps the next tile's first copies.  Where whole tiles do not deal
-// out evenly over the CUs the ranges are equal shares of the stream instead: a tile's k range is then covered by
-// two or more workgroups, each leaves its fp32 partial sums in the workspace, and the last one to arrive adds the
-// others' to its own and runs the epilogue (no workgroup ever waits for another).
+// (two MFMA k steps) per LDS stage.  Workgroups are persistent (one per CU) and treat their tiles as ONE
+// flat stream of (tile, k tile) items: asynchronous global->LDS copies run kAhead items ahead of the
+// MFMAs and roll straight into the next tile, so a tile's epilogue overlaps the next tile's first copies.
 // Per item there is one vmcnt wait + one barrier; the fragments of the next k step leave LDS while the
 // MFMAs of the current one run.  A wave owns its SIMD alone and issues in order, so everything that is not
 // an MFMA is placed in the shadow of one: the MFMAs are volatile asm statements (they keep source order;
@@ -163,9 +159,6 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
 // the next tile's gather indices (once per tile) are fetched per span of four items.
 // Rows are fetched 128 bytes at a time (full cache lines): the texture path handles about one line per
 // cycle and CU, which a 64-byte k tile would saturate.
-// A launch may also be given a range of the final output to zero (the rows of tokens that no local expert
-// serves, most of a rank's share): every wave then sends a few 1 KiB zero stores per item into its part of that
-// range, a steady trickle beside the weight stream instead of a burst of its own after the GEMMs.
 constexpr int kBK = 128;           // k per LDS stage = two MFMA k steps
 constexpr int kCT = 4;             // 32-column MFMA tiles per wave
 constexpr int kBN = 2 * kCT * 32;  // columns per workgroup tile
@@ -173,9 +166,8 @@ constexpr int kGemmThreads = 256;
 constexpr int kGemmWaves = kGemmThreads / 64;
 constexpr int kMaxMoeExperts = 128;
 constexpr int kStagingRowStride = 80;  // 32 BF16 + 16 B pad: conflict-free 16-byte reads
-constexpr int kMaxGemmWorkers = 1024;  // workgroups of a launch (one per CU)
 
-template <int RT>
+template <int RT, bool kGather>
 struct GemmCfg : GemmRing<RT> {
     using GemmRing<RT>::kStages;
     static constexpr int kBM = 64 * RT;
@@ -193,9 +185,7 @@ struct GemmCfg : GemmRing<RT> {
     static constexpr int kStagingWave = 32 * kStagingRowStride;  // the epilogue handles one 32-row tile at a time
     static constexpr int kOffStaging = kOffColScales + 2 * kColScaleSlot;
     static constexpr int kLdsBytes = kOffStaging + 4 * kStagingWave;
-    static constexpr size_t kPartialBytes = static_cast<size_t>(kBM) * kBN * 4;  // one workgroup's accumulators
 };
-constexpr size_t kMaxPartialBytes = GemmCfg<3>::kPartialBytes;
 
 struct GemmParams {
     const uint8_t* a_codes;    // [*, K] e4m3
@@ -213,15 +203,21 @@ struct GemmParams {
     uint8_t* act_codes;        // first GEMM: [rows, N/2] e4m3
     uint8_t* act_scales;       //             [rows, N/64] e8m0
     uint16_t* out;             // second GEMM: [rows, N] bf16
-    // Tiles whose k range is shared between workgroups: worker w leaves the accumulators of the piece at the head of
-    // its range in partials[2 * w] and of the piece at its tail in partials[2 * w + 1] (kMaxPartialBytes each), and
-    // counts its arrival in arrivals[first worker of the tile] (all zero between launches).
-    uint8_t* partials;
-    int* arrivals;
-    // 1 KiB blocks [zero_begin, zero_end) of zero_out that this launch sets to zero (nullptr: none).
-    u32x4* zero_out;
-    long long zero_begin, zero_end;
-    int forced_rt;  // 1..3: tile height 64 * forced_rt whatever the cost model says (tests); 0: the model decides
+    // Zero rows of the final output.  When a launch has fewer tiles than workgroups, the workgroups left
+    // without a tile stream zeros into the output rows of the tokens that no local expert serves (most tokens of a
+    // rank's share), which the weighted reduce would otherwise have to write after the GEMMs: the stores cost the
+    // matrix pipes nothing.  Every wave of such a workgroup is a filler f and takes tokens f, f + fillers, ...
+    // until a workgroup with a tile reaches its epilogue and writes the launch's number into *fill_stop (a number,
+    // not a flag, so that nothing has to clear it and a word left over from an earlier launch stops nobody);
+    // fill_state[0] = number of fillers, fill_state[1 + f] = tokens filler f got through.  All of it is null / zero in
+    // launches that do not fill.
+    u32x4* fill_out;                // [fill_tokens, fill_vec] or nullptr
+    const int* fill_route_to_row;   // [fill_tokens, fill_topk]
+    int fill_tokens, fill_vec, fill_topk;
+    int* fill_state;
+    int* fill_stop;
+    int launch_id;                  // never 0
+    int forced_rt;                  // 1..3: tile height 64 * forced_rt whatever the cost model says (tests); 0: the model decides
 };
 
 // gate / (1 + exp(-gate)) * up with the hardware exponential and reciprocal (about 1 ulp each; the
@@ -235,7 +231,12 @@ __device__ __forceinline__ float silu_mul(float gate, float up)
 // Asynchronous copy global -> LDS: lane l's bytes land at lds_base + l * size.  lds_base is wave-uniform.
 // Written as assembly so that the compiler's own wait-count bookkeeping does not serialise the ring;
 // completion is awaited explicitly with wait_copies_then_barrier<N>().
-// The address is split into a wave-uniform 64-bit base (SGPR pair) and a 32-bit lane offset.
+__device__ __forceinline__ void copy16_to_lds(const void* src, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(src) : "memory");
+}
+// The same with the address split into a wave-uniform 64-bit base (SGPR pair) and a 32-bit lane offset.
 __device__ __forceinline__ void copy16_to_lds(const void* uniform_base, uint32_t lane_offset, uint32_t lds_base)
 {
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
@@ -248,7 +249,7 @@ __device__ __forceinline__ void copy4_to_lds(const void* src, uint32_t lds_base)
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(src) : "memory");
 }
-// The same copies, skipped when the (wave-uniform) value skip is not zero.  The jump stays inside
+// The same 16-byte copy, skipped when the (wave-uniform) value skip is not zero.  The jump stays inside
 // the asm statement so that the loop body around it remains straight-line code.
 __device__ __forceinline__ void copy16_to_lds_unless(const void* src, uint32_t lds_base, int skip)
 {
@@ -270,42 +271,13 @@ __device__ __forceinline__ void copy4_to_lds_unless(const void* src, uint32_t ld
         "v"(src), "s"(flag)
         : "memory", "scc");
 }
-// kZeroPerItem streaming 16-byte zero stores per lane (1 KiB per wave each) at uniform_base + lane_offset + j KiB,
-// skipped when skip is not zero.
-__device__ __forceinline__ void zero_stores_unless(void* uniform_base, uint32_t lane_offset, const u32x4& zero, int skip)
-{
-    static_assert(kZeroPerItem == 4, "the statement below issues four stores");
-    const int flag = __builtin_amdgcn_readfirstlane(skip);
-    asm volatile(
-        "s_cmp_lg_u32 %3, 0\n\ts_cbranch_scc1 .Lskip_zero_%=\n\t"
-        "global_store_dwordx4 %0, %1, %2 nt\n\t"
-        "global_store_dwordx4 %0, %1, %2 offset:1024 nt\n\t"
-        "global_store_dwordx4 %0, %1, %2 offset:2048 nt\n\t"
-        "global_store_dwordx4 %0, %1, %2 offset:3072 nt\n.Lskip_zero_%=:" ::"v"(lane_offset),
-        "v"(zero), "s"(uniform_base), "s"(flag)
-        : "memory", "scc");
-}
 // Also waits for the wave's own LDS reads: past the barrier nothing reads the stage that is refilled next.
-// (Never weaken this for a timing experiment: the gather indices of the next tile travel through LDS too, so a
-// wave that runs ahead of a copy reads a stale index and fetches from a wild address.)
 template <int kOutstanding>
 __device__ __forceinline__ void wait_copies_then_barrier()
 {
+    // (Never weaken this for a timing experiment: the gather indices of the next tile travel through LDS too, so a
+    // wave that runs ahead of a copy reads a stale index and fetches from a wild address.)
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
-}
-// The same with the more generous count when `zeroing` (wave-uniform) is not zero.
-template <int kPlain, int kZeroing>
-__device__ __forceinline__ void wait_copies_then_barrier(int zeroing)
-{
-    static_assert(kZeroing <= 63 && kPlain <= kZeroing, "vmcnt is a 6-bit counter");
-    const int flag = __builtin_amdgcn_readfirstlane(zeroing);
-    asm volatile(
-        "s_cmp_lg_u32 %2, 0\n\ts_cbranch_scc1 .Lwait_zeroing_%=\n\t"
-        "s_waitcnt vmcnt(%0)\n\ts_branch .Lwait_done_%=\n"
-        ".Lwait_zeroing_%=:\n\ts_waitcnt vmcnt(%1)\n"
-        ".Lwait_done_%=:\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(kPlain),
-        "n"(kZeroing), "s"(flag)
-        : "memory", "scc");
 }
 
 // One scaled MFMA (FP8 A, FP4 B) as a volatile asm statement: volatile statements keep their source order,
@@ -339,13 +311,12 @@ template <int RT, bool kGateUp>
 __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParams p)
 {
     constexpr bool kGather = kGateUp;
-    using Cfg = GemmCfg<RT>;
+    using Cfg = GemmCfg<RT, kGather>;
     constexpr int kBM = Cfg::kBM, kStages = Cfg::kStages, kAhead = Cfg::kAhead, kStageBytes = Cfg::kStageBytes;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     __shared__ int tile_base[kMaxMoeExperts + 1];
     __shared__ int row_offsets[kMaxMoeExperts + 1];
     __shared__ int tile_index[2][kGemmThreads];  // row_to_route of a tile's rows; slots alternate per tile
-    __shared__ int arrival_order;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS copy targets in SGPRs
@@ -372,40 +343,36 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     __syncthreads();
     const int total_tiles = tile_base[p.num_local];
 
-    // Consecutive ranges of the item stream share weights; workgroups are dealt round-robin over the 8 XCDs, so
-    // worker numbers are chosen such that each XCD holds a consecutive run of ranges and its L2 sees each weight
-    // tile from one place.
-    const int grid = gridDim.x;
-    const int worker = (grid & 7) == 0 ? (blockIdx.x & 7) * (grid >> 3) + (blockIdx.x >> 3) : blockIdx.x;
-    const WorkSplit split = choose_split(total_tiles, ktiles, grid);
-    const WorkRange range = worker_range(split, worker);
-    const int sp = split.spans_per_tile;
-    const int n_items = static_cast<int>(range_items(split, range, ktiles));
-
-    // This wave's part of the output range to zero, in 1 KiB blocks.
-    const u32x4 zero = {0u, 0u, 0u, 0u};
-    long long zero_at = 0, zero_end = 0;
-    if (p.zero_out != nullptr) {
-        const long long blocks = p.zero_end - p.zero_begin;
-        const long long part = static_cast<long long>(worker) * kGemmWaves + wave, parts = static_cast<long long>(grid) * kGemmWaves;
-        zero_at = p.zero_begin + blocks * part / parts;
-        zero_end = p.zero_begin + blocks * (part + 1) / parts;
-    }
-    // Whatever the items did not carry (all of it for a workgroup without a range) goes out in one piece at the end.
-    auto zero_the_rest = [&]() {
-        for (long long b = zero_at; b < zero_end; ++b) store16_nt(p.zero_out + b * 64 + lane, zero);
-    };
-    if (n_items == 0) {
-        zero_the_rest();
+    // Consecutive tile ids share weights; give each XCD (workgroups are dealt round-robin over 8 XCDs)
+    // a contiguous range of tiles so that its L2 sees each weight tile from one place.  With fewer tiles than
+    // workgroups: a launch that fills keeps the ranges whole, so that the first XCDs are full and the workgroups
+    // without a tile, the fillers, sit together on the XCDs left over (their stores then stay out of the L2s the
+    // GEMM works from: fillers on every XCD fill faster but cost the GEMM three times as much); a launch that
+    // does not fill shrinks the ranges evenly (about 4 % faster than leaving two XCDs idle).
+    const bool one_round = total_tiles < static_cast<int>(gridDim.x);
+    const int fillers = one_round && p.fill_out != nullptr ? (static_cast<int>(gridDim.x) - total_tiles) * kGemmWaves : 0;
+    const bool spread = one_round && fillers == 0 && (gridDim.x & 7) == 0;
+    const int per_xcd = spread ? (total_tiles + 7) / 8 : (gridDim.x + 7) / 8;
+    const int first = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    const int stride = one_round ? total_tiles + 1 : per_xcd * 8;  // one round: a single tile each
+    const bool has_tile = first < total_tiles && (!spread || static_cast<int>(blockIdx.x >> 3) < per_xcd);
+    if (blockIdx.x == 0 && tid == 0 && p.fill_state != nullptr) p.fill_state[0] = fillers;  // workgroup 0 always has tile 0
+    if (!has_tile) {
+        if (fillers == 0) return;
+        const int filler = (first - total_tiles) * kGemmWaves + wave;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        int done = 0;
+        for (int token = filler; token < p.fill_tokens; token += fillers, ++done) {
+            if (__hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.launch_id) break;
+            const bool mine = lane < p.fill_topk && p.fill_route_to_row[static_cast<size_t>(token) * p.fill_topk + lane] >= 0;
+            if (__ballot(mine) != 0ull) continue;  // some local expert serves the token: the reduce writes its row
+            u32x4* row = p.fill_out + static_cast<size_t>(token) * p.fill_vec;
+            for (int v = lane; v < p.fill_vec; v += 64) store16_nt(row + v, zero);
+        }
+        if (lane == 0) p.fill_state[1 + filler] = done;
         return;
     }
-    const int zero_items = static_cast<int>(min(static_cast<long long>(n_items), (zero_end - zero_at) / kZeroPerItem));
-    uint8_t* zero_base = reinterpret_cast<uint8_t*>(p.zero_out) + zero_at * 1024;  // wave-uniform
-    zero_at += static_cast<long long>(zero_items) * kZeroPerItem;  // what zero_the_rest() has left to do
-
-    const int first_tile = static_cast<int>(range.begin / sp);
-    const int first_kt = static_cast<int>(range.begin % sp) * kSpanItems;
-    const int last_tile = static_cast<int>((range.end - 1) / sp);
+    const int my_tiles = one_round ? 1 : (total_tiles - first + stride - 1) / stride;
 
     auto decode = [&](int tile) {
         int e = 0;
@@ -431,11 +398,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     const uint8_t* b_base = p.w;
     const uint8_t* sb_src;
     const int* index_src = p.row_to_route;
-    int copy_tile = first_tile, copy_kt = first_kt, copy_stage = 0, copy_span = -1, copy_ordinal = 0;
-    int copy_left = n_items;    // items of the range the cursor has not issued yet
-    int tile_items_issued = 0;  // items of copy_tile this workgroup has issued
+    int copy_tile = first, copy_kt = 0, copy_stage = 0, copy_span = -1, copy_ordinal = 0;
     const int scale_bytes = p.k / 32;  // per row
-    TileInfo next_info = decode(first_tile);
+    const int spans = (ktiles + 3) / 4;
+    TileInfo next_info = decode(first);
 
     // Tile number j of this workgroup keeps its gather indices in tile_index[j & 1].
     auto point_at_tile = [&](const TileInfo& info) {
@@ -463,7 +429,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             const int q = j * 4 + wave;
             b_off[j] = static_cast<uint32_t>(q * 1024 + lane * 16);
         }
-        sb_src = (shared ? p.ws_shared : p.ws) + (weight_index * n_tiles + info.nt) * sp * Cfg::kColScaleSlot + tid * 16;
+        sb_src = (shared ? p.ws_shared : p.ws) + (weight_index * n_tiles + info.nt) * spans * Cfg::kColScaleSlot + tid * 16;
     };
     auto aim_index_prefetch = [&](const TileInfo& info) {
         if (kGather) index_src = p.row_to_route + info.row0 + min(tid, info.valid - 1);
@@ -479,8 +445,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                           stage + Cfg::kOffB + ((c - 2 * RT) * 4 + wave) * 1024);
     };
     // Every fourth item starts a new span: a 16-byte window of row scales per row (clamped so that it never
-    // leaves the row: k % 512 may be 256) and the span's 4 KiB of column scales.  The first item a workgroup issues
-    // of a tile also fetches the gather indices of its next tile.  These extra copies only make the counted
+    // leaves the row: k % 512 may be 256) and the span's 4 KiB of column scales.  A tile's first item also
+    // fetches the gather indices of the workgroup's next tile.  These extra copies only make the counted
     // waits stricter.
     auto issue_span_copies = [&]() {
         copy_span += (copy_kt & 3) == 0 ? 1 : 0;
@@ -490,28 +456,25 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                              copy_kt & 3);
         copy16_to_lds_unless(sb_src + static_cast<size_t>(copy_kt >> 2) * Cfg::kColScaleSlot,
                              lds0 + Cfg::kOffColScales + slot * Cfg::kColScaleSlot + wave * 1024, copy_kt & 3);
-        if (kGather)
-            copy4_to_lds_unless(index_src, lds_index + ((copy_ordinal + 1) & 1) * (kGemmThreads * 4) + wave * 256, tile_items_issued);
+        if (kGather) copy4_to_lds_unless(index_src, lds_index + ((copy_ordinal + 1) & 1) * (kGemmThreads * 4) + wave * 256, copy_kt);
     };
-    // Past the last item of the range the cursor stays on it and keeps re-copying it (never read).
     auto advance_copy_cursor = [&](bool in_prologue) {
         copy_stage = copy_stage + 1 == kStages ? 0 : copy_stage + 1;
-        ++tile_items_issued;
-        if (--copy_left <= 0) {
-            copy_left = 0;
-            return;
-        }
         if (++copy_kt == ktiles) {
-            // The next tile's indices were fetched with the first item this workgroup issued of this tile; they
-            // have landed unless that was too recent for any wait to have covered it (gemm_schedule.h).
-            if (kGather && switch_needs_drain(in_prologue, tile_items_issued, kAhead)) wait_copies_then_barrier<0>();
-            ++copy_tile;
-            copy_kt = 0;
-            ++copy_ordinal;
-            tile_items_issued = 0;
-            point_at_tile(next_info);
-            if (copy_tile < last_tile) next_info = decode(copy_tile + 1);
-            aim_index_prefetch(next_info);
+            if (copy_tile + stride < total_tiles) {
+                // The next tile's indices were fetched with this tile's first item, so switching needs no global
+                // load; they have landed unless the tile is too short for any counted wait to have covered that
+                // fetch (gemm_schedule.h), in which case the cursor lets everything land first.
+                if (kGather && switch_needs_drain(in_prologue, ktiles, kAhead)) wait_copies_then_barrier<0>();
+                copy_tile += stride;
+                copy_kt = 0;
+                ++copy_ordinal;
+                point_at_tile(next_info);
+                if (copy_tile + stride < total_tiles) next_info = decode(copy_tile + stride);
+                aim_index_prefetch(next_info);
+            } else {
+                copy_kt = ktiles - 1;  // past the last tile: keep re-copying its last item (never read)
+            }
         }
     };
     auto issue_item = [&]() {
@@ -528,7 +491,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         wait_copies_then_barrier<0>();
     }
     point_at_tile(next_info);
-    if (first_tile < last_tile) next_info = decode(first_tile + 1);
+    if (first + stride < total_tiles) next_info = decode(first + stride);
     aim_index_prefetch(next_info);
 
     // ---- fragment addresses inside a stage ---------------------------------------------------------
@@ -606,6 +569,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         // The staging region holds one 32 x 32 tile as BF16 rows.
 #pragma unroll
         for (int i = 0; i < RT; ++i) {
+            // The last row tile of the epilogue is about what a filler needs to finish the row it is on: tell them to
+            // stop (the first workgroup to get here does; the others are at most a few microseconds behind).
+            if (i == RT - 1 && fillers != 0 && tid == 0)
+                __hip_atomic_store(p.fill_stop, p.launch_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int tile_rows = min(32, info.valid - wm * 32 * RT - 32 * i);  // may be <= 0
             const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT + 32 * i;
 #pragma unroll
@@ -680,84 +647,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         }
     };
 
-    // ---- a piece that is not a whole tile ------------------------------------------------------------
-    // The workers of a tile are consecutive; the first one's piece lies at the tail of its range (slot 1), the
-    // others' at the head of theirs (slot 0).  A partial is this workgroup's accumulators as they sit in the
-    // registers: [wave][row tile][column tile][register pair][lane] x 8 bytes.  Partials are written and read with
-    // device-scope accesses that go past the per-XCD caches, so the arrival counter only has to order them: every
-    // thread waits until its own stores are acknowledged before the workgroup's arrival is counted.
-    // Returns true for the workgroup that arrives last, with the tile's full sums in acc.
-    auto partial_of = [&](int w, int first_worker) {
-        return reinterpret_cast<unsigned long long*>(p.partials + (static_cast<size_t>(w) * 2 + (w == first_worker ? 1 : 0)) * kMaxPartialBytes) +
-               static_cast<size_t>(wave) * (RT * kCT * 8 * 64) + lane;
-    };
-    // The tile's sums from the partials of workers [from, to], one row tile (32 loads of 8 bytes per lane and
-    // partial) at a time: more in flight would not fit the registers.  keep_own: this workgroup's own piece is taken
-    // from its accumulators as they are, the others are added to it.
-    auto sum_partials = [&](int from, int to, int first_worker, bool keep_own) {
-#pragma unroll
-        for (int i = 0; i < RT; ++i) {
-            if (!keep_own) {
-#pragma unroll
-                for (int c = 0; c < kCT; ++c)
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) acc[i][c][j] = 0.0f;
-            }
-            for (int w = from; w <= to; ++w) {
-                if (keep_own && w == worker) continue;
-                const unsigned long long* src = partial_of(w, first_worker);
-                unsigned long long pair[kCT][8];
-#pragma unroll
-                for (int c = 0; c < kCT; ++c)
-#pragma unroll
-                    for (int q = 0; q < 8; ++q)
-                        pair[c][q] = __hip_atomic_load(src + ((i * kCT + c) * 8 + q) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                for (int c = 0; c < kCT; ++c)
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) {
-                        acc[i][c][2 * q] += __uint_as_float(static_cast<uint32_t>(pair[c][q]));
-                        acc[i][c][2 * q + 1] += __uint_as_float(static_cast<uint32_t>(pair[c][q] >> 32));
-                    }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    auto exchange_partials = [&](int tile) -> bool {
-        const long long tile_begin = static_cast<long long>(tile) * sp;
-        const int first_worker = span_owner(split, tile_begin), last_worker = span_owner(split, tile_begin + sp - 1);
-        const int pieces = last_worker - first_worker + 1;
-        unsigned long long* mine = partial_of(worker, first_worker);
-#pragma unroll
-        for (int i = 0; i < RT; ++i) {
-#pragma unroll
-            for (int c = 0; c < kCT; ++c)
-#pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    const unsigned long long pair = static_cast<unsigned long long>(__float_as_uint(acc[i][c][2 * q])) |
-                                                    (static_cast<unsigned long long>(__float_as_uint(acc[i][c][2 * q + 1])) << 32);
-                    __hip_atomic_store(mine + ((i * kCT + c) * 8 + q) * 64, pair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        wait_copies_then_barrier<0>();  // every thread's stores are acknowledged
-        if (tid == 0)
-            arrival_order = __hip_atomic_fetch_add(p.arrivals + first_worker, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        if (arrival_order != pieces - 1) return false;
-        if (tid == 0) __hip_atomic_store(p.arrivals + first_worker, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // Two pieces: own + other gives the same bits whichever of the two arrives last.  More than two: all of them
-        // from memory in worker order, own one included, so that the result does not depend on who arrived last.
-        sum_partials(first_worker, last_worker, first_worker, pieces == 2);
-        return true;
-    };
-
     // ---- the flat item stream --------------------------------------------------------------------------
 #pragma unroll
     for (int j = 0; j < kAhead; ++j) issue_item();
     wait_copies_then_barrier<(kAhead - 1) * Cfg::kCopies>();  // item 0 has landed
     // Scale bookkeeping of the item whose fragments are read next: span counter (ring slot) and k tile.
-    int read_span = -1, read_kt = first_kt;
+    int read_span = -1, read_kt = 0;
     int row_at = 0, col_at = 0;
     auto next_scale_offsets = [&]() {
         if ((read_kt & 3) == 0) ++read_span;
@@ -776,19 +671,18 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     clear_acc();
     asm volatile("s_nop 3");
     int stage_now = 0;  // stage of the item whose MFMAs run
-    int tile = first_tile, kt = first_kt;
-    int piece_begin = first_kt;  // k tile the piece in the accumulators started at
-    int item = 0;
-    TileInfo info = decode(first_tile);
-    for (int left = n_items; left > 0; left -= 2) {
+    int tile = first, kt = 0;
+    TileInfo info = decode(first);
+    const long long total_items = static_cast<long long>(my_tiles) * ktiles;
+    for (long long item = 0; item < total_items; item += 2) {
 #pragma unroll
-        for (int parity = 0; parity < 2; ++parity) {  // ktiles and span lengths are even, so pieces start on even items
+        for (int parity = 0; parity < 2; ++parity) {  // ktiles is even, so tiles start on even items
             const int stage_next = stage_now + 1 == kStages ? 0 : stage_now + 1;
             // A wave issues in order and owns its SIMD alone, so whatever is not an MFMA should sit in the
             // shadow of one.  First k step: its MFMAs are followed, one piece each, by the LDS reads of the
-            // second k step's fragments and, once the barrier has passed, by the zero stores and the copies of the
-            // item kAhead ahead.  Second k step: the remaining copies and the reads of the next item's scales and
-            // first fragments (whose registers the first k step has released).
+            // second k step's fragments and, once the barrier has passed, by the copies of the item kAhead
+            // ahead.  Second k step: the remaining copies and the reads of the next item's scales and first
+            // fragments (whose registers the first k step has released).
             shift_scales(parity);
             constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
             // enough read groups per MFMA that the second k step's fragments have all left LDS before the barrier
@@ -802,9 +696,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                 if (n == kMfmas / 2 - 1) {
                     // item+1 has landed for every thread once each has at most kAhead-2 items of its own copies
                     // in flight; past the barrier every wave has also finished reading the stage refilled next.
-                    wait_copies_then_barrier<Cfg::kWaitPlain, Cfg::kWaitZeroing>(wait_counts_zero_stores(item, zero_items, kAhead));
-                    zero_stores_unless(zero_base, lane * 16, zero, item >= zero_items);
-                    zero_base += item < zero_items ? kZeroPerItem * 1024 : 0;
+                    wait_copies_then_barrier<Cfg::kWaitPlain>();
                 }
                 if (n >= kMfmas / 2) {
                     const int slot = n - kMfmas / 2;
@@ -831,32 +723,25 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             issue_span_copies();
             advance_copy_cursor(false);
             stage_now = stage_next;
-            ++item;
         }
         kt += 2;
-        const bool tile_ends = kt == ktiles;
-        if (tile_ends || left == 2) {
-            settle_accumulators();
+        if (kt == ktiles) {
+                    settle_accumulators();
             // tie every accumulator to a statement behind the wait, so that no read of it can be moved above
 #pragma unroll
             for (int i = 0; i < RT; ++i)
 #pragma unroll
                 for (int c = 0; c < kCT; ++c) asm volatile("" : "+a"(acc[i][c]));
-            const bool whole = tile_ends && piece_begin == 0;
-            if (whole || exchange_partials(tile)) epilogue(info);
-            clear_acc();
+            epilogue(info);
+                    clear_acc();
             asm volatile("s_nop 3");  // accumulator writes settle before the next MFMA reads them
-            if (tile_ends) {
-                kt = 0;
-                ++tile;
-                if (left > 2) info = decode(tile);
-            }
-            piece_begin = kt;
+            kt = 0;
+            tile += stride;
+            if (tile < total_tiles) info = decode(tile);
         }
     }
     // No copy may still be in flight into this workgroup's LDS when it retires.
     wait_copies_then_barrier<0>();
-    zero_the_rest();
 }
 
 // Shared experts take every token: their rows follow the routed ones, expert-major, token order.
@@ -889,14 +774,13 @@ int gemm_grid()
         int value = 0;
         if (hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0) cus = value;
     }
-    cus = cus / 8 * 8;  // one resident workgroup per CU (the LDS ring takes most of the 160 KiB)
-    return cus > kMaxGemmWorkers ? kMaxGemmWorkers : cus;
+    return cus / 8 * 8;  // one resident workgroup per CU (the LDS ring takes most of the 160 KiB)
 }
 
 template <int RT, bool kGateUp>
 int launch_gemm_rt(const GemmParams& p, hipStream_t stream, const char* what)
 {
-    constexpr int kLds = GemmCfg<RT>::kLdsBytes;
+    constexpr int kLds = GemmCfg<RT, kGateUp>::kLdsBytes;
     static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
     if (!configured) {
         DPEP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<RT, kGateUp>),
@@ -910,9 +794,9 @@ int launch_gemm_rt(const GemmParams& p, hipStream_t stream, const char* what)
 // Row-tile height: the cheapest of 64 / 128 / 192 rows by a small cost model, judged from the expected rows per expert (the true counts
 // stay on the device).  Routing scatters the counts around that mean (about +-sqrt(mean)), and one expert a few
 // rows over a multiple of the tile height costs a whole extra row tile each: the tile count is therefore the
-// expectation of ceil(rows / height) under a normal spread, not ceil(mean / height).  Where the tiles do not fill
-// whole rounds of the CUs the kernel deals out equal shares of the item stream instead (gemm_schedule.h), so the
-// cost is then the tiles' work divided by the CUs plus the exchange of partial sums, not a number of rounds.
+// expectation of ceil(rows / height) under a normal spread, not ceil(mean / height).  (Mean 256 over 8 experts:
+// 128-row tiles need 2.5 row tiles per expert on average = 320 tiles = two rounds on 256 CUs, 192-row tiles need
+// 2 = one round; measured 103 vs 80 us.)
 template <bool kGateUp>
 int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t stream, const char* what)
 {
@@ -927,16 +811,15 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
         double m_tiles = 1.0;  // E[ceil(X / bm)] = sum over j >= 0 of P(X > j * bm)
         for (int j = 1; j * bm < mean + 6.0 * sigma; ++j) m_tiles += 0.5 * erfc((j * bm - mean) / (sigma * 1.4142135623730951));
         const double tiles = p.num_local * m_tiles * n_tiles;
+        const double rounds = ceil(tiles / cus - 0.02);  // a stray tile in one launch out of fifty does not count
         // Microseconds per tile, fitted to kernel traces on an MI355X over shares from 32 to 512 rows per expert,
-        // 4 to 32 experts and two problem sizes: a fixed part (prologue, epilogue) plus a part per k tile;
+        // 4 to 32 experts and two problem sizes (it reproduced the measured order of the three heights in 14 of 16
+        // cases, and was within 7 % in the other two): a fixed part (prologue, epilogue) plus a part per k tile;
         // an expert with a single row tile streams its weight tile from HBM with nobody to share it with, which
         // adds about 0.3 us per k tile whatever the height.
-        constexpr double kFixed[3] = {4.2, 2.9, 7.9}, kPerItem[3] = {0.53, 0.87, 1.29}, kExchange = 5.0;
+        constexpr double kFixed[3] = {4.2, 2.9, 7.9}, kPerItem[3] = {0.53, 0.87, 1.29};
         const double per_item = kPerItem[rt - 1] + (m_tiles <= 1.2 ? 0.3 : 0.0);
-        const double per_tile = kFixed[rt - 1] + (p.k / kBK) * per_item;
-        const WorkSplit split = choose_split(static_cast<int>(tiles + 0.5), p.k / kBK, cus);
-        const double rounds = ceil(tiles / cus - 0.02);  // a stray tile in one launch out of fifty does not count
-        const double cost = split.split ? tiles / split.workers * per_tile + kExchange : (rounds < 1.0 ? 1.0 : rounds) * per_tile;
+        const double cost = (rounds < 1.0 ? 1.0 : rounds) * (kFixed[rt - 1] + (p.k / kBK) * per_item);
         if (cost < best_cost - 1e-9) {
             best_cost = cost;
             best = rt;
@@ -953,62 +836,60 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
 // ---- host replay of one workgroup's schedule ---------------------------------------------------------------
 // Vector-memory operations complete in issue order, and a wait for "at most N in flight" guarantees no more than
 // that all but the newest N have completed.  The replay issues what the kernel issues, in the kernel's order (the
-// prologue's kAhead items; per item: the counted wait, the zero stores, the copies of the item kAhead ahead with
-// their scale and index copies, the cursor's tile switch; drains and epilogue stores at piece ends), lets
-// nothing complete that a wait has not forced, and checks that every item's copies have completed when its
-// fragments are read and that the gather indices of a tile have when the cursor reads them.
+// prologue's kAhead items; per item: the counted wait, the copies of the item kAhead ahead with their scale and index
+// copies, the cursor's tile switch; epilogue stores at tile ends), lets nothing complete that a wait has not
+// forced, and checks that every item's copies have completed when its fragments are read and that the gather
+// indices of a tile have when the cursor reads them.
 struct ScheduleFault {
-    int worker, item, what;  // what: 1 = an item's copies, 2 = gather indices
+    int item, what;  // what: 1 = an item's copies, 2 = gather indices
 };
 
 template <int RT>
-bool replay_worker(const WorkSplit& split, int worker, int ktiles, int zero_blocks, int epilogue_stores, ScheduleFault* fault)
+bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, ScheduleFault* fault)
 {
     using Ring = GemmRing<RT>;
     constexpr int kAhead = Ring::kAhead, kCopies = Ring::kCopies;
-    const WorkRange range = worker_range(split, worker);
-    const int n_items = static_cast<int>(range_items(split, range, ktiles));
+    const long long n_items = static_cast<long long>(my_tiles) * ktiles;
     if (n_items == 0) return true;
-    const int sp = split.spans_per_tile;
-    const int zero_items = zero_blocks / kZeroPerItem < n_items ? zero_blocks / kZeroPerItem : n_items;
     long long issued = 0, done = 0;  // operations [0, done) have certainly completed
     auto wait = [&](long long in_flight) {
         if (issued - in_flight > done) done = issued - in_flight;
     };
-    // cursor
-    int copy_kt = static_cast<int>(range.begin % sp) * kSpanItems, copy_left = n_items, tile_items_issued = 0;
-    long long copy_item = 0;                       // ordinal of the item under the cursor within the range
-    long long index_op = -1;                       // operation that fetches the indices of the cursor's next tile
+    int copy_kt = 0, copy_tile = 0;
+    long long copy_item = 0;   // ordinal of the item under the cursor
+    long long index_op = -1;   // operation that fetches the indices of the cursor's next tile
     static thread_local long long item_last_op[1 << 16];
-    if (n_items >= (1 << 16)) return true;         // not replayed (far beyond any real range)
-    bool ok = true;
+    if (n_items >= (1 << 16)) return true;  // not replayed (far beyond any real workgroup's share)
+    bool ok = true, past_end = false;
     auto issue_copies = [&]() {
         issued += kCopies;
-        if ((copy_kt & 3) == 0) issued += 2;       // row and column scales of the span
-        if (tile_items_issued == 0) index_op = issued++;
-        if (copy_left > 0) item_last_op[copy_item] = issued - 1;
+        if ((copy_kt & 3) == 0) issued += 2;      // row and column scales of the span
+        if (copy_kt == 0) index_op = issued++;    // (re-copies past the end sit on the last k tile, never 0)
+        if (!past_end) item_last_op[copy_item] = issued - 1;
     };
     auto advance = [&](bool in_prologue, int item) {
-        ++tile_items_issued;
-        if (--copy_left <= 0) {
-            copy_left = 0;
-            return;
-        }
-        ++copy_item;
         if (++copy_kt == ktiles) {
-            if (switch_needs_drain(in_prologue, tile_items_issued, kAhead)) wait(0);
-            if (index_op >= done && ok) {
-                ok = false;
-                *fault = {worker, item, 2};
+            if (copy_tile + 1 < my_tiles) {
+                if (switch_needs_drain(in_prologue, ktiles, kAhead)) wait(0);
+                if (index_op >= done && ok) {
+                    ok = false;
+                    *fault = {item, 2};
+                }
+                ++copy_tile;
+                copy_kt = 0;
+                ++copy_item;
+            } else {
+                copy_kt = ktiles - 1;  // past the last tile: keep re-copying its last item (never read)
+                past_end = true;
             }
-            copy_kt = 0;
-            tile_items_issued = 0;
+        } else if (!past_end) {
+            ++copy_item;
         }
     };
-    auto check_item = [&](int item) {
+    auto check_item = [&](long long item) {
         if (item < n_items && item_last_op[item] >= done && ok) {
             ok = false;
-            *fault = {worker, item, 1};
+            *fault = {static_cast<int>(item), 1};
         }
     };
     ++issued;  // the first tile's own indices, fetched synchronously
@@ -1019,18 +900,15 @@ bool replay_worker(const WorkSplit& split, int worker, int ktiles, int zero_bloc
     }
     wait((kAhead - 1) * kCopies);
     check_item(0);
-    int kt = static_cast<int>(range.begin % sp) * kSpanItems, piece_begin = kt;
-    for (int item = 0; item < n_items; ++item) {
-        wait(wait_counts_zero_stores(item, zero_items, kAhead) ? Ring::kWaitZeroing : Ring::kWaitPlain);
+    int kt = 0;
+    for (long long item = 0; item < n_items; ++item) {
+        wait(Ring::kWaitPlain);
         check_item(item + 1);  // its first fragments leave LDS during this item's second k step
-        if (item < zero_items) issued += kZeroPerItem;
         issue_copies();
-        advance(false, item);
-        if (++kt == ktiles || item == n_items - 1) {
-            if (kt != ktiles || piece_begin != 0) wait(0);  // not a whole tile: the exchange of partial sums drains
+        advance(false, static_cast<int>(item));
+        if (++kt == ktiles) {
             issued += epilogue_stores;
-            if (kt == ktiles) kt = 0;
-            piece_begin = kt;
+            kt = 0;
         }
     }
     return ok;
@@ -1068,42 +946,19 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
     return launch_status("mx_quant");
 }
 
-int dpep_megamoe_schedule_check(int tile_rows, int total_tiles, int ktiles, int grid, int zero_blocks_per_wave,
-                                int epilogue_stores)
+int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores)
 {
     using namespace dpep;
     DPEP_REQUIRE(tile_rows == 64 || tile_rows == 128 || tile_rows == 192, "schedule_check: tile_rows is 64, 128 or 192");
-    DPEP_REQUIRE(total_tiles >= 0 && ktiles >= 2 && ktiles % 2 == 0 && grid >= 1 && grid <= kMaxGemmWorkers &&
-                     zero_blocks_per_wave >= 0 && epilogue_stores >= 0,
+    DPEP_REQUIRE(tiles_per_workgroup >= 0 && ktiles >= 2 && ktiles % 2 == 0 && epilogue_stores >= 0,
                  "schedule_check: bad arguments");
-    const WorkSplit split = choose_split(total_tiles, ktiles, grid);
-    // the ranges tile the span stream, in order, without gaps
-    long long at = 0;
-    for (int w = 0; w < grid; ++w) {
-        const WorkRange r = worker_range(split, w);
-        if (w >= split.workers) {
-            DPEP_REQUIRE(r.begin == r.end, "schedule_check: worker %d beyond the %d working ones has a range", w, split.workers);
-            continue;
-        }
-        DPEP_REQUIRE(r.begin == at && r.end >= r.begin, "schedule_check: worker %d starts at span %lld, expected %lld", w, r.begin, at);
-        DPEP_REQUIRE(split.split || (r.begin % split.spans_per_tile == 0 && r.end % split.spans_per_tile == 0),
-                     "schedule_check: worker %d's range cuts a tile in a launch that does not split tiles", w);
-        if (split.split)
-            for (long long span = r.begin; span < r.end; ++span)
-                DPEP_REQUIRE(span_owner(split, span) == w, "schedule_check: span %lld of worker %d is attributed to worker %d",
-                             span, w, span_owner(split, span));
-        at = r.end;
-    }
-    DPEP_REQUIRE(at == split.total_spans, "schedule_check: the ranges cover %lld of %lld spans", at, split.total_spans);
-    for (int w = 0; w < split.workers; ++w) {
-        ScheduleFault fault = {0, 0, 0};
-        const bool ok = tile_rows == 64    ? replay_worker<1>(split, w, ktiles, zero_blocks_per_wave, epilogue_stores, &fault)
-                        : tile_rows == 128 ? replay_worker<2>(split, w, ktiles, zero_blocks_per_wave, epilogue_stores, &fault)
-                                           : replay_worker<3>(split, w, ktiles, zero_blocks_per_wave, epilogue_stores, &fault);
-        if (!ok)
-            return fail(DPEP_EINVAL, "schedule_check: worker %d reads %s before any wait covers them (item %d)", fault.worker,
-                        fault.what == 1 ? "an item's copies" : "the next tile's gather indices", fault.item);
-    }
+    ScheduleFault fault = {0, 0};
+    const bool ok = tile_rows == 64    ? replay_workgroup<1>(tiles_per_workgroup, ktiles, epilogue_stores, &fault)
+                    : tile_rows == 128 ? replay_workgroup<2>(tiles_per_workgroup, ktiles, epilogue_stores, &fault)
+                                       : replay_workgroup<3>(tiles_per_workgroup, ktiles, epilogue_stores, &fault);
+    if (!ok)
+        return fail(DPEP_EINVAL, "schedule_check: %s read before any wait covers them (item %d)",
+                    fault.what == 1 ? "an item's copies are" : "the next tile's gather indices are", fault.item);
     return DPEP_OK;
 }
 
@@ -1134,7 +989,7 @@ int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scale
 
 // Workspace carve-up shared by workspace_bytes and forward.
 struct MegaLayout {
-    size_t hist, meta, partials, route_to_row, row_to_route, act_codes, act_scales, out2, total;
+    size_t hist, meta, fill_state, route_to_row, row_to_route, act_codes, act_scales, out2, total;
 };
 
 static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int intermediate, int num_local, int num_shared)
@@ -1147,7 +1002,7 @@ static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int inte
     size_t at = 0;
     l.hist = at;         at += up(dpep_layout_workspace_bytes(num_tokens, num_topk, num_local));
     l.meta = at;         at += up((3 * static_cast<size_t>(num_local) + num_shared + 2) * 4);
-    l.partials = at;     at += up(static_cast<size_t>(dpep::gemm_grid()) * 2 * dpep::kMaxPartialBytes);  // partial sums of tiles shared between workgroups
+    l.fill_state = at;   at += up((1 + 4096) * 4);  // fillers of the first GEMM: count + progress of each (<= 1024 CUs x 4 waves)
     l.route_to_row = at; at += up(routes * 4);
     l.row_to_route = at; at += up((routes + shared_rows) * 4);
     l.act_codes = at;    at += up(max_rows * intermediate);
@@ -1233,26 +1088,28 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g1.k = hidden;
     g1.act_codes = base + l.act_codes;
     g1.act_scales = base + l.act_scales;
-    g1.partials = base + l.partials;
-    g1.arrivals = reinterpret_cast<int*>(static_cast<char*>(w->barrier) + kSyncArrivals);
-    g1.forced_rt = w->gemm_tile_rows / 64;
     // Expected rows (the true counts stay on the device): tokens * topk / experts per routed expert, every
     // token for a shared one.
     const long long expected_routed = static_cast<long long>(num_tokens) * num_topk * num_local / num_experts;
     const long long expected_rows = expected_routed + static_cast<long long>(num_tokens) * num_shared;
     const int per_expert = static_cast<int>((expected_rows + g1.num_local - 1) / g1.num_local);
-    // In a sparse share (no shared experts, fewer rows than half the tokens) most tokens have no row and their
-    // rows of y are zeros: the two GEMMs set all of y to zero while they run, a few stores per item, in proportion
-    // to their work (2 : 1), and the weighted reduce then writes the rows of the served tokens only.
-    const long long y_bytes = static_cast<long long>(num_tokens) * hidden * 2;
-    const bool zero_in_gemms = num_shared == 0 && 2 * expected_rows < num_tokens && y_bytes % 1024 == 0;
-    const long long y_blocks = y_bytes / 1024;
-    const long long y_split = y_blocks * 2 / 3;
-    if (zero_in_gemms) {
-        g1.zero_out = static_cast<u32x4*>(y);
-        g1.zero_begin = 0;
-        g1.zero_end = y_split;
+    // Without shared experts most tokens of a share have no row: workgroups of the first GEMM that get no tile
+    // zero those rows of y meanwhile, and the weighted reduce skips what they got through.
+    int* fill_state = reinterpret_cast<int*>(base + l.fill_state);
+    int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->barrier) + kSyncFillStop);
+    w->gemm_launches = w->gemm_launches >= 0x7fffffffu ? 1u : w->gemm_launches + 1u;  // never 0
+    g1.launch_id = static_cast<int>(w->gemm_launches);
+    g1.forced_rt = w->gemm_tile_rows / 64;
+    const bool fill = num_shared == 0 && w->gemm_zero_fill;
+    if (fill) {
+        g1.fill_out = static_cast<u32x4*>(y);
+        g1.fill_route_to_row = route_to_row;
+        g1.fill_tokens = num_tokens;
+        g1.fill_vec = hidden / 8;
+        g1.fill_topk = num_topk;
+        g1.fill_stop = fill_stop;
     }
+    g1.fill_state = fill_state;  // written even when nothing fills (then as "no fillers")
     if (int rc = launch_gemm1(g1, per_expert, s)) return rc;
     GemmParams g2{};
     g2.a_codes = base + l.act_codes;
@@ -1269,18 +1126,11 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g2.n = hidden;
     g2.k = intermediate;
     g2.out = reinterpret_cast<uint16_t*>(base + l.out2);
-    g2.partials = g1.partials;
-    g2.arrivals = g1.arrivals;
     g2.forced_rt = g1.forced_rt;
-    if (zero_in_gemms) {
-        g2.zero_out = static_cast<u32x4*>(y);
-        g2.zero_begin = y_split;
-        g2.zero_end = y_blocks;
-    }
     if (int rc = launch_gemm2(g2, per_expert, s)) return rc;
     return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,
                           static_cast<int>(expected_rows),
-                          hidden, y, num_shared > 0 ? num_rows : nullptr, num_shared, zero_in_gemms, s);
+                          hidden, y, num_shared > 0 ? num_rows : nullptr, num_shared, fill ? fill_state : nullptr, s);
 }
 
 }  // extern "C"

@@ -74,6 +74,8 @@ int dpep_workspace_create(size_t bytes, void** ws)
     w->barrier_extra_arrivals = 0;
     w->layout_one_launch = 1;
     w->gemm_tile_rows = 0;
+    w->gemm_launches = 0;
+    w->gemm_zero_fill = 1;
     w->layout_launches = 0;
     w->timeout_seen = 0;
     *ws = w;
@@ -139,6 +141,8 @@ int dpep_workspace_tune(void* ws, const char* key, long long value)
     } else if (strcmp(key, "layout_barrier_extra_arrivals") == 0) {
         DPEP_REQUIRE(value >= 0 && value <= 1, "workspace_tune: layout_barrier_extra_arrivals is 0 or 1");
         w->barrier_extra_arrivals = static_cast<int>(value);
+    } else if (strcmp(key, "gemm_zero_fill") == 0) {
+        w->gemm_zero_fill = value != 0;
     } else if (strcmp(key, "gemm_tile_rows") == 0) {
         DPEP_REQUIRE(value == 0 || value == 64 || value == 128 || value == 192,
                      "workspace_tune: gemm_tile_rows is 0 (automatic), 64, 128 or 192");

@@ -45,6 +45,8 @@ int dpep_workspace_capacity(void* ws, size_t* bytes);
  *   "layout_barrier_ticks"          bound of that barrier's wait in 10 ns ticks (default 2 s)
  *   "layout_barrier_extra_arrivals" 1: the barrier expects one workgroup more than there are, so that its wait
  *                                   runs out (exercises the error path)
+ *   "gemm_zero_fill"                1 (default): workgroups of dpep_megamoe_forward's first GEMM that get no tile zero
+ *                                   the output rows of tokens no local expert serves; 0: the weighted reduce writes them
  *   "gemm_tile_rows"                0 (default): dpep_megamoe_forward chooses the row-tile height of its grouped GEMMs
  *                                   from the expected rows per expert; 64, 128 or 192: that height for both */
 int dpep_workspace_tune(void* ws, const char* key, long long value);
@@ -130,15 +132,13 @@ int dpep_combine_fp16(const void* y, const float* row_weights, const int32_t* ro
  *   x bf16 [B,H], H % 32 == 0 -> codes e4m3 [B,H], scales e8m0 [B,H/32] */
 int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* scales, void* stream);
 
-/* Host-only check of the grouped GEMM's work partition and copy/wait schedule; no counterpart in the reference (it
- * is how this build shows, without a GPU, that a launch of `total_tiles` tiles of `tile_rows` rows and `ktiles`
- * k tiles of 128 on `grid` workgroups deals every span of work to exactly one workgroup, and that under in-order
- * completion of vector-memory operations every asynchronous copy is covered by a counted wait before it is read:
- * an item's operands before its MFMAs, the next tile's gather indices before the copy cursor switches tiles).
- * zero_blocks_per_wave = 1 KiB zero stores each wave interleaves; epilogue_stores = stores a piece end issues.
- * Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
-int dpep_megamoe_schedule_check(int tile_rows, int total_tiles, int ktiles, int grid, int zero_blocks_per_wave,
-                                int epilogue_stores);
+/* Host-only check of the grouped GEMM's copy/wait schedule; no counterpart in the reference (it is how this build
+ * shows, without a GPU, that for a workgroup that walks `tiles_per_workgroup` tiles of `tile_rows` (64, 128 or 192)
+ * rows and `ktiles` k tiles of 128 every asynchronous copy is covered by a counted wait before it is read, under
+ * in-order completion of vector-memory operations: an item's operands before its MFMAs, the next tile's gather
+ * indices before the copy cursor switches tiles).  epilogue_stores = stores a tile end issues (they only make the
+ * counted waits stricter).  Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
+int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores);
 
 /* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480).
  * num_shared = number of shared experts (0..8) whose rows (every token, each) are held next to the routed ones. */
