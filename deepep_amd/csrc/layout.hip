@@ -450,6 +450,45 @@ int chunk_routes(int n_routes, int padded_local)
     return chunk < kMinChunk ? kMinChunk : chunk;
 }
 
+int check_layout_arguments(const void* idx, int num_tokens, int num_topk, int num_experts, int expert_begin, int num_local,
+                           const int32_t* counts, const int32_t* psum, const int32_t* offsets, const int32_t* route_to_row,
+                           const int32_t* row_to_route, const int32_t* num_rows)
+{
+    DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "layout: bad T=%d K=%d", num_tokens,
+                 num_topk);
+    DPEP_REQUIRE(num_experts >= 1 && expert_begin >= 0 && num_local >= 1 && num_local <= DPEP_MAX_LOCAL_EXPERTS &&
+                     expert_begin + num_local <= num_experts,
+                 "layout: bad expert range E=%d begin=%d L=%d (at most %d local experts)", num_experts, expert_begin, num_local,
+                 DPEP_MAX_LOCAL_EXPERTS);
+    DPEP_REQUIRE(static_cast<long long>(num_tokens) * num_topk < (1ll << 31), "layout: T*K must fit int32");
+    DPEP_REQUIRE(counts && psum && offsets && num_rows, "layout: NULL output");
+    DPEP_REQUIRE(static_cast<long long>(num_tokens) * num_topk == 0 || (idx && route_to_row && row_to_route),
+                 "layout: NULL routing buffer");
+    return DPEP_OK;
+}
+
+// The two-launch form: count, then assign.  The count launch writes every histogram entry the assign launch reads, so
+// the scratch needs no clearing and holds nothing between calls.
+template <typename IdxT>
+int enqueue_count_and_assign(const IdxT* idx, int n_routes, int num_experts, int expert_begin, int num_local, int padded, int chunk,
+                             int num_chunks, int* wave_hist, int* block_hist, int32_t* counts, int32_t* psum, int32_t* offsets,
+                             int32_t* num_rows, int32_t* route_to_row, int32_t* row_to_route, uint32_t* mailbox, uint32_t sequence,
+                             hipStream_t stream)
+{
+    const int blocks = (num_chunks + kWaves - 1) / kWaves;
+    if (blocks > 0) {
+        hipLaunchKernelGGL(layout_count_kernel<IdxT>, dim3(blocks), dim3(kThreads), 0, stream, idx, n_routes, num_experts,
+                           expert_begin, num_local, chunk, num_chunks, wave_hist, block_hist);
+        if (int rc = launch_status("layout_count")) return rc;
+    }
+    // One workgroup more than there are chunks to assign: the reporter (with no routes, it alone publishes the
+    // all-zero counts and prefix sums).
+    hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks + 1), dim3(kThreads), 0, stream, idx,
+                       n_routes, num_experts, expert_begin, num_local, padded, chunk, num_chunks, wave_hist, block_hist, counts,
+                       psum, offsets, num_rows, route_to_row, row_to_route, mailbox, sequence);
+    return launch_status("layout_assign");
+}
+
 template <typename IdxT>
 int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int num_experts, int expert_begin,
                   int num_local, int32_t* counts, int32_t* psum, int32_t* offsets, int32_t* route_to_row,
@@ -457,15 +496,10 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
 {
     Workspace* w = as_workspace(ws);
     DPEP_REQUIRE(w != nullptr, "layout: not a live workspace");
-    DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "layout: bad T=%d K=%d", num_tokens,
-                 num_topk);
-    DPEP_REQUIRE(num_experts >= 1 && expert_begin >= 0 && num_local >= 1 && num_local <= DPEP_MAX_LOCAL_EXPERTS &&
-                     expert_begin + num_local <= num_experts,
-                 "layout: bad expert range E=%d begin=%d L=%d", num_experts, expert_begin, num_local);
-    DPEP_REQUIRE(static_cast<long long>(num_tokens) * num_topk < (1ll << 31), "layout: T*K must fit int32");
-    DPEP_REQUIRE(counts && psum && offsets && num_rows, "layout: NULL output");
+    if (int rc = check_layout_arguments(idx, num_tokens, num_topk, num_experts, expert_begin, num_local, counts, psum, offsets,
+                                        route_to_row, row_to_route, num_rows))
+        return rc;
     const int n_routes = num_tokens * num_topk;
-    DPEP_REQUIRE(n_routes == 0 || (idx && route_to_row && row_to_route), "layout: NULL routing buffer");
     const size_t need = dpep_layout_workspace_bytes(num_tokens, num_topk, num_local);
     DPEP_REQUIRE(need <= w->bytes, "layout: workspace too small (%zu needed, %zu available)", need, w->bytes);
     // A one-launch layout whose barrier wait ran out left its number in the mailbox.  If nobody has been told yet
@@ -497,17 +531,9 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
                            w->barrier_ticks, w->mailbox_device + kMailboxTimeout, w->layout_launches);
         return launch_status("layout_fused");
     }
-    if (blocks > 0) {
-        hipLaunchKernelGGL(layout_count_kernel<IdxT>, dim3(blocks), dim3(kThreads), 0, stream, idx, n_routes, num_experts,
-                           expert_begin, num_local, chunk, num_chunks, wave_hist, block_hist);
-        if (int rc = launch_status("layout_count")) return rc;
-    }
-    // One workgroup more than there are chunks to assign: the reporter (with no routes, it alone publishes the
-    // all-zero counts and prefix sums).
-    hipLaunchKernelGGL(layout_assign_kernel<IdxT>, dim3(blocks + 1), dim3(kThreads), 0, stream, idx,
-                       n_routes, num_experts, expert_begin, num_local, padded, chunk, num_chunks, wave_hist, block_hist, counts,
-                       psum, offsets, num_rows, route_to_row, row_to_route, mailbox, w->sequence);
-    return launch_status("layout_assign");
+    return enqueue_count_and_assign<IdxT>(idx, n_routes, num_experts, expert_begin, num_local, padded, chunk, num_chunks, wave_hist,
+                                          block_hist, counts, psum, offsets, num_rows, route_to_row, row_to_route, mailbox,
+                                          w->sequence, stream);
 }
 
 }  // namespace
