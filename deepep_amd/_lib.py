@@ -26,6 +26,7 @@ SIGNATURES = {
     "dpep_workspace_tune": (_I, (_P, ctypes.c_char_p, ctypes.c_longlong)),
     "dpep_layout_workspace_bytes": (_Z, (_I, _I, _I)),
     "dpep_layout": (_I, (_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P)),
+    "dpep_layout_static": (_I, (_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P)),
     "dpep_layout_wait": (_I, (_P, _P, _I, ctypes.POINTER(ctypes.c_int32), ctypes.c_longlong)),
     "dpep_dispatch_copy": (_I, (_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_dispatch_quant_fp8": (_I, (_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),

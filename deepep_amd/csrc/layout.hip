@@ -20,6 +20,8 @@
 // assigns nothing (its histograms may be stale): it reports no rows, marks every route as having none, and leaves
 // its number in the workspace's mailbox, where the host finds it; later layouts on that workspace take two
 // launches.  Larger inputs take two launches anyway.
+#include <mutex>
+
 #include "common.h"
 
 namespace dpep {
@@ -549,6 +551,44 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
 
 }  // namespace dpep
 
+// ---- the layout for callers that cannot allocate -------------------------------------------------------------
+// Scratch of dpep_layout_static: the histograms a workspace would hold, in a device array of this library instead.
+// Every GPU the library runs on has its own copy, at its own address, for the life of the process.
+namespace dpep {
+namespace {
+constexpr size_t kStaticScratchInts = kHistInts + kBlockHistInts;  // 21 504 ints = 84 KiB
+}
+}
+static __device__ __align__(256) int scratch[dpep::kStaticScratchInts];
+
+namespace dpep {
+namespace {
+
+constexpr int kMaxDevices = 64;
+int* g_scratch_of_device[kMaxDevices];  // device address of `scratch` on each GPU, looked up on first use
+std::mutex g_scratch_mutex;
+
+// The address of this GPU's copy of `scratch` (the current device's).  In host code the array's name is only a
+// handle for the runtime, not a device address: kernels and memory calls get the looked-up pointer, never the name.
+int scratch_of_current_device(int** out)
+{
+    int device = -1;
+    DPEP_HIP(hipGetDevice(&device));
+    DPEP_REQUIRE(device >= 0 && device < kMaxDevices, "layout_static: device %d outside [0, %d)", device, kMaxDevices);
+    std::lock_guard<std::mutex> guard(g_scratch_mutex);
+    if (g_scratch_of_device[device] == nullptr) {
+        int* ptr = nullptr;
+        DPEP_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+        DPEP_REQUIRE(ptr != nullptr, "layout_static: the scratch array has no address on device %d", device);
+        g_scratch_of_device[device] = ptr;
+    }
+    *out = g_scratch_of_device[device];
+    return DPEP_OK;
+}
+
+}  // namespace
+}  // namespace dpep
+
 extern "C" {
 
 size_t dpep_layout_workspace_bytes(int num_tokens, int num_topk, int num_local_experts)
@@ -564,6 +604,31 @@ int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk,
     return dpep::launch_layout<int64_t>(ws, topk_idx, num_tokens, num_topk, num_experts, expert_begin, num_local,
                                         counts, psum, offsets, route_to_row, row_to_route, num_rows,
                                         /*report_to_host=*/true, static_cast<hipStream_t>(stream));
+}
+
+int dpep_layout_static(const int64_t* topk_idx, int num_tokens, int num_topk, int num_experts, int expert_begin,
+                       int num_local, int32_t* counts, int32_t* psum, int32_t* offsets, int32_t* route_to_row,
+                       int32_t* row_to_route, int32_t* num_rows, void* stream)
+{
+    using namespace dpep;
+    if (int rc = check_layout_arguments(topk_idx, num_tokens, num_topk, num_experts, expert_begin, num_local, counts, psum,
+                                        offsets, route_to_row, row_to_route, num_rows))
+        return rc;
+    const int n_routes = num_tokens * num_topk;
+    const int padded = padded_experts(num_local);
+    const int chunk = chunk_routes(n_routes, padded);
+    const int num_chunks = (n_routes + chunk - 1) / chunk;
+    const int blocks = (num_chunks + kWaves - 1) / kWaves;
+    // what the two launches address: num_chunks rows of wave histograms, blocks rows of workgroup histograms
+    DPEP_REQUIRE(static_cast<size_t>(num_chunks) * num_local <= static_cast<size_t>(kHistInts) &&
+                     static_cast<size_t>(blocks) * num_local <= static_cast<size_t>(kBlockHistInts),
+                 "layout_static: %d chunks x %d local experts exceed the static scratch of %zu bytes", num_chunks, num_local,
+                 kStaticScratchInts * sizeof(int));
+    int* base = nullptr;
+    if (int rc = scratch_of_current_device(&base)) return rc;
+    return enqueue_count_and_assign<int64_t>(topk_idx, n_routes, num_experts, expert_begin, num_local, padded, chunk, num_chunks,
+                                             base, base + kHistInts, counts, psum, offsets, num_rows, route_to_row, row_to_route,
+                                             /*mailbox=*/nullptr, 0u, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

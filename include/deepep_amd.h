@@ -69,6 +69,19 @@ int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk,
                 int expert_begin, int num_local, int32_t* counts, int32_t* psum, int32_t* offsets,
                 int32_t* route_to_row, int32_t* row_to_route, int32_t* num_rows, void* stream);
 
+/* dpep_layout for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference (whose notify always works in its pre-allocated symmetric
+ * workspace).  Same inputs, outputs and results as dpep_layout, but no workspace: the histograms live in a device
+ * array inside the library (84 KiB per GPU, held until the process ends), and the call allocates nothing - no
+ * hipMalloc, hipFree or pinned memory, on the first call or any later one.  Always the two-launch form (count, then
+ * assign); it reports nothing to the host, so R is read from num_rows on the device.  Limits: those of dpep_layout
+ * (at most DPEP_MAX_LOCAL_EXPERTS local experts, T*K < 2^31), checked before anything is launched.  All calls on one
+ * GPU share that GPU's array: calls whose kernels overlap on one GPU (different streams) race; calls on one stream
+ * do not.  Nothing in the array has to be zero or is kept between calls. */
+int dpep_layout_static(const int64_t* topk_idx, int num_tokens, int num_topk, int num_experts, int expert_begin,
+                       int num_local, int32_t* counts, int32_t* psum, int32_t* offsets, int32_t* route_to_row,
+                       int32_t* row_to_route, int32_t* num_rows, void* stream);
+
 /* Host side of the layout's single synchronisation: blocks until the most recent dpep_layout launched on ws has
  * run, then returns R and (optionally) the rows per local expert.  Replaces the device-to-host read-back that sizes
  * the outputs of a fresh dispatch (deep_ep/backends/mesh_clos/elastic.py:1476, `.cpu()` of the notify outputs):
