@@ -14,13 +14,9 @@
 namespace dpep {
 namespace {
 
-#ifndef DPEP_TUNE_MAX_THREADS
-#define DPEP_TUNE_MAX_THREADS 256
-#endif
-#ifndef DPEP_TUNE_TARGET_BLOCKS
-#define DPEP_TUNE_TARGET_BLOCKS 1000000  // split every token row into 1-2 KiB parts: measured best at all sizes
-#endif
-constexpr int kMaxThreads = DPEP_TUNE_MAX_THREADS;
+constexpr int kMaxThreads = 256;
+constexpr int kDenseTargetBlocks = 1000000;  // dense routing: split every token row into 1-2 KiB parts (measured best at all sizes)
+constexpr int kSparseTargetBlocks = 2048;    // sparse shares: a workgroup per token while that fills the chip
 constexpr int kBatch = 8;  // rows fetched per thread before the dependent adds start
 
 // kWeights: 0 = plain sum, 1 = weight per expert row (w[row]), 2 = weight per route (w[t*K + s]).
@@ -110,14 +106,8 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
 // times as many tokens are in flight per CU (the kernel above spends its time on the chain of dependent loads
 // each of its workgroups starts with).  Same arithmetic in the same order as combine_kernel<2>: slots
 // ascending, separate fp32 multiply and add, one RNE rounding to BF16.
-#ifndef DPEP_TUNE_SPARSE_BATCH
-#define DPEP_TUNE_SPARSE_BATCH 8
-#endif
-#ifndef DPEP_TUNE_SPARSE_WAVES
-#define DPEP_TUNE_SPARSE_WAVES 4
-#endif
-constexpr int kSparseBatch = DPEP_TUNE_SPARSE_BATCH;  // 16-byte vectors per lane in flight per slot
-constexpr int kSparseWaves = DPEP_TUNE_SPARSE_WAVES;  // tokens (= waves) per workgroup
+constexpr int kSparseBatch = 8;  // 16-byte vectors per lane in flight per slot
+constexpr int kSparseWaves = 4;  // tokens (= waves) per workgroup
 __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ route_weights, const int* __restrict__ route_to_row,
     int num_topk, int vec_per_row, u32x4* __restrict__ out, int num_tokens, const int* __restrict__ fill_state)
@@ -186,9 +176,6 @@ __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
 struct CombineGrid {
     int parts, per_part, threads, blocks;
 };
-#ifndef DPEP_TUNE_SPARSE_TARGET
-#define DPEP_TUNE_SPARSE_TARGET 2048
-#endif
 
 
 // Dense routing (at least one row per token on average): split every token row into 1-2 KiB parts.
@@ -197,7 +184,7 @@ struct CombineGrid {
 CombineGrid combine_grid(int num_tokens, int num_rows, int vec)
 {
     CombineGrid g;
-    const int target = num_rows >= num_tokens ? DPEP_TUNE_TARGET_BLOCKS : DPEP_TUNE_SPARSE_TARGET;
+    const int target = num_rows >= num_tokens ? kDenseTargetBlocks : kSparseTargetBlocks;
     int parts = 1;
     while (num_tokens * parts < target && vec / (parts * 2) >= 64 && parts < 16) parts *= 2;
     g.per_part = (vec + parts - 1) / parts;

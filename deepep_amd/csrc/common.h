@@ -98,27 +98,9 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
-#ifndef DPEP_TUNE_STORE_NT
-#define DPEP_TUNE_STORE_NT 1
-#endif
-#ifndef DPEP_TUNE_LOAD_NT
-#define DPEP_TUNE_LOAD_NT 1
-#endif
-__device__ __forceinline__ void store16_nt(void* p, u32x4 v)
-{
-#if DPEP_TUNE_STORE_NT
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
-#else
-    *reinterpret_cast<u32x4*>(p) = v;
-#endif
-}
-__device__ __forceinline__ u32x4 load16_nt(const void* p)
-{
-#if DPEP_TUNE_LOAD_NT
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-#else
-    return *reinterpret_cast<const u32x4*>(p);
-#endif
-}
+// Streaming (non-temporal) 16-byte accesses: the byte movers write rows nobody reads again soon, and combine reads
+// rows once.
+__device__ __forceinline__ void store16_nt(void* p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
+__device__ __forceinline__ u32x4 load16_nt(const void* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)); }
 
 }  // namespace dpep

@@ -11,17 +11,10 @@
 namespace dpep {
 namespace {
 
-#ifndef DPEP_TUNE_MAX_THREADS
-#define DPEP_TUNE_MAX_THREADS 256
-#endif
-#ifndef DPEP_TUNE_TARGET_BLOCKS
-#define DPEP_TUNE_TARGET_BLOCKS 2048
-#endif
-constexpr int kMaxThreads = DPEP_TUNE_MAX_THREADS;
+constexpr int kMaxThreads = 256;
+constexpr int kTargetBlocks = 2048;  // rows are split into column parts until a launch has about this many workgroups
 constexpr int kMaxScaleCols = 1024;  // hidden <= 131072 for the fused quantiser
-#ifndef DPEP_TUNE_ROW_MAJOR_RATIO
-#define DPEP_TUNE_ROW_MAJOR_RATIO 1  // row-major kernels when rows <= ratio * tokens
-#endif
+constexpr int kRowMajorRatio = 1;  // row-major kernels when rows <= ratio * tokens
 
 // ---- token-major copy: one workgroup per (token, column part); read once, write K times -----------
 __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
@@ -214,7 +207,7 @@ struct Split {
 Split choose_split(int rows, int units, int granule)
 {
     Split s;
-    const int target_blocks = DPEP_TUNE_TARGET_BLOCKS;
+    const int target_blocks = kTargetBlocks;
     int parts = 1;
     while (rows * parts < target_blocks && units / (parts * 2) >= 64 && parts < 16) parts *= 2;
     int per_part = (units + parts - 1) / parts;
@@ -259,7 +252,7 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
     const int vec = row_bytes / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // the token-major grid does not depend on R, so a launch that does not know R yet takes it
-    if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
+    if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(kRowMajorRatio) * num_tokens) {
         const Split sp = choose_split(num_tokens, vec, 1);
         hipLaunchKernelGGL(dispatch_copy_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
                            static_cast<const u32x4*>(x), scales, topk_weights, route_to_row, num_topk, vec, sp.per_part,
@@ -287,7 +280,7 @@ int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int3
     const int units = hidden / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // the token-major grid does not depend on R, so a launch that does not know R yet takes it
-    if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(DPEP_TUNE_ROW_MAJOR_RATIO) * num_tokens) {
+    if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(kRowMajorRatio) * num_tokens) {
         const Split sp = choose_split(num_tokens, units, 8);
         hipLaunchKernelGGL(dispatch_quant_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
                            static_cast<const u32x4*>(x), topk_weights, route_to_row, num_topk, units, sp.per_part,

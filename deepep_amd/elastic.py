@@ -41,6 +41,22 @@ LOW_LATENCY_MAX_TOKENS = 256
 _ROUTING = ("topk_idx", "route_to_row", "weight_return_meta", "expert_totals", "psum_num_recv_tokens_per_expert")
 
 
+def _enforce(*rules):
+    """Runs argument rules in order: each is ``(holds, exception type, message)``, where ``holds`` is a bool or a
+    callable evaluated only when the earlier rules have passed.  The first rule that does not hold raises."""
+    for holds, error, message in rules:
+        if not (holds() if callable(holds) else holds):
+            raise error(message)
+
+
+def _is_bool(value):
+    return type(value) is bool
+
+
+def _int_among(value, allowed):
+    return type(value) is int and value in allowed
+
+
 def _integer(name, value, lower, upper):
     if type(value) is not int or not lower <= value <= upper:
         raise ValueError(f"{name} must be an integer in [{lower}, {upper}]")
@@ -216,24 +232,17 @@ class ElasticBuffer:
         rootinfo_path: Optional[str] = None,
     ):
         native = _load_native()
-        if (
-            num_cpu_bytes != 0
-            or deterministic is not False
-            or allow_hybrid_mode is not True
-            or allow_multiple_reduction is not True
-            or prefer_overlap_with_compute is not True
-            or sl_idx != 3
-            or type(num_allocated_qps) is not int
-            or num_allocated_qps not in (0, 6)
-            or num_gpu_timeout_secs != 100
-        ):
-            raise NotImplementedError("ElasticBuffer supports default options and num_allocated_qps=0/6")
-        if type(use_fp8_dispatch) is not bool:
-            raise TypeError("use_fp8_dispatch must be bool")
-        if explicitly_destroy is not True:
-            raise NotImplementedError("Runtime currently requires explicitly_destroy=True")
-        if type(combine_only) is not bool or type(debug_collectives) is not bool:
-            raise TypeError("combine_only and debug_collectives must be bool")
+        defaults_only = (
+            num_cpu_bytes == 0 and deterministic is False and allow_hybrid_mode is True and allow_multiple_reduction is True
+            and prefer_overlap_with_compute is True and sl_idx == 3 and _int_among(num_allocated_qps, (0, 6))
+            and num_gpu_timeout_secs == 100
+        )
+        _enforce(
+            (defaults_only, NotImplementedError, "ElasticBuffer supports default options and num_allocated_qps=0/6"),
+            (_is_bool(use_fp8_dispatch), TypeError, "use_fp8_dispatch must be bool"),
+            (explicitly_destroy is True, NotImplementedError, "Runtime currently requires explicitly_destroy=True"),
+            (_is_bool(combine_only) and _is_bool(debug_collectives), TypeError, "combine_only and debug_collectives must be bool"),
+        )
         _integer("num_max_tokens_per_rank", num_max_tokens_per_rank, 0, MAX_TOKENS)
         _integer("num_topk", num_topk, 0, MAX_TOPK)
         _integer("hidden", hidden, 0, MAX_HIDDEN)
@@ -448,97 +457,86 @@ class ElasticBuffer:
         with runtime.notify_lock:
             if runtime.notify_failed:
                 raise RuntimeError("A previous communication launch failed; restart the distributed job")
-            for name, value in (
-                ("async_with_compute_stream", async_with_compute_stream),
-                ("allocate_on_comm_stream", allocate_on_comm_stream),
-                ("do_handle_copy", do_handle_copy),
-                ("do_zero_padding", do_zero_padding),
-                ("use_aligned_col_major_sf", use_tma_aligned_col_major_sf),
-            ):
-                if type(value) is not bool:
-                    raise TypeError(f"{name} must be bool")
-            if do_expand is not None and do_expand is not True:
-                raise NotImplementedError("Dispatch supports only the expanded expert layout")
-            if do_cpu_sync is not None and type(do_cpu_sync) is not bool:
-                raise TypeError("do_cpu_sync must be bool or None")
-            if handle is None and do_cpu_sync is False:
-                raise NotImplementedError("Fresh notify requires do_cpu_sync=None/True")
-            if expert_alignment is not None and (type(expert_alignment) is not int or expert_alignment != 1):
-                raise NotImplementedError("Dispatch supports expert_alignment=1")
-            if (
-                cumulative_local_expert_recv_stats is not None
-                or previous_event_before_epilogue is not None
-                or allocate_on_comm_stream
-                or do_zero_padding
-                or use_tma_aligned_col_major_sf
-            ):
-                raise NotImplementedError(
-                    "Stats, epilogue events, padding and alternate allocation/scale layouts are unavailable"
-                )
-            if previous_event is not None and (
-                not isinstance(previous_event, EventHandle) or previous_event._device != runtime.device
-            ):
-                raise ValueError("previous_event must belong to the buffer GPU")
             fp8_input = isinstance(x, tuple)
-            if fp8_input and len(x) != 2:
-                raise ValueError("FP8 input must be (hidden, scales)")
-            hidden, scales = x if fp8_input else (x, None)
-            if not self._check_tensor(hidden, torch.float8_e4m3fn if fp8_input else torch.bfloat16) or hidden.ndim != 2:
-                raise ValueError(
-                    "x must be contiguous BF16, or (FP8 E4M3FN, FP32 scales), on the buffer GPU without grad"
-                )
-            tokens, width = hidden.shape
+            hidden, scales = x if fp8_input and len(x) == 2 else (x, None)
             fuse_quant = self.use_fp8_dispatch and not fp8_input
             fp8 = fp8_input or fuse_quant
+            extras_unused = (
+                cumulative_local_expert_recv_stats is None and previous_event_before_epilogue is None
+                and not allocate_on_comm_stream and not do_zero_padding and not use_tma_aligned_col_major_sf
+            )
+            _enforce(
+                # options
+                *((_is_bool(value), TypeError, f"{name} must be bool") for name, value in (
+                    ("async_with_compute_stream", async_with_compute_stream),
+                    ("allocate_on_comm_stream", allocate_on_comm_stream),
+                    ("do_handle_copy", do_handle_copy),
+                    ("do_zero_padding", do_zero_padding),
+                    ("use_aligned_col_major_sf", use_tma_aligned_col_major_sf),
+                )),
+                (do_expand is None or do_expand is True, NotImplementedError, "Dispatch supports only the expanded expert layout"),
+                (do_cpu_sync is None or _is_bool(do_cpu_sync), TypeError, "do_cpu_sync must be bool or None"),
+                (handle is not None or do_cpu_sync is not False, NotImplementedError, "Fresh notify requires do_cpu_sync=None/True"),
+                (expert_alignment is None or _int_among(expert_alignment, (1,)), NotImplementedError,
+                 "Dispatch supports expert_alignment=1"),
+                (extras_unused, NotImplementedError,
+                 "Stats, epilogue events, padding and alternate allocation/scale layouts are unavailable"),
+                (previous_event is None or (isinstance(previous_event, EventHandle) and previous_event._gpu_index == runtime.device),
+                 ValueError, "previous_event must belong to the buffer GPU"),
+                # payload
+                (not fp8_input or len(x) == 2, ValueError, "FP8 input must be (hidden, scales)"),
+                (lambda: self._check_tensor(hidden, torch.float8_e4m3fn if fp8_input else torch.bfloat16) and hidden.ndim == 2,
+                 ValueError, "x must be contiguous BF16, or (FP8 E4M3FN, FP32 scales), on the buffer GPU without grad"),
+            )
+            tokens, width = hidden.shape
             _validate_hidden(width, fp8)
-            if self.hidden and width != self.hidden:
-                raise ValueError("hidden differs from buffer configuration")
-            if fp8_input and not self._check_tensor(scales, torch.float32, (tokens, width // 128)):
-                raise ValueError("FP8 scales must be contiguous FP32 [T,H/128] on the buffer GPU without grad")
-            if type(num_sms) is not int or num_sms not in (0, 64 if fp8 else 32):
-                raise ValueError("num_compute_units must be 0/32 for BF16 or 0/64 for FP8")
-            if type(num_qps) is not int or num_qps not in (0, 2):
-                raise ValueError("Primary dispatch uses two QPs per peer; num_qps=0/2")
+            _enforce(
+                (not self.hidden or width == self.hidden, ValueError, "hidden differs from buffer configuration"),
+                (lambda: not fp8_input or self._check_tensor(scales, torch.float32, (tokens, width // 128)), ValueError,
+                 "FP8 scales must be contiguous FP32 [T,H/128] on the buffer GPU without grad"),
+                (_int_among(num_sms, (0, 64 if fp8 else 32)), ValueError, "num_compute_units must be 0/32 for BF16 or 0/64 for FP8"),
+                (_int_among(num_qps, (0, 2)), ValueError, "Primary dispatch uses two QPs per peer; num_qps=0/2"),
+            )
             world = runtime.world_size
             if handle is not None:
-                if (
-                    not isinstance(handle, EPHandle)
-                    or handle._buffer_token is not self._handle_token
-                    or handle.metadata_only
-                    or handle.metadata_version != 7
-                ):
-                    raise ValueError("Cached handle must come from this buffer's successful payload dispatch")
-                if topk_idx is not None:
-                    raise ValueError("Cached dispatch inherits routing; omit topk_idx")
-                if num_experts is not None and num_experts != handle.num_experts:
-                    raise ValueError("num_experts differs from cached routing")
+                from_here = (
+                    isinstance(handle, EPHandle) and handle._buffer_token is self._handle_token
+                    and not handle.metadata_only and handle.metadata_version == 7
+                )
+                _enforce(
+                    (from_here, ValueError, "Cached handle must come from this buffer's successful payload dispatch"),
+                    (topk_idx is None, ValueError, "Cached dispatch inherits routing; omit topk_idx"),
+                    (lambda: num_experts is None or num_experts == handle.num_experts, ValueError,
+                     "num_experts differs from cached routing"),
+                )
                 self._check_versions(handle)
                 num_experts, topk = handle.num_experts, handle.num_topk
-                if tokens != handle.num_tokens:
-                    raise ValueError("Cached dispatch requires the original token count")
-                if width != handle.hidden:
-                    raise ValueError("Cached dispatch requires the original hidden size")
+                _enforce(
+                    (tokens == handle.num_tokens, ValueError, "Cached dispatch requires the original token count"),
+                    (width == handle.hidden, ValueError, "Cached dispatch requires the original hidden size"),
+                )
             else:
-                if not self._check_tensor(topk_idx, torch.int64) or topk_idx.ndim != 2 or topk_idx.shape[0] != tokens:
-                    raise ValueError("topk_idx must be contiguous int64 [T,K] on the buffer GPU")
-                if not do_handle_copy and torch.is_inference(topk_idx):
-                    raise ValueError("Inference routing tensors require do_handle_copy=True")
+                _enforce(
+                    (lambda: self._check_tensor(topk_idx, torch.int64) and topk_idx.ndim == 2 and topk_idx.shape[0] == tokens,
+                     ValueError, "topk_idx must be contiguous int64 [T,K] on the buffer GPU"),
+                    (lambda: do_handle_copy or not torch.is_inference(topk_idx), ValueError,
+                     "Inference routing tensors require do_handle_copy=True"),
+                )
                 topk = topk_idx.shape[1]
             _integer("tokens", tokens, 1, MAX_TOKENS * world)
             _integer("topk", topk, 1, MAX_TOPK)
             _integer("experts", num_experts, world, MAX_EXPERTS)
-            if num_experts % world:
-                raise ValueError("num_experts must be divisible by EP")
             bound = self.num_max_tokens_per_rank
             per_rank = -(-tokens // world)
             capacity = (bound or per_rank) if num_max_tokens_per_rank is None else num_max_tokens_per_rank
+            _enforce((num_experts % world == 0, ValueError, "num_experts must be divisible by EP"))
             _integer("num_max_tokens_per_rank", capacity, per_rank, MAX_TOKENS)
-            if bound and capacity > bound:
-                raise ValueError("Input/capacity exceeds the buffer token bound")
-            if self.num_topk and self.num_topk != topk:
-                raise ValueError("topk differs from buffer configuration")
-            if topk_weights is not None and not self._check_tensor(topk_weights, torch.float32, (tokens, topk)):
-                raise ValueError("topk_weights must be contiguous FP32 [T,K] on the buffer GPU without grad")
+            _enforce(
+                (not bound or capacity <= bound, ValueError, "Input/capacity exceeds the buffer token bound"),
+                (not self.num_topk or self.num_topk == topk, ValueError, "topk differs from buffer configuration"),
+                (lambda: topk_weights is None or self._check_tensor(topk_weights, torch.float32, (tokens, topk)), ValueError,
+                 "topk_weights must be contiguous FP32 [T,K] on the buffer GPU without grad"),
+            )
 
             # ---- launch: everything from here runs on the communication stream --------------
             try:
@@ -578,7 +576,7 @@ class ElasticBuffer:
                     handle._routing_versions = {
                         name: (getattr(handle, name).data_ptr(), getattr(handle, name)._version) for name in _ROUTING
                     }
-                    event = EventOverlap._from_resources(EventHandle(), retained)
+                    event = EventOverlap._holding(EventHandle(), retained)
                 if not async_with_compute_stream:
                     event.current_stream_wait(release_handle=True)
                 runtime.notify_inflight = None
@@ -688,7 +686,7 @@ class ElasticBuffer:
                     handle.num_tokens, handle.num_topk, handle.hidden = tokens, topk, width
                     retained = (hidden, scales, topk_weights, indices, out, out_scales, row_weights, send_counts,
                                 layout["route_to_row"], layout["row_to_route"], layout["meta"])
-                    event = EventOverlap._from_resources(EventHandle(), retained)
+                    event = EventOverlap._holding(EventHandle(), retained)
                 event.current_stream_wait(release_handle=True)
                 runtime.notify_inflight = None
                 return (out, out_scales) if scales is not None else out, None, None, handle, event
@@ -730,7 +728,7 @@ class ElasticBuffer:
                     producer.current_stream_wait()
                     output, _ = runtime.native.combine(x, handle.route_to_row, handle.source_weights, None)
                     retained = (x, output, handle.route_to_row, handle.source_weights, handle.topk_idx)
-                    event = EventOverlap._from_resources(EventHandle(), retained)
+                    event = EventOverlap._holding(EventHandle(), retained)
                 event.current_stream_wait(release_handle=True)
                 runtime.notify_inflight = None
                 return output, None, event
@@ -803,44 +801,34 @@ class ElasticBuffer:
         with runtime.notify_lock:
             if runtime.notify_failed:
                 raise RuntimeError("A previous communication launch failed; restart the distributed job")
-            if type(async_with_compute_stream) is not bool or type(allocate_on_comm_stream) is not bool:
-                raise TypeError("Stream options must be bool")
-            if bias is not None:
-                raise NotImplementedError("Combine currently supports bias=None")
-            if previous_event_before_epilogue is not None or allocate_on_comm_stream:
-                raise NotImplementedError("Epilogue events and allocate_on_comm_stream are unavailable")
-            if type(num_sms) is not int or num_sms not in (0, 64):
-                raise ValueError("Combine uses 64 compute units; num_compute_units=0/64")
-            if type(num_qps) is not int or num_qps not in (0, 2):
-                raise ValueError("Combine uses two QPs per cross sender; num_qps=0/2")
-            if previous_event is not None and (
-                not isinstance(previous_event, EventHandle) or previous_event._device != runtime.device
-            ):
-                raise ValueError("previous_event must belong to the buffer GPU")
-            if (
-                not isinstance(handle, EPHandle)
-                or handle._buffer_token is not self._handle_token
-                or handle.metadata_only
-                or handle.metadata_version != 7
-            ):
-                raise ValueError("Combine needs this buffer's successful expanded payload dispatch handle")
-            if not handle.do_expand or handle.expert_alignment != 1:
-                raise ValueError("Combine supports expanded layout without padding")
-            if handle.rank != runtime.rank or handle.world_size != runtime.world_size:
-                raise ValueError("Handle topology differs from the buffer")
+            from_here = (
+                isinstance(handle, EPHandle) and handle._buffer_token is self._handle_token
+                and not handle.metadata_only and handle.metadata_version == 7
+            )
+            _enforce(
+                (_is_bool(async_with_compute_stream) and _is_bool(allocate_on_comm_stream), TypeError, "Stream options must be bool"),
+                (bias is None, NotImplementedError, "Combine currently supports bias=None"),
+                (previous_event_before_epilogue is None and not allocate_on_comm_stream, NotImplementedError,
+                 "Epilogue events and allocate_on_comm_stream are unavailable"),
+                (_int_among(num_sms, (0, 64)), ValueError, "Combine uses 64 compute units; num_compute_units=0/64"),
+                (_int_among(num_qps, (0, 2)), ValueError, "Combine uses two QPs per cross sender; num_qps=0/2"),
+                (previous_event is None or (isinstance(previous_event, EventHandle) and previous_event._gpu_index == runtime.device),
+                 ValueError, "previous_event must belong to the buffer GPU"),
+                (from_here, ValueError, "Combine needs this buffer's successful expanded payload dispatch handle"),
+                (lambda: handle.do_expand and handle.expert_alignment == 1, ValueError, "Combine supports expanded layout without padding"),
+                (lambda: handle.rank == runtime.rank and handle.world_size == runtime.world_size, ValueError,
+                 "Handle topology differs from the buffer"),
+            )
             self._check_versions(handle)
             rows = handle.num_expanded_tokens
-            if not self._check_tensor(x, torch.bfloat16, (rows, handle.hidden)):
-                raise ValueError(
-                    "x must be contiguous BF16 [num_expanded_tokens,H] matching the handle on the buffer GPU without grad"
-                )
-            if topk_weights is not None and not self._check_tensor(topk_weights, torch.float32, (rows,)):
-                raise ValueError(
-                    "topk_weights must be contiguous FP32 [num_expanded_tokens] on the buffer GPU without grad"
-                )
             weighted = handle.is_low_latency
-            if weighted and handle.source_weights is None:
-                raise ValueError("Low-latency handle carries no saved route weights")
+            _enforce(
+                (lambda: self._check_tensor(x, torch.bfloat16, (rows, handle.hidden)), ValueError,
+                 "x must be contiguous BF16 [num_expanded_tokens,H] matching the handle on the buffer GPU without grad"),
+                (lambda: topk_weights is None or self._check_tensor(topk_weights, torch.float32, (rows,)), ValueError,
+                 "topk_weights must be contiguous FP32 [num_expanded_tokens] on the buffer GPU without grad"),
+                (not weighted or handle.source_weights is not None, ValueError, "Low-latency handle carries no saved route weights"),
+            )
             try:
                 if previous_event is not None:
                     previous_event.current_stream_wait()
@@ -853,7 +841,7 @@ class ElasticBuffer:
                     retained = (x, topk_weights, output, output_weights, handle.topk_idx) + tuple(
                         getattr(handle, name) for name in _ROUTING
                     )
-                    event = EventOverlap._from_resources(EventHandle(), retained)
+                    event = EventOverlap._holding(EventHandle(), retained)
                 if not async_with_compute_stream:
                     event.current_stream_wait(release_handle=True)
                 runtime.notify_inflight = None
