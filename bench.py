@@ -1,5 +1,6 @@
 #!/usr/bin/env python3
-"""Headline benchmark: prefill dispatch + combine on one MI355X.
+"""Headline benchmark: prefill dispatch + combine on one MI355X, with the decode and rank-share shapes and the W4A8
+expert FFN measured beside it.
 
 A step is one pass of the hot path over one synthetic batch at the prefill shape
 (T=4096, H=7168, 256 experts, top-8 with Zipf(1.2) popularity, seed 0):
@@ -7,7 +8,17 @@ A step is one pass of the hot path over one synthetic batch at the prefill shape
   needs) -> FP8 e4m3 dispatch with the per-128 quantiser fused into the expand-permute ->
   combine of BF16 gradients N(0,1) [R,H] (the backward of dispatch).
 `value` is the algorithmic HBM bytes of dispatch + combine per second of wall time of that step.
-Prints ONE JSON line.
+
+Every kernel is then timed by itself with HIP events on the stream it is launched on, two ways: with the caches
+flushed before every launch by a 256 MiB fill (the reference's protocol, deep_ep/utils/testing.py:27-35; at least 20
+warm-ups and 100 launches: mean / min / p50 / p95) and back to back.  `roofline` is the dominant kernel under the
+flush protocol.  Prints ONE JSON line.
+
+Other modes:
+  --ingest-pmc FETCH.csv WRITE.csv   turn two rocprofv3 --pmc counter files of this command (run with --calibrate-copy)
+                                     into profiles/hbm_traffic.json, which `roofline.traffic` is read from
+  --protocol PRESET                  the reference's generic benchmark workloads (benchmarks/_config.py) through this
+                                     library: one `measured` record per operation in the v1 result schema
 """
 
 from __future__ import annotations
@@ -23,6 +34,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 (the mixed FP8 x FP4 MFMA issues at the FP8 cadence)
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+FLUSH_BYTES = 256 << 20
 
 
 def algorithmic_bytes(tokens, hidden, topk, rows):
@@ -34,95 +48,156 @@ def algorithmic_bytes(tokens, hidden, topk, rows):
     return dict(layout=layout, dispatch=dispatch, combine=combine)
 
 
-def time_kernel(fn, iters, torch, head_start=None):
-    """Average device time of `fn` in microseconds, HIP events on the stream the kernels run on.  `head_start`: the
-    GPU is kept busy first (a spin kernel of about 2 ms where torch offers one, else fills of that tensor), so that
-    the host queues launches meanwhile and a kernel shorter than its Python launch path is still timed back to back."""
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(3):
-        fn()
-    torch.cuda.synchronize()
-    if head_start is not None:
-        if hasattr(torch.cuda, "_sleep"):
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+class Timer:
+    """Device times of one launch closure, HIP events on torch's current stream (the one ops launches on)."""
+
+    def __init__(self, torch, iters, warmups):
+        self.torch = torch
+        self.iters = max(1, iters)
+        self.warmups = max(1, warmups)
+        self.flush = None
+
+    def back_to_back(self, fn, head_start=False):
+        """Average microseconds over `iters` launches queued without gaps.  head_start: the GPU is kept busy first
+        (a spin kernel of about 2 ms), so that the host queues launches meanwhile and a kernel shorter than its Python
+        launch path is still timed back to back."""
+        torch = self.torch
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(self.warmups):
+            fn()
+        torch.cuda.synchronize()
+        if head_start and hasattr(torch.cuda, "_sleep"):
             torch.cuda._sleep(4_000_000)  # cycles; no memory traffic that the timed kernels would have to wait out
-        else:
-            for _ in range(8):
-                head_start.zero_()
-    start.record()
-    for _ in range(iters):
-        fn()
-    stop.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(stop) * 1000.0 / iters
-
-
-def time_kernel_cold(fn, iters, torch, flush):
-    """Per-launch device times with the caches flushed before every launch (a 256 MiB fill, the way the
-    reference's flush_l2_cache does, deep_ep/utils/testing.py:27-35): mean / min / p50 / p95 in microseconds."""
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    fn()
-    for start, stop in pairs:
-        flush.zero_()
         start.record()
-        fn()
+        for _ in range(self.iters):
+            fn()
         stop.record()
-    torch.cuda.synchronize()
-    times = sorted(a.elapsed_time(b) * 1000.0 for a, b in pairs)
-    pick = lambda q: times[min(len(times) - 1, int(q * len(times)))]
-    return dict(mean=sum(times) / len(times), min=times[0], p50=pick(0.5), p95=pick(0.95))
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1000.0 / self.iters
+
+    def flushed(self, fn):
+        """Per-launch times with the caches flushed before every launch by a 256 MiB fill."""
+        torch = self.torch
+        if self.flush is None:
+            self.flush = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device="cuda")
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(self.iters)]
+        for _ in range(self.warmups):
+            fn()
+        for start, stop in pairs:
+            self.flush.zero_()
+            start.record()
+            fn()
+            stop.record()
+        torch.cuda.synchronize()
+        times = sorted(a.elapsed_time(b) * 1000.0 for a, b in pairs)
+        pick = lambda q: times[min(len(times) - 1, int(q * len(times)))]
+        return dict(mean=sum(times) / len(times), min=times[0], p50=pick(0.5), p95=pick(0.95))
+
+    def kernel(self, fn, nbytes, head_start=False, extra=None):
+        """One `kernels` entry: flushed statistics, the back-to-back figure, and GB/s of both against 8 TB/s."""
+        warm = self.back_to_back(fn, head_start)
+        cold = self.flushed(fn)
+        entry = dict(
+            bytes=nbytes,
+            us=cold["mean"],
+            flushed_us=cold,
+            back_to_back_us=warm,
+            GBps=nbytes / cold["mean"] / 1e3,
+            frac_of_8TBps=nbytes / cold["mean"] / 1e3 / HBM_PEAK_GBS,
+            GBps_back_to_back=nbytes / warm / 1e3,
+            frac_back_to_back=nbytes / warm / 1e3 / HBM_PEAK_GBS,
+        )
+        if extra:
+            entry.update(extra)
+        return entry
 
 
-def cpu_baseline(x, idx, w, grads, cfg, nbytes):
-    """The reference CPU path (torch CPU, all host threads) on the same inputs."""
+def cpu_baseline(x, idx, w, grads, cfg):
+    """The reference CPU path (torch CPU, all host threads) on the same full batch: 3 warm-ups + 10 timed passes."""
     import torch
 
     from oracle import baseline
 
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    tokens = min(cfg["tokens"], 1024)  # bounded sample: the first 1024 tokens of the same batch
-    xs, ids, ws = x[:tokens], idx[:tokens], w[:tokens]
 
     def step():
-        counts, psum, r2row, r2route = baseline.layout(ids, cfg["experts"])
-        baseline.dispatch_fp8(xs, ws, r2route, cfg["topk"])
+        counts, psum, r2row, r2route = baseline.layout(idx, cfg["experts"])
+        baseline.dispatch_fp8(x, w, r2route, cfg["topk"])
         baseline.combine(grads[: r2route.numel()], r2row)
         return r2route.numel()
 
-    rows = step()
+    for _ in range(3):
+        rows = step()
     times = []
-    for _ in range(5):
+    for _ in range(10):
         t0 = time.perf_counter_ns()
         step()
         times.append((time.perf_counter_ns() - t0) / 1e9)
     mean = sum(times) / len(times)
-    sample_bytes = algorithmic_bytes(tokens, cfg["hidden"], cfg["topk"], rows)
-    moved = sample_bytes["dispatch"] + sample_bytes["combine"]
-    model = "unknown"
-    try:
-        for line in open("/proc/cpuinfo"):
-            if line.startswith("model name"):
-                model = line.split(":", 1)[1].strip()
-                break
-    except OSError:
-        pass
+    nbytes = algorithmic_bytes(cfg["tokens"], cfg["hidden"], cfg["topk"], rows)
+    moved = nbytes["dispatch"] + nbytes["combine"]
     return dict(
         value=moved / mean / 1e9,
         unit="GB/s",
         cores=cores,
         kind="port",
-        sample=f"first {tokens} tokens of the same batch ({rows} rows), 1 warm-up + 5 timed passes, "
-        f"mean {mean * 1e3:.1f} ms per pass, torch CPU {torch.get_num_threads()} threads, {model}",
+        sample=f"the full batch ({cfg['tokens']} tokens, {rows} rows), 3 warm-ups + 10 timed passes, mean {mean * 1e3:.1f} ms "
+        f"(min {min(times) * 1e3:.1f}) per pass of layout + FP8 quantise + expand + combine, torch CPU "
+        f"{torch.get_num_threads()} threads, {cpu_model()}",
     )
 
 
-MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 (the mixed FP8 x FP4 MFMA issues at the FP8 cadence)
+def megamoe_cpu_baseline(hidden, inter):
+    """The reference's CPU form of the expert FFN (reference.py:84-89) on dequantised fp32 operands, the two
+    contractions by torch.matmul: one expert, a sample of 256 of its rows, 3 warm-ups + 10 timed passes."""
+    import numpy as np
+    import torch
+
+    from oracle import baseline
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    rows = 256
+    rng = np.random.default_rng(0)
+    x = torch.from_numpy(rng.normal(size=(rows, hidden)).astype(np.float32))
+    w1 = torch.from_numpy((rng.normal(size=(2 * inter, hidden)) * 0.02).astype(np.float32))
+    w2 = torch.from_numpy((rng.normal(size=(hidden, inter)) * 0.02).astype(np.float32))
+    for _ in range(3):
+        baseline.megamoe_expert_forward(x, w1, w2)
+    times = []
+    for _ in range(10):
+        t0 = time.perf_counter_ns()
+        baseline.megamoe_expert_forward(x, w1, w2)
+        times.append((time.perf_counter_ns() - t0) / 1e9)
+    mean = sum(times) / len(times)
+    flops = 2.0 * rows * hidden * 2 * inter + 2.0 * rows * inter * hidden
+    return dict(
+        value=flops / mean / 1e12,
+        unit="TFLOP/s",
+        cores=cores,
+        kind="port",
+        sample=f"{rows} rows of one expert (H={hidden}, I={inter}: {flops / 1e9:.1f} GFLOP), dense fp32 weights as the oracle "
+        f"materialises them, 3 warm-ups + 10 timed passes, mean {mean * 1e3:.1f} ms, torch CPU {torch.get_num_threads()} "
+        f"threads, {cpu_model()}",
+    )
 
 
-def megamoe_bench(torch, ops, dev, iters):
+def megamoe_bench(torch, ops, timer, with_cpu):
     """W4A8 fused expert FFN for one EP64 rank's share: 64 source ranks x 256 tokens, 384 experts of which
-    6 are local, top-8 uniform routing (about 2048 rows), H=7168, I=2048.  Random codes: the arithmetic
-    does not depend on the values.  FLOPs = 2*R*H*2I + 2*R*I*H for the R rows that reach a local expert."""
+    6 are local, top-8 uniform routing (about 2048 rows), H=7168, I=2048.  Random codes and constant scale bytes: the
+    time does not depend on the values.  FLOPs = 2*R*H*2I + 2*R*I*H for the R rows that reach a local expert."""
+    dev = "cuda"
     tokens, hidden, inter, experts, local, topk = 64 * 256, 7168, 2048, 384, 6, 8
     gen = torch.Generator().manual_seed(0)
     idx = torch.multinomial(torch.ones(tokens, experts), topk, generator=gen).to(torch.int32).to(dev)
@@ -148,36 +223,154 @@ def megamoe_bench(torch, ops, dev, iters):
         calls[0] += 1
         ops.megamoe_forward(ws, x_codes, x_scales, idx, w, w1, s1, w2, s2, experts, 0, local, y, counts)
 
-    us = time_kernel(run, iters, torch)
+    us = timer.back_to_back(run)
+    cold = timer.flushed(run)
     rows = int(counts.sum().item())
     flops = 2.0 * rows * hidden * 2 * inter + 2.0 * rows * inter * hidden
     ws.destroy()
-    return {
+    result = {
         "workload": "EP64 rank share: 16384 candidate tokens, 6 of 384 experts local, top-8, H=7168, I=2048, "
-        "MXFP8 activations x MXFP4 weights, three weight sets in turn; layout + GMM1(+SwiGLU+requant) + GMM2 + "
-        "weighted reduce",
+        "MXFP8 activations x MXFP4 weights (random codes, constant scale bytes), three weight sets in turn; layout + "
+        "GMM1(+SwiGLU+requant) + GMM2 + weighted reduce into [16384,7168] (rows of unserved tokens zero-filled)",
         "rows": rows,
         "us_forward": us,
+        "flushed_us": cold,
         "gflop": flops / 1e9,
         "tflops_forward": flops / us / 1e6,
         "roofline": {"bound": "mfma", "achieved": flops / us / 1e6, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
-                     "note": "whole forward (4 launches); per-kernel GEMM times are in profiles/"},
+                     "note": "whole forward (4 launches), back to back; per-kernel GEMM times are in profiles/"},
     }
+    if with_cpu:
+        result["cpu_baseline"] = megamoe_cpu_baseline(hidden, inter)
+    return result
+
+
+def decode_kernels(torch, ops, cases, timer):
+    """Decode shape (T=128, H=7168, 256 experts, top-8 uniform, all experts local): BF16 dispatch with expand +
+    weighted combine, and their layout."""
+    dev = "cuda"
+    x, idx, w, cfg = cases.make_inputs("C2", seed=0)
+    tokens, hidden, topk, experts = cfg["tokens"], cfg["hidden"], cfg["topk"], cfg["experts"]
+    xd, idxd, wd = x.to(dev), idx.to(dev), w.to(dev)
+    ws = ops.Workspace(1 << 20)
+    lay = ops.layout(ws, idxd, experts)
+    _, rows = ops.layout_wait(ws)
+    r2row, r2route = lay["route_to_row"], lay["row_to_route"]
+    recv, _, recv_w = ops.dispatch_copy(xd, None, wd, r2row, r2route, rows)
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    dispatch_bytes = tokens * hidden * 2 + tokens * topk * 8 + rows * hidden * 2 + rows * 4
+    combine_bytes = rows * hidden * 2 + rows * 4 + tokens * topk * 4 + tokens * hidden * 2
+    entries = {
+        "layout": timer.kernel(lambda: ops.layout(ws, idxd, experts), tokens * topk * 16, head_start=True),
+        "dispatch_bf16": timer.kernel(lambda: ops.dispatch_copy(xd, None, wd, r2row, r2route, rows), dispatch_bytes, head_start=True),
+        "combine_weighted": timer.kernel(lambda: ops.combine(recv, r2row, recv_w, out=out), combine_bytes, head_start=True),
+        # what a fresh dispatch of this size runs: layout and payload in one launch
+        "layout_dispatch_bf16_one_launch": timer.kernel(
+            lambda: ops.layout_dispatch_small(ws, idxd, xd, None, wd, experts), dispatch_bytes + tokens * topk * 8, head_start=True),
+    }
+    ws.destroy()
+    return {"workload": f"decode: T={tokens}, H={hidden}, {experts} experts, top-{topk} uniform, {rows} rows", "kernels": entries}
+
+
+def rank_share_kernels(torch, ops, cases, timer):
+    """One EP64 rank's receive share (64 x 256 candidate tokens, 6 of 384 experts local): layout, fused FP8 dispatch
+    of the rows that hit a local expert, weighted combine back into [16384,H]."""
+    dev = "cuda"
+    x, idx, w, cfg = cases.make_inputs("C4", seed=0)
+    tokens, hidden, topk, experts, local = cfg["tokens"], cfg["hidden"], cfg["topk"], cfg["experts"], cfg["num_local"]
+    xd, idxd, wd = x.to(dev), idx.to(dev), w.to(dev)
+    ws = ops.Workspace(1 << 20)
+    lay = ops.layout(ws, idxd, experts, 0, local)
+    _, rows = ops.layout_wait(ws, local)
+    r2row, r2route = lay["route_to_row"], lay["row_to_route"]
+    recv_w = ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows)[2]
+    y = torch.randn(rows, hidden, generator=torch.Generator().manual_seed(1)).bfloat16().to(dev)
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    served = int((r2row >= 0).any(dim=1).sum().item())
+    dispatch_bytes = tokens * topk * 8 + rows * hidden * 2 + rows * (hidden + (hidden // 128) * 4 + 4)
+    combine_bytes = rows * hidden * 2 + rows * 4 + tokens * topk * 4 + served * hidden * 2
+    zero_fill = (tokens - served) * hidden * 2
+    entries = {
+        "layout": timer.kernel(lambda: ops.layout(ws, idxd, experts, 0, local), tokens * topk * 16, head_start=True),
+        "dispatch_fp8_quant": timer.kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), dispatch_bytes, head_start=True),
+        "combine_weighted": timer.kernel(
+            lambda: ops.combine(y, r2row, recv_w, out=out), combine_bytes,
+            extra={"zero_fill_bytes": zero_fill,
+                   "note": "rows of unserved tokens are zero-filled, not skipped: the kernel also writes zero_fill_bytes, "
+                   "which `bytes` (the survey's algorithmic figure) leaves out"}),
+    }
+    entries["combine_weighted"]["GBps_with_zero_fill"] = (combine_bytes + zero_fill) / entries["combine_weighted"]["us"] / 1e3
+    ws.destroy()
+    return {"workload": f"EP64 rank share: {tokens} candidate tokens, {local} of {experts} experts local, top-{topk} uniform, "
+            f"H={hidden}, {rows} rows, {served} served tokens", "kernels": entries}
+
+
+def read_traffic(kernel):
+    """HBM bytes per launch of `kernel` from profiles/hbm_traffic.json (written by --ingest-pmc), or None."""
+    try:
+        table = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        return None
+    entry = table.get("kernels", {}).get(kernel)
+    return None if entry is None else entry.get("hbm_bytes")
+
+
+def ingest_pmc(fetch_csv, write_csv):
+    """Two rocprofv3 --pmc runs of `bench.py --calibrate-copy` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch) ->
+    profiles/hbm_traffic.json.  Both counters are scaled by what they read for the calibration copy, whose traffic is
+    known: [32768,7168] BF16 rows through dispatch_copy_row_kernel = 458 752 KiB read and as much written."""
+    import csv
+    import re
+
+    def averages(path, counter):
+        sums, calls = {}, {}
+        for row in csv.DictReader(open(path)):
+            if row.get("Counter_Name") != counter:
+                continue
+            name = re.sub(r"\(.*", "", row["Kernel_Name"]).replace("void ", "").replace("dpep::(anonymous namespace)::", "").strip()
+            sums[name] = sums.get(name, 0.0) + float(row["Counter_Value"])
+            calls[name] = calls.get(name, 0) + 1
+        return {name: sums[name] / calls[name] for name in sums}
+
+    fetch, write = averages(fetch_csv, "FETCH_SIZE"), averages(write_csv, "WRITE_SIZE")
+    known_kib = 32768 * 7168 * 2 / 1024
+    copy = "dispatch_copy_row_kernel"
+    if copy not in fetch or copy not in write:
+        raise SystemExit("the counter files hold no dispatch_copy_row_kernel: run bench.py with --calibrate-copy")
+    fetch_scale, write_scale = known_kib / fetch[copy], known_kib / write[copy]
+    kernels = {}
+    for name in sorted(set(fetch) & set(write)):
+        read_bytes, written = fetch[name] * fetch_scale * 1024, write[name] * write_scale * 1024
+        kernels[name] = dict(fetch_kib=fetch[name], write_kib=write[name], hbm_read_bytes=read_bytes, hbm_written_bytes=written,
+                             hbm_bytes=read_bytes + written)
+    table = dict(source="rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs) of `python3 bench.py --calibrate-copy ...`; "
+                 "KiB per dispatch, averaged over the dispatches of each kernel",
+                 fetch_scale=fetch_scale, write_scale=write_scale, calibration_kib=known_kib, kernels=kernels)
+    json.dump(table, open(TRAFFIC_FILE, "w"), indent=1, sort_keys=True)
+    print(f"wrote {TRAFFIC_FILE}: {len(kernels)} kernels, scale factors {fetch_scale:.3f} / {write_scale:.3f}")
 
 
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=50)
-    parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--kernel-iters", type=int, default=50)
+    parser.add_argument("--steps", type=int, default=100)
+    parser.add_argument("--warmup", type=int, default=20)
+    parser.add_argument("--kernel-iters", type=int, default=100, help="timed launches per kernel (each protocol)")
+    parser.add_argument("--kernel-warmup", type=int, default=20, help="untimed launches per kernel before them")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-megamoe", action="store_true", help="skip the W4A8 expert-FFN measurement")
+    parser.add_argument("--no-extra-shapes", action="store_true", help="skip the decode and rank-share kernel timings")
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="also launch a plain copy of known size (identity dispatch of [32768,7168] BF16: 469.76 MB "
                         "read + 469.76 MB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled")
+    parser.add_argument("--ingest-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"))
+    parser.add_argument("--protocol", metavar="PRESET", help="run the reference's generic benchmark workload PRESET "
+                        "(smoke, decode, prefill) and print one `measured` record per operation")
     args = parser.parse_args()
+    if args.ingest_pmc:
+        ingest_pmc(*args.ingest_pmc)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU's share; --gpus must be 1 (no multi-GPU path in this build)", file=sys.stderr)
         sys.exit(2)
@@ -192,6 +385,12 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.protocol:
+        from deepep_amd import protocol_bench
+
+        for record in protocol_bench.run(args.protocol, torch, ops, iters=args.kernel_iters, warmups=args.kernel_warmup):
+            print(json.dumps(record))
+        return
 
     x, idx, w, cfg = cases.make_inputs("C3", seed=0)
     tokens, hidden, topk, experts = cfg["tokens"], cfg["hidden"], cfg["topk"], cfg["experts"]
@@ -224,38 +423,23 @@ def main():
     moved = nbytes["dispatch"] + nbytes["combine"]
 
     # Per-kernel device time (HIP events on the launch stream), same inputs.
+    timer = Timer(torch, args.kernel_iters, args.kernel_warmup)
     lay = ops.layout(ws, idxd, experts)
     r2row, r2route = lay["route_to_row"], lay["row_to_route"]
     grows = gd[:rows]
     out_buf = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
-    it = args.kernel_iters
+    q_pre, s_pre = ops.cast_to_fp8(xd)  # the reference semantic: the caller quantises, dispatch moves codes and scales
     recv_w = ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows)[2]
-    head_start = torch.empty(1 << 30, dtype=torch.uint8, device=dev)  # 8 fills of 1 GiB: about 1.4 ms
-    us = dict(
-        layout=time_kernel(lambda: ops.layout(ws, idxd, experts), min(it, 40), torch, head_start),
-        dispatch_fp8_quant=time_kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), it, torch),
-        dispatch_bf16=time_kernel(lambda: ops.dispatch_copy(xd, None, wd, r2row, r2route, rows), it, torch),
-        combine=time_kernel(lambda: ops.combine(grows, r2row, out=out_buf), it, torch),
-        combine_weighted=time_kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), it, torch),
-    )
-    del head_start
-    flush = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
-    cold = dict(
-        dispatch_fp8_quant=time_kernel_cold(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), 30, torch, flush),
-        combine=time_kernel_cold(lambda: ops.combine(grows, r2row, out=out_buf), 30, torch, flush),
-    )
-    del flush
     bf16_dispatch_bytes = tokens * hidden * 2 + tokens * topk * 4 + rows * hidden * 2 + rows * 4
+    copy_dispatch_bytes = tokens * (hidden + (hidden // 128) * 4) + tokens * topk * 4 + rows * (hidden + (hidden // 128) * 4 + 4)
     kernels = {
-        "layout": dict(us=us["layout"], bytes=nbytes["layout"]),
-        "dispatch_fp8_quant": dict(us=us["dispatch_fp8_quant"], bytes=nbytes["dispatch"]),
-        "dispatch_bf16": dict(us=us["dispatch_bf16"], bytes=bf16_dispatch_bytes),
-        "combine": dict(us=us["combine"], bytes=nbytes["combine"]),
-        "combine_weighted": dict(us=us["combine_weighted"], bytes=nbytes["combine"] + rows * 4),
+        "layout": timer.kernel(lambda: ops.layout(ws, idxd, experts), nbytes["layout"], head_start=True),
+        "dispatch_fp8_quant": timer.kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), nbytes["dispatch"]),
+        "dispatch_fp8_copy": timer.kernel(lambda: ops.dispatch_copy(q_pre, s_pre, wd, r2row, r2route, rows), copy_dispatch_bytes),
+        "dispatch_bf16": timer.kernel(lambda: ops.dispatch_copy(xd, None, wd, r2row, r2route, rows), bf16_dispatch_bytes),
+        "combine": timer.kernel(lambda: ops.combine(grows, r2row, out=out_buf), nbytes["combine"]),
+        "combine_weighted": timer.kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), nbytes["combine"] + rows * 4),
     }
-    for entry in kernels.values():
-        entry["GBps"] = entry["bytes"] / entry["us"] / 1e3
-        entry["frac_of_8TBps"] = entry["GBps"] / HBM_PEAK_GBS
 
     dominant = kernels["combine"]
     result = {
@@ -280,6 +464,9 @@ def main():
             "experts": experts,
             "rows": rows,
             "bytes_per_step": moved,
+            "kernel_timing": f"{args.kernel_warmup} warm-ups + {args.kernel_iters} launches per kernel and protocol; "
+            "`us` / `GBps` / `frac_of_8TBps` are the cache-flushed mean (256 MiB fill before every launch), "
+            "`back_to_back_us` / `frac_back_to_back` the same launches queued without gaps",
         },
         "roofline": {
             "kernel": "combine_kernel<0, false>",
@@ -287,25 +474,31 @@ def main():
             "achieved": dominant["GBps"],
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": dominant["GBps"] / HBM_PEAK_GBS,
-            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of known
-            # size (factors 1.991 / 1.000): 468.7 MB read + 58.7 MB written (profiles/prefill_hbm_traffic_pmc.md)
-            "traffic": 527.5e6,
+            "frac": dominant["frac_of_8TBps"],
+            "protocol": "mean of cache-flushed launches (256 MiB fill before each); back to back: "
+            f"{dominant['GBps_back_to_back']:.0f} GB/s = {dominant['frac_back_to_back']:.3f}",
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by a plain copy of known
+            # size; read from the file `--ingest-pmc` writes
+            "traffic": read_traffic("combine_kernel<0, false>"),
         },
         "kernels": kernels,
-        "kernels_cache_flushed_us": cold,
-        "dispatch_plus_combine_us": us["dispatch_fp8_quant"] + us["combine"],
+        "dispatch_plus_combine_us": kernels["dispatch_fp8_quant"]["us"] + kernels["combine"]["us"],
+        "dispatch_plus_combine_frac_of_8TBps": moved / (kernels["dispatch_fp8_quant"]["us"] + kernels["combine"]["us"]) / 1e3 / HBM_PEAK_GBS,
     }
     if args.calibrate_copy:
         ident = torch.arange(rows, dtype=torch.int32, device=dev)
         for _ in range(5):
             ops.dispatch_copy(gd[:rows], None, None, ident.view(rows, 1), ident, rows)
         torch.cuda.synchronize()
-    if not args.no_megamoe:
-        result["megamoe"] = megamoe_bench(torch, ops, dev, args.kernel_iters)
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(x, idx, w, grads, cfg, nbytes)
     ws.destroy()
+    del gd, grows, out_buf, q_pre, s_pre
+    if not args.no_extra_shapes:
+        result["decode"] = decode_kernels(torch, ops, cases, timer)
+        result["rank_share"] = rank_share_kernels(torch, ops, cases, timer)
+    if not args.no_megamoe:
+        result["megamoe"] = megamoe_bench(torch, ops, timer, not args.no_cpu_baseline)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(x, idx, w, grads, cfg)
     print(json.dumps(result))
 
 

@@ -30,6 +30,7 @@ SIGNATURES = {
     "dpep_layout_wait": (_I, (_P, _P, _I, ctypes.POINTER(ctypes.c_int32), ctypes.c_longlong)),
     "dpep_dispatch_copy": (_I, (_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_dispatch_quant_fp8": (_I, (_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
+    "dpep_layout_dispatch_small": (_I, (_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P)),
     "dpep_cast_to_fp8": (_I, (_P, _I, _I, _P, _P, _P)),
     "dpep_combine": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_combine_fp16": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),

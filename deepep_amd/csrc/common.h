@@ -94,6 +94,15 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, dpep_f16x2));
 }
 
+// Local expert of a raw id, -1 if the route is past `end` or its expert is not one of this rank's.
+__device__ __forceinline__ int local_expert(long long e, int route, int end, int num_experts, int expert_begin,
+                                            int num_local)
+{
+    const long long local = e - expert_begin;
+    const bool valid = route < end && e >= 0 && e < num_experts && local >= 0 && local < num_local;
+    return valid ? static_cast<int>(local) : -1;
+}
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 

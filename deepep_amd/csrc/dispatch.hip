@@ -25,6 +25,13 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
     __shared__ int rows[DPEP_MAX_TOPK];
     __shared__ int any_valid;
     const int token = blockIdx.x / parts, part = blockIdx.x % parts;
+    const int v_begin = part * vec_per_part;
+    const int v_end = min(v_begin + vec_per_part, vec_per_row);
+    const u32x4* src = x + static_cast<size_t>(token) * vec_per_row;
+    // The token's first values are asked for before its routes are known (see the quantising kernel below).
+    const int v_first = v_begin + threadIdx.x;
+    u32x4 first = {0u, 0u, 0u, 0u};
+    if (v_first < v_end) first = load16(src + v_first);  // plain loads with streaming stores measured fastest here
     if (threadIdx.x == 0) any_valid = 0;
     __syncthreads();
     if (threadIdx.x < num_topk) {
@@ -34,11 +41,8 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
     }
     __syncthreads();
     if (!any_valid) return;
-    const int v_begin = part * vec_per_part;
-    const int v_end = min(v_begin + vec_per_part, vec_per_row);
-    const u32x4* src = x + static_cast<size_t>(token) * vec_per_row;
-    for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x) {
-        const u32x4 value = load16(src + v);  // plain loads with streaming stores measured fastest here
+    for (int v = v_first; v < v_end; v += blockDim.x) {
+        const u32x4 value = v == v_first ? first : load16(src + v);
         for (int s = 0; s < num_topk; ++s) {
             const int row = rows[s];
             if (row >= 0) store16_nt(out + static_cast<size_t>(row) * vec_per_row + v, value);
@@ -141,6 +145,22 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
     __shared__ int any_valid;
     __shared__ float part_scales[kMaxScaleCols];
     const int token = blockIdx.x / parts, part = blockIdx.x % parts;
+    const int u_begin = part * units_per_part;
+    const int u_end = min(u_begin + units_per_part, units_per_row);
+    const u32x4* src = x + static_cast<size_t>(token) * units_per_row * 2;
+    // The token's first values are asked for before its routes are known: this grid is only used where most tokens own
+    // rows, and the row lookup and the payload then travel together instead of one after the other.
+    const int u_first = u_begin + threadIdx.x;
+    constexpr int kEarly = 2;  // units per thread fetched up front (all of a 7168-wide row with 256 threads)
+    u32x4 lo[kEarly], hi[kEarly];
+#pragma unroll
+    for (int j = 0; j < kEarly; ++j) {
+        const int u = u_first + j * static_cast<int>(blockDim.x);
+        if (u < u_end) {
+            lo[j] = load16(src + 2 * u);
+            hi[j] = load16(src + 2 * u + 1);
+        }
+    }
     if (threadIdx.x == 0) any_valid = 0;
     __syncthreads();
     if (threadIdx.x < num_topk) {
@@ -150,12 +170,29 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
     }
     __syncthreads();
     if (!any_valid) return;
-    const int u_begin = part * units_per_part;
-    const int u_end = min(u_begin + units_per_part, units_per_row);
     const int scale_cols = units_per_row / 8;
-    const u32x4* src = x + static_cast<size_t>(token) * units_per_row * 2;
     // units_per_part is a multiple of 8 and blockDim of 64, so the 8 lanes of a block stay together.
-    for (int u = u_begin + threadIdx.x; u < u_end; u += blockDim.x) {
+    // Quantise first, then write row by row: at any moment the workgroup's stores run along ONE output row.
+    u32x4 codes[kEarly];
+#pragma unroll
+    for (int j = 0; j < kEarly; ++j) {
+        const int u = u_first + j * static_cast<int>(blockDim.x);
+        if (u < u_end) {
+            const Quant16 q = quantize16(lo[j], hi[j]);
+            codes[j] = q.codes;
+            if ((u & 7) == 0) part_scales[(u - u_begin) >> 3] = q.scale;
+        }
+    }
+    for (int s = 0; s < num_topk; ++s) {
+        const int row = rows[s];
+        if (row < 0) continue;
+#pragma unroll
+        for (int j = 0; j < kEarly; ++j) {
+            const int u = u_first + j * static_cast<int>(blockDim.x);
+            if (u < u_end) store16_nt(out + static_cast<size_t>(row) * units_per_row + u, codes[j]);
+        }
+    }
+    for (int u = u_first + kEarly * static_cast<int>(blockDim.x); u < u_end; u += blockDim.x) {  // rows wider than that
         const Quant16 q = quantize16(load16(src + 2 * u), load16(src + 2 * u + 1));
         for (int s = 0; s < num_topk; ++s) {
             const int row = rows[s];
@@ -196,6 +233,175 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_row_kernel(
         if ((u & 7) == 0) out_scales[static_cast<size_t>(row) * scale_cols + (u >> 3)] = q.scale;
     }
     if (part == 0 && weights != nullptr && threadIdx.x == 0) out_weights[row] = weights[route];
+}
+
+// ---- small batches: routing layout and payload in ONE launch -------------------------------------------------
+// With at most kSmallRoutes routes (a decode step) the whole routing table fits a workgroup's LDS, and a workgroup
+// gets the rows of its own token faster by working them out itself than by waiting for a layout kernel: every
+// workgroup (one per token and column part) reads all ids, histograms them (LDS atomics: a count does not depend on
+// order), scans the histogram over the experts, and counts, for each of its token's routes, the earlier routes with
+// the same expert.  row = first row of the expert + that count: the same stable permutation the layout kernels
+// produce.  Nothing travels between workgroups.  Part 0 of each token writes the token's entries of route_to_row and
+// row_to_route, workgroup 0 the per-expert outputs and the host mailbox.
+constexpr int kSmallRoutes = 2048;
+
+template <bool kQuant>
+__global__ __launch_bounds__(kMaxThreads) void layout_dispatch_small_kernel(
+    const long long* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int num_topk,
+    const u32x4* __restrict__ x, const float* __restrict__ scales, const float* __restrict__ weights, int units_per_row,
+    int units_per_part, int parts, int scale_cols, int* __restrict__ counts, int* __restrict__ psum, int* __restrict__ offsets,
+    int* __restrict__ num_rows, int* __restrict__ route_to_row, int* __restrict__ row_to_route, u32x4* __restrict__ out,
+    float* __restrict__ out_scales, float* __restrict__ out_weights, uint32_t* __restrict__ mailbox, uint32_t sequence)
+{
+    __shared__ short local_id[kSmallRoutes];
+    __shared__ int first_row[DPEP_MAX_LOCAL_EXPERTS];  // per expert: count, then exclusive prefix
+    __shared__ int before[DPEP_MAX_TOPK];
+    __shared__ int rows[DPEP_MAX_TOPK];
+    __shared__ int wave_sums[kMaxThreads / kWave];
+    __shared__ float part_scales[kMaxScaleCols];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int token = blockIdx.x / parts, part = blockIdx.x % parts;
+    // in units of 16 bytes of input (kQuant: 32 bytes = 16 BF16 values = 16 bytes of output)
+    const int u_begin = part * units_per_part, u_end = min(u_begin + units_per_part, units_per_row);
+    constexpr int kIn = kQuant ? 2 : 1;
+    const u32x4* src = x + static_cast<size_t>(token) * units_per_row * kIn;
+    // the payload is asked for first: it does not depend on the routing
+    constexpr int kEarly = 2;
+    u32x4 early[kEarly][kIn];
+#pragma unroll
+    for (int j = 0; j < kEarly; ++j) {
+        const int u = u_begin + tid + j * kMaxThreads;
+        if (u < u_end) {
+#pragma unroll
+            for (int h = 0; h < kIn; ++h) early[j][h] = load16(src + kIn * u + h);
+        }
+    }
+    for (int e = tid; e < num_local; e += kMaxThreads) first_row[e] = 0;
+    if (tid < DPEP_MAX_TOPK) before[tid] = 0;
+    __syncthreads();
+    for (int j = tid; j < n_routes; j += kMaxThreads) {
+        const int e = local_expert(idx[j], j, n_routes, num_experts, expert_begin, num_local);
+        local_id[j] = static_cast<short>(e);
+        if (e >= 0) atomicAdd(&first_row[e], 1);
+    }
+    __syncthreads();
+    // exclusive scan over the experts: four consecutive experts per thread, wave scan, then the waves' sums
+    int mine[4], sum = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = tid * 4 + j;
+        mine[j] = e < num_local ? first_row[e] : 0;
+        sum += mine[j];
+    }
+    int incl = sum;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) wave_sums[wave] = incl;
+    __syncthreads();
+    int offset = incl - sum;
+    for (int w = 0; w < wave; ++w) offset += wave_sums[w];
+    const bool reporter = blockIdx.x == 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = tid * 4 + j;
+        if (e < num_local) {
+            first_row[e] = offset;
+            if (reporter) {
+                counts[e] = mine[j];
+                psum[e] = offset + mine[j];
+                offsets[e + 1] = offset + mine[j];
+                if (mailbox != nullptr)
+                    __hip_atomic_store(mailbox + 2 + e, static_cast<uint32_t>(mine[j]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+        offset += mine[j];
+    }
+    if (reporter && tid == kMaxThreads - 1) {
+        offsets[0] = 0;
+        num_rows[0] = offset;  // the last thread's running offset is the total
+    }
+    if (reporter && mailbox != nullptr) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's counts have reached the host
+    __syncthreads();
+    if (reporter && mailbox != nullptr && tid == kMaxThreads - 1) {
+        const unsigned long long word = (static_cast<unsigned long long>(sequence) << 32) | static_cast<uint32_t>(offset);
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    // earlier routes with the same expert, for each route of this token
+    const int my_first = token * num_topk;
+    int want[DPEP_MAX_TOPK], seen[DPEP_MAX_TOPK];
+#pragma unroll
+    for (int s = 0; s < DPEP_MAX_TOPK; ++s) {
+        want[s] = s < num_topk ? local_id[my_first + s] : -1;
+        seen[s] = 0;
+    }
+    for (int j = tid; j < my_first + num_topk; j += kMaxThreads) {
+        const int e = local_id[j];
+        if (e < 0) continue;
+#pragma unroll
+        for (int s = 0; s < DPEP_MAX_TOPK; ++s)
+            if (s < num_topk && e == want[s] && j < my_first + s) ++seen[s];
+    }
+#pragma unroll
+    for (int s = 0; s < DPEP_MAX_TOPK; ++s)
+        if (seen[s] != 0) atomicAdd(&before[s], seen[s]);
+    __syncthreads();
+    if (tid < num_topk) {
+        const int e = local_id[my_first + tid];
+        const int row = e >= 0 ? first_row[e] + before[tid] : -1;
+        rows[tid] = row;
+        if (part == 0) {
+            route_to_row[my_first + tid] = row;
+            if (row >= 0) {
+                row_to_route[row] = my_first + tid;
+                if (weights != nullptr) out_weights[row] = weights[my_first + tid];
+            }
+        }
+    }
+    __syncthreads();
+    // payload: read once, write to every row of the token
+    auto emit = [&](int u, const u32x4 (&in)[kIn]) {
+        u32x4 value = in[0];
+        if (kQuant) {
+            const Quant16 q = quantize16(in[0], in[kIn - 1]);
+            value = q.codes;
+            if ((u & 7) == 0) part_scales[(u - u_begin) >> 3] = q.scale;
+        }
+        for (int s = 0; s < num_topk; ++s) {
+            const int row = rows[s];
+            if (row >= 0) store16_nt(out + static_cast<size_t>(row) * units_per_row + u, value);
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < kEarly; ++j) {
+        const int u = u_begin + tid + j * kMaxThreads;
+        if (u < u_end) emit(u, early[j]);
+    }
+    for (int u = u_begin + tid + kEarly * kMaxThreads; u < u_end; u += kMaxThreads) {
+        u32x4 in[kIn];
+#pragma unroll
+        for (int h = 0; h < kIn; ++h) in[h] = load16(src + kIn * u + h);
+        emit(u, in);
+    }
+    if (kQuant) {
+        __syncthreads();
+        const int part_cols = (u_end - u_begin) >> 3, col0 = u_begin >> 3, out_cols = units_per_row / 8;
+        for (int i = tid; i < num_topk * part_cols; i += kMaxThreads) {
+            const int s = i / part_cols, c = i - s * part_cols;
+            const int row = rows[s];
+            if (row >= 0) out_scales[static_cast<size_t>(row) * out_cols + col0 + c] = part_scales[c];
+        }
+    } else if (part == 0 && scales != nullptr) {
+        for (int c = tid; c < scale_cols; c += kMaxThreads) {
+            const float value = scales[static_cast<size_t>(token) * scale_cols + c];
+            for (int s = 0; s < num_topk; ++s) {
+                const int row = rows[s];
+                if (row >= 0) out_scales[static_cast<size_t>(row) * scale_cols + c] = value;
+            }
+        }
+    }
 }
 
 // Split a row of `units` work items over `parts` workgroups so that a launch of `rows` rows has
@@ -292,6 +498,57 @@ int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int3
                        static_cast<const u32x4*>(x), topk_weights, row_to_route, num_topk, units, sp.per_part, sp.parts,
                        static_cast<u32x4*>(out), out_scales, out_weights);
     return launch_status("dispatch_quant_row");
+}
+
+int dpep_layout_dispatch_small(void* ws, const int64_t* topk_idx, const void* x, const float* scales,
+                               const float* topk_weights, int num_tokens, int num_topk, int num_experts, int expert_begin,
+                               int num_local, int row_bytes, int scale_cols, int quantize, int32_t* counts, int32_t* psum,
+                               int32_t* offsets, int32_t* route_to_row, int32_t* row_to_route, int32_t* num_rows, void* out,
+                               float* out_scales, float* out_weights, void* stream)
+{
+    using namespace dpep;
+    Workspace* w = as_workspace(ws);
+    DPEP_REQUIRE(w != nullptr, "layout_dispatch_small: not a live workspace");
+    DPEP_REQUIRE(num_tokens >= 1 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK &&
+                     static_cast<long long>(num_tokens) * num_topk <= kSmallRoutes,
+                 "layout_dispatch_small: T=%d K=%d: needs 1 <= T*K <= %d routes (larger batches take dpep_layout and a "
+                 "dispatch call)", num_tokens, num_topk, kSmallRoutes);
+    DPEP_REQUIRE(num_experts >= 1 && expert_begin >= 0 && num_local >= 1 && num_local <= DPEP_MAX_LOCAL_EXPERTS &&
+                     expert_begin + num_local <= num_experts,
+                 "layout_dispatch_small: bad expert range E=%d begin=%d L=%d", num_experts, expert_begin, num_local);
+    DPEP_REQUIRE(topk_idx && counts && psum && offsets && route_to_row && row_to_route && num_rows, "layout_dispatch_small: NULL routing buffer");
+    DPEP_REQUIRE(x && out && aligned16(x) && aligned16(out), "layout_dispatch_small: x/out must be 16-byte aligned");
+    DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "layout_dispatch_small: weights and out_weights go together");
+    int units = 0;
+    if (quantize) {
+        DPEP_REQUIRE(row_bytes > 0 && row_bytes % 256 == 0 && row_bytes / 256 <= kMaxScaleCols,
+                     "layout_dispatch_small: a quantised row needs a BF16 width that is a multiple of 128 (row_bytes=%d)", row_bytes);
+        DPEP_REQUIRE(scales == nullptr && out_scales != nullptr, "layout_dispatch_small: the fused quantiser takes no input scales and needs out_scales");
+        units = row_bytes / 32;
+    } else {
+        DPEP_REQUIRE(row_bytes > 0 && row_bytes % 16 == 0, "layout_dispatch_small: row_bytes=%d must be a positive multiple of 16", row_bytes);
+        DPEP_REQUIRE((scales == nullptr) == (out_scales == nullptr), "layout_dispatch_small: scales and out_scales go together");
+        DPEP_REQUIRE(scales == nullptr || scale_cols > 0, "layout_dispatch_small: scale_cols must be positive with scales");
+        units = row_bytes / 16;
+    }
+    w->sequence = w->sequence == 0xffffffffu ? 1u : w->sequence + 1u;  // never 0: that is "nothing launched"
+    w->mailbox_local = num_local;
+    const Split sp = choose_split(num_tokens, units, 8);
+    const int n_routes = num_tokens * num_topk;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (quantize)
+        hipLaunchKernelGGL(layout_dispatch_small_kernel<true>, dim3(num_tokens * sp.parts), dim3(kMaxThreads), 0, s,
+                           reinterpret_cast<const long long*>(topk_idx), n_routes, num_experts, expert_begin, num_local, num_topk,
+                           static_cast<const u32x4*>(x), nullptr, topk_weights, units, sp.per_part, sp.parts, 0, counts, psum, offsets,
+                           num_rows, route_to_row, row_to_route, static_cast<u32x4*>(out), out_scales, out_weights,
+                           w->mailbox_device, w->sequence);
+    else
+        hipLaunchKernelGGL(layout_dispatch_small_kernel<false>, dim3(num_tokens * sp.parts), dim3(kMaxThreads), 0, s,
+                           reinterpret_cast<const long long*>(topk_idx), n_routes, num_experts, expert_begin, num_local, num_topk,
+                           static_cast<const u32x4*>(x), scales, topk_weights, units, sp.per_part, sp.parts, scale_cols, counts, psum,
+                           offsets, num_rows, route_to_row, row_to_route, static_cast<u32x4*>(out), out_scales, out_weights,
+                           w->mailbox_device, w->sequence);
+    return launch_status("layout_dispatch_small");
 }
 
 int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float* out_scales, void* stream)

@@ -49,15 +49,6 @@ __device__ __forceinline__ void wave_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Local expert of a raw id, -1 if the route is past `end` or its expert is not one of this rank's.
-__device__ __forceinline__ int local_expert(long long e, int route, int end, int num_experts, int expert_begin,
-                                            int num_local)
-{
-    const long long local = e - expert_begin;
-    const bool valid = route < end && e >= 0 && e < num_experts && local >= 0 && local < num_local;
-    return valid ? static_cast<int>(local) : -1;
-}
-
 // Local experts of kSteps consecutive 64-route steps from `base` on.  All loads are issued before the first is
 // used (a route past the end reads the last id instead of branching around the load), so that the wave pays
 // one memory latency for the batch, not one per step.  Needs n_routes > 0.

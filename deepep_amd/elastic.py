@@ -552,13 +552,23 @@ class ElasticBuffer:
                         return native.dispatch_copy(hidden, scales, topk_weights, route_to_row, row_to_route, rows)
 
                     if handle is None:
-                        plan, indices = self._notify_launch(topk_idx, num_experts, do_handle_copy)
-                        route_to_row, row_to_route = plan["route_to_row"], plan["row_to_route"]
                         # Where most routes stay on this rank, outputs allocated for all T*K routes cost little, and
                         # the payload kernel can be queued right behind the layout: the host reads R while both
-                        # run and narrows the outputs, instead of leaving the GPU idle between the two.
+                        # run and narrows the outputs, instead of leaving the GPU idle between the two.  A small
+                        # batch (a decode step) goes further: layout and payload are one launch.
                         early = 2 * (num_experts // world) >= num_experts
-                        full = payload(None) if early else None
+                        if early and 1 <= tokens * topk <= native.SMALL_BATCH_ROUTES:
+                            local = num_experts // world
+                            with torch.inference_mode(False), torch.no_grad():
+                                indices = topk_idx.clone() if do_handle_copy else topk_idx
+                                plan, *full = native.layout_dispatch_small(
+                                    runtime.workspace, indices, hidden, scales, topk_weights, num_experts, runtime.rank * local,
+                                    local, quantize=fuse_quant)
+                            route_to_row, row_to_route = plan["route_to_row"], plan["row_to_route"]
+                        else:
+                            plan, indices = self._notify_launch(topk_idx, num_experts, do_handle_copy)
+                            route_to_row, row_to_route = plan["route_to_row"], plan["row_to_route"]
+                            full = payload(None) if early else None
                         handle = self._notify_finish(hidden, plan, indices, num_experts, capacity)
                         rows = handle.num_expanded_tokens
                         if early:
@@ -655,19 +665,23 @@ class ElasticBuffer:
                 producer = EventHandle()
                 with gpu_api().stream(runtime.stream):
                     producer.current_stream_wait()
+                    # The payload kernel does not depend on R.  Batches of up to SMALL_BATCH_ROUTES routes (every
+                    # low-latency batch with the usual top-k) take one launch for layout and payload; larger ones
+                    # queue the payload kernel right behind the layout.  (Experts repeated within a token are
+                    # outside the low-latency contract; their surplus rows fall beyond C and are dropped from the
+                    # returned view, never written out of bounds.)
                     with torch.inference_mode(False), torch.no_grad():
                         indices = topk_idx.clone() if do_handle_copy else topk_idx
-                        layout = native.layout(runtime.workspace, indices, num_experts, begin, local)
-                    # The payload kernel does not depend on R: it is queued right behind the layout.  (Experts
-                    # repeated within a token are outside the low-latency contract; their surplus rows fall
-                    # beyond C and are dropped from the returned view, never written out of bounds.)
-                    out, out_scales, row_weights = (
-                        None if t is None else t[:rows]
-                        for t in native.dispatch_copy(
-                            hidden, scales, topk_weights, layout["route_to_row"], layout["row_to_route"], None,
-                            capacity_rows=rows,
-                        )
-                    )
+                        if tokens * topk <= native.SMALL_BATCH_ROUTES:
+                            layout, *moved = native.layout_dispatch_small(
+                                runtime.workspace, indices, hidden, scales, topk_weights, num_experts, begin, local,
+                                capacity_rows=rows)
+                        else:
+                            layout = native.layout(runtime.workspace, indices, num_experts, begin, local)
+                            moved = native.dispatch_copy(
+                                hidden, scales, topk_weights, layout["route_to_row"], layout["row_to_route"], None,
+                                capacity_rows=rows)
+                    out, out_scales, row_weights = (None if t is None else t[:rows] for t in moved)
                     # send_counts[e]: rows of experts 0..e on this rank (inclusive), so that its last entry is R
                     send_counts = torch.zeros((num_experts,), dtype=torch.int32, device=hidden.device)
                     send_counts[begin : begin + local] = layout["psum"]

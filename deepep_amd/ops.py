@@ -196,6 +196,76 @@ def dispatch_copy(x, scales, topk_weights, route_to_row, row_to_route, num_rows:
     return out, out_scales, out_weights
 
 
+SMALL_BATCH_ROUTES = 2048  # T*K up to which layout and dispatch share one launch (dpep_layout_dispatch_small)
+
+
+def layout_dispatch_small(ws: Workspace, topk_idx, x, scales, topk_weights, num_experts: int, expert_begin: int = 0,
+                          num_local: Optional[int] = None, quantize: bool = False, capacity_rows: Optional[int] = None):
+    """Routing layout and payload dispatch of a small batch in one launch (``1 <= T*K <= SMALL_BATCH_ROUTES``).
+
+    Returns ``(layout, out, out_scales, out_weights)``: ``layout`` as from ``layout()`` (``layout_wait`` works on it),
+    the payload outputs as from ``dispatch_copy`` / ``dispatch_quant_fp8`` with ``num_rows=None``: allocated with T*K rows
+    (at least ``capacity_rows``), of which the first R are written."""
+    lib = _lib.load()
+    _require("topk_idx", topk_idx, torch.int64, device=ws.device)
+    if topk_idx.ndim != 2:
+        raise ValueError("topk_idx must be [T, K]")
+    tokens, topk = topk_idx.shape
+    if not 1 <= tokens * topk <= SMALL_BATCH_ROUTES:
+        raise ValueError(f"layout_dispatch_small takes 1..{SMALL_BATCH_ROUTES} routes")
+    dev = topk_idx.device
+    allowed = (torch.bfloat16,) if quantize else (torch.bfloat16, torch.float8_e4m3fn, torch.float16)
+    if not isinstance(x, torch.Tensor) or x.dtype not in allowed:
+        raise ValueError("x must be BF16 (quantize) or a BF16, FP16 or FP8 E4M3FN tensor")
+    _require("x", x, x.dtype, device=dev)
+    if x.ndim != 2 or x.shape[0] != tokens:
+        raise ValueError("x must be [T, H]")
+    hidden = x.shape[1]
+    row_bytes = hidden * x.element_size()
+    if quantize and hidden % 128:
+        raise ValueError("hidden must be a multiple of 128 for FP8 dispatch")
+    if row_bytes % 16:
+        raise ValueError("hidden row size must be a multiple of 16 bytes")
+    num_local = num_experts - expert_begin if num_local is None else num_local
+    rows = max(tokens * topk, capacity_rows or 0)
+    meta = torch.empty(3 * num_local + 2, dtype=torch.int32, device=dev)
+    counts, psum = meta[:num_local], meta[num_local : 2 * num_local]
+    offsets, num_rows = meta[2 * num_local : 3 * num_local + 1], meta[3 * num_local + 1 :]
+    route_to_row = torch.empty((tokens, topk), dtype=torch.int32, device=dev)
+    row_to_route = torch.empty((tokens * topk,), dtype=torch.int32, device=dev)
+    scale_cols = 0
+    out_scales = None
+    if quantize:
+        if scales is not None:
+            raise ValueError("the fused quantiser takes no input scales")
+        out = torch.empty((rows, hidden), dtype=torch.float8_e4m3fn, device=dev)
+        out_scales = torch.empty((rows, hidden // 128), dtype=torch.float32, device=dev)
+    else:
+        out = torch.empty((rows, hidden), dtype=x.dtype, device=dev)
+        if scales is not None:
+            if not isinstance(scales, torch.Tensor) or scales.dtype not in (torch.float32, torch.int32):
+                raise ValueError("scales must be FP32 or packed int32")
+            _require("scales", scales, scales.dtype, device=dev)
+            if scales.ndim != 2 or scales.shape[0] != tokens:
+                raise ValueError("scales must be [T, C]")
+            scale_cols = scales.shape[1]
+            out_scales = torch.empty((rows, scale_cols), dtype=scales.dtype, device=dev)
+    out_weights = None
+    if topk_weights is not None:
+        _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)
+        out_weights = torch.empty((rows,), dtype=torch.float32, device=dev)
+    with _on_device(dev):
+        status = lib.dpep_layout_dispatch_small(
+            ws.handle, _ptr(topk_idx), _ptr(x), _ptr(scales), _ptr(topk_weights), tokens, topk, num_experts, expert_begin,
+            num_local, row_bytes, scale_cols, int(bool(quantize)), _ptr(counts), _ptr(psum), _ptr(offsets), _ptr(route_to_row),
+            _ptr(row_to_route), _ptr(num_rows), _ptr(out), _ptr(out_scales), _ptr(out_weights), _stream(dev),
+        )
+    _lib.check(status, "layout_dispatch_small")
+    layout_out = dict(counts=counts, psum=psum, offsets=offsets, route_to_row=route_to_row, row_to_route=row_to_route,
+                      num_rows=num_rows, meta=meta)
+    return layout_out, out, out_scales, out_weights
+
+
 def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: Optional[int]):
     """Fused per-128 FP8 quantisation + expand-permute of BF16 x [T,H]; ``num_rows=None`` as in ``dispatch_copy``."""
     lib = _lib.load()

@@ -117,6 +117,22 @@ int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int3
                             const int32_t* row_to_route, int num_tokens, int num_topk, int num_rows,
                             int hidden, void* out, float* out_scales, float* out_weights, void* stream);
 
+/* Routing layout and payload dispatch of a small batch (at most 2048 routes: a decode step) in ONE launch.
+ * Replaces the low-latency dispatch (csrc/ops/low_latency.cpp:80-216 -> dispatch_low_latency, csrc/kernels/dispatch/
+ * low_latency.cpp:73), which likewise derives the rows inside the payload kernel instead of running notify first; for
+ * larger batches dpep_layout followed by dpep_dispatch_copy / dpep_dispatch_quant_fp8 produce the same results.
+ * Every workgroup works out the rows of its own token from the whole routing table (which fits its LDS), so nothing
+ * waits for a layout kernel.  Arguments as for dpep_layout plus dpep_dispatch_copy (quantize == 0: x of row_bytes
+ * bytes per token, optional scales and weights) or dpep_dispatch_quant_fp8 (quantize != 0: x BF16, row_bytes = 2H,
+ * H % 128 == 0, out FP8 + out_scales FP32 [.,H/128]).  out / out_scales / out_weights must hold T*K rows; the first R are
+ * written.  The per-expert counts and R also go to the workspace's host mailbox: dpep_layout_wait works as after
+ * dpep_layout. */
+int dpep_layout_dispatch_small(void* ws, const int64_t* topk_idx, const void* x, const float* scales,
+                               const float* topk_weights, int num_tokens, int num_topk, int num_experts, int expert_begin,
+                               int num_local, int row_bytes, int scale_cols, int quantize, int32_t* counts, int32_t* psum,
+                               int32_t* offsets, int32_t* route_to_row, int32_t* row_to_route, int32_t* num_rows, void* out,
+                               float* out_scales, float* out_weights, void* stream);
+
 /* Stand-alone per-128 quantiser (deep_ep/utils/math.py:45-61): x bf16 [T,H] -> fp8 [T,H], fp32 [T,H/128]. */
 int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float* out_scales, void* stream);
 

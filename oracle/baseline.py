@@ -59,3 +59,17 @@ def combine(y, route_to_row, row_weights=None):
             tmp = tmp * row_weights.index_select(0, safe)[:, None]
         acc = torch.where(valid[:, None], acc + tmp, acc)
     return acc.bfloat16()
+
+
+def megamoe_expert_forward(x, w1, w2):
+    """One expert of the W4A8 FFN the way the reference's CPU oracle evaluates it (experiments/megamoe/python/
+    deep_ep_experimental/megamoe/reference.py:84-89) on dense fp32 operands, with torch.matmul for the two
+    contractions: first = bf16(x @ w1^T); act = bf16(silu(gate) * up); qa = dequant(mx_quant(act));
+    out = bf16(qa @ w2^T).  x [m,H], w1 [2I,H] (gate rows then up rows), w2 [H,I]; returns BF16 [m,H].
+    The roundings, SwiGLU and the MXFP8 step are the NumPy oracle's."""
+    from . import megamoe
+
+    first = torch.matmul(x, w1.T).bfloat16().float()
+    act = megamoe.swiglu(first.numpy())
+    qa = torch.from_numpy(megamoe.mx_dequantize(*megamoe.mx_quantize(act)))
+    return torch.matmul(qa, w2.T).bfloat16()

@@ -65,6 +65,21 @@ class FakeNative:
         return (padded(out).view(x.dtype), padded(None if scales is None else scales[token]),
                 padded(None if w is None else w.reshape(-1)[route]))
 
+    SMALL_BATCH_ROUTES = 2048
+
+    def layout_dispatch_small(self, ws, topk_idx, x, scales, w, num_experts, expert_begin=0, num_local=None, quantize=False,
+                              capacity_rows=None):
+        """One launch for both in the library; here the two oracle steps in a row."""
+        self.calls["layout_dispatch_small"] += 1
+        plan = self.layout(ws, topk_idx, num_experts, expert_begin, num_local)
+        if self.fail_next:
+            raise RuntimeError(self.fail_next)
+        if quantize:
+            moved = self.dispatch_quant_fp8(x, w, plan["route_to_row"], plan["row_to_route"], None)
+        else:
+            moved = self.dispatch_copy(x, scales, w, plan["route_to_row"], plan["row_to_route"], None, capacity_rows=capacity_rows)
+        return (plan, *moved)
+
     def dispatch_quant_fp8(self, x, w, route_to_row, row_to_route, rows):
         self.calls["dispatch_quant_fp8"] += 1
         q, s = oquant.cast_to_fp8_torch(x)

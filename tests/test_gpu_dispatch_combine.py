@@ -409,3 +409,66 @@ def test_random_shapes_end_to_end(ops, ws):
         y = torch.randn(rows, hidden, generator=gen).bfloat16()
         combined, _ = ops.combine(y.cuda(), got["route_to_row"], torch.from_numpy(w_rows).cuda())
         np.testing.assert_array_equal(bf16_bits(combined), ocombine.combine(bf16_bits(y), want["route_to_row"], w_rows), err_msg=label)
+
+
+SMALL_SHAPES = [
+    # tokens, topk, experts, begin, local, hidden
+    (128, 8, 256, 0, 256, 7168),   # the decode shape
+    (128, 8, 256, 64, 32, 1024),   # a rank's share: most routes elsewhere
+    (1, 1, 4, 0, 4, 128),
+    (37, 6, 48, 8, 24, 384),
+    (64, 32, 1024, 0, 1024, 256),  # the largest top-k and expert count, 2048 routes
+    (256, 8, 16, 0, 16, 512),      # few experts: long runs per expert
+]
+
+
+@pytest.mark.parametrize("tokens,topk,experts,begin,local,hidden", SMALL_SHAPES)
+@pytest.mark.parametrize("mode", ["bf16", "fp8_copy", "fp8_quant", "fp16"])
+def test_layout_and_dispatch_in_one_launch(ops, ws, tokens, topk, experts, begin, local, hidden, mode):
+    """Small batches: layout and payload from one kernel, every workgroup working out its own token's rows.  All
+    layout outputs, the host mailbox and the dispatched payload / scales / weights against the oracle, bit for bit."""
+    rng = np.random.default_rng(tokens * 7 + topk + hidden)
+    idx_np = rng.integers(-1, experts + 1, size=(tokens, topk))  # includes -1 and == E, and repeated experts
+    idx = torch.from_numpy(idx_np).cuda()
+    x = torch.from_numpy(rng.normal(size=(tokens, hidden)).astype(np.float32)).bfloat16()
+    w = torch.from_numpy(rng.random((tokens, topk)).astype(np.float32))
+    want = olayout.layout(idx_np, experts, begin, local)
+    rows = want["num_rows"]
+    scales = None
+    if mode == "fp8_copy":
+        q, s = oquant.cast_to_fp8_torch(x) if hidden % 128 == 0 else (x.to(torch.float8_e4m3fn), torch.rand(tokens, 3))
+        payload, scales = q.cuda(), s.cuda()
+    elif mode == "fp16":
+        payload = x.to(torch.float16).cuda()
+    else:
+        payload = x.cuda()
+    if mode == "fp8_quant" and hidden % 128:
+        pytest.skip("the fused quantiser needs a width that is a multiple of 128")
+    lay, out, out_scales, out_w = ops.layout_dispatch_small(ws, idx, payload, scales, w.cuda(), experts, begin, local,
+                                                            quantize=mode == "fp8_quant")
+    counts, got_rows = ops.layout_wait(ws, local)
+    assert got_rows == rows == int(lay["num_rows"].item()) and counts == [int(c) for c in want["counts"]]
+    np.testing.assert_array_equal(i32(lay["counts"]), want["counts"])
+    np.testing.assert_array_equal(i32(lay["psum"]), want["psum"])
+    np.testing.assert_array_equal(i32(lay["offsets"]), want["offsets"])
+    np.testing.assert_array_equal(i32(lay["route_to_row"]), want["route_to_row"])
+    np.testing.assert_array_equal(i32(lay["row_to_route"])[:rows], want["row_to_route"])
+    assert out.shape[0] == tokens * topk
+    if mode == "fp8_quant":
+        q_ref, s_ref = oquant.cast_to_fp8_torch(x)
+        np.testing.assert_array_equal(fp8_bits(out[:rows]), olayout.expand_rows(q_ref.view(torch.uint8).numpy(), want["row_to_route"], topk))
+        np.testing.assert_array_equal(f32_bits(out_scales[:rows]), olayout.expand_rows(s_ref.numpy().view(np.uint32), want["row_to_route"], topk))
+    else:
+        source = payload.cpu().view(torch.uint8 if payload.element_size() == 1 else torch.int16).numpy()
+        got = out[:rows].cpu().view(torch.uint8 if payload.element_size() == 1 else torch.int16).numpy()
+        np.testing.assert_array_equal(got, olayout.expand_rows(source, want["row_to_route"], topk))
+        if scales is not None:
+            np.testing.assert_array_equal(f32_bits(out_scales[:rows]), olayout.expand_rows(f32_bits(scales), want["row_to_route"], topk))
+    np.testing.assert_array_equal(f32_bits(out_w[:rows]), olayout.expand_weights(w.numpy(), want["row_to_route"]).view(np.uint32))
+
+
+def test_layout_dispatch_small_limits(ops, ws):
+    idx = torch.zeros((300, 8), dtype=torch.int64, device="cuda")  # 2400 routes
+    x = torch.zeros((300, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="routes"):
+        ops.layout_dispatch_small(ws, idx, x, None, None, 16)

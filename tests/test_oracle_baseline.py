@@ -32,3 +32,18 @@ def test_baseline_equals_oracle():
         got = baseline.combine(y, r2row, weights)
         ref = ocombine.combine(_bits(y), want["route_to_row"], None if weights is None else weights.numpy())
         np.testing.assert_array_equal(_bits(got), ref)
+
+
+def test_megamoe_baseline_matches_numpy_oracle():
+    # the timed torch.matmul form against the NumPy oracle (different BLAS, same roundings): all but a few
+    # elements identical, those one BF16 / e4m3 step apart
+    from oracle import megamoe as mm
+
+    rng = np.random.default_rng(4)
+    x = mm.round_bf16(rng.normal(size=(12, 128)))
+    w1 = (rng.normal(size=(256, 128)) * 0.1).astype(np.float32)
+    w2 = (rng.normal(size=(128, 128)) * 0.1).astype(np.float32)
+    got = baseline.megamoe_expert_forward(torch.from_numpy(x), torch.from_numpy(w1), torch.from_numpy(w2)).float().numpy()
+    want = mm.expert_forward(x, w1, w2)
+    assert mm.relative_frobenius(got, want) < 5e-3
+    assert (got == want).mean() > 0.95
