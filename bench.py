@@ -66,18 +66,36 @@ class Timer:
         self.iters = max(1, iters)
         self.warmups = max(1, warmups)
         self.flush = None
+        self.cycles_per_us = None
+
+    def spin_cycles_per_us(self):
+        """How many `torch.cuda._sleep` cycles make one microsecond on this GPU (measured once)."""
+        if self.cycles_per_us is None:
+            torch = self.torch
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda._sleep(100_000)
+            start.record()
+            torch.cuda._sleep(2_000_000)
+            stop.record()
+            torch.cuda.synchronize()
+            self.cycles_per_us = 2_000_000 / (start.elapsed_time(stop) * 1000.0)
+        return self.cycles_per_us
 
     def back_to_back(self, fn, head_start=False):
-        """Average microseconds over `iters` launches queued without gaps.  head_start: the GPU is kept busy first
-        (a spin kernel of about 2 ms), so that the host queues launches meanwhile and a kernel shorter than its Python
-        launch path is still timed back to back."""
+        """Average microseconds over `iters` launches queued without gaps.  head_start: the GPU is kept busy first by a
+        spin kernel (no memory traffic that the timed kernels would have to wait out) for as long as the host needs to
+        queue all the launches, measured on the warm-up launches, so that a kernel shorter than its Python launch path
+        is still timed back to back."""
         torch = self.torch
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
         for _ in range(self.warmups):
             fn()
+        host_us = (time.perf_counter() - t0) * 1e6 / self.warmups
         torch.cuda.synchronize()
         if head_start and hasattr(torch.cuda, "_sleep"):
-            torch.cuda._sleep(4_000_000)  # cycles; no memory traffic that the timed kernels would have to wait out
+            torch.cuda._sleep(int(self.spin_cycles_per_us() * host_us * self.iters * 1.5) + 100_000)
         start.record()
         for _ in range(self.iters):
             fn()
@@ -307,45 +325,51 @@ def rank_share_kernels(torch, ops, cases, timer):
 
 
 def read_traffic(kernel):
-    """HBM bytes per launch of `kernel` from profiles/hbm_traffic.json (written by --ingest-pmc), or None."""
+    """HBM bytes per launch of `kernel` from profiles/hbm_traffic.json (written by --ingest-pmc), or None.  The file
+    keys its entries "<kernel> @<grid size>"; of several grids of one kernel the one that moved most is the
+    benchmark's own shape (the counter runs skip the smaller workloads)."""
     try:
         table = json.load(open(TRAFFIC_FILE))
     except (OSError, ValueError):
         return None
-    entry = table.get("kernels", {}).get(kernel)
-    return None if entry is None else entry.get("hbm_bytes")
+    found = [entry for name, entry in table.get("kernels", {}).items() if name.rsplit(" @", 1)[0] == kernel]
+    return max((entry["hbm_bytes"] for entry in found), default=None)
 
 
 def ingest_pmc(fetch_csv, write_csv):
-    """Two rocprofv3 --pmc runs of `bench.py --calibrate-copy` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch) ->
-    profiles/hbm_traffic.json.  Both counters are scaled by what they read for the calibration copy, whose traffic is
-    known: [32768,7168] BF16 rows through dispatch_copy_row_kernel = 458 752 KiB read and as much written."""
+    """Two rocprofv3 --pmc runs of `bench.py --calibrate-copy --no-extra-shapes` (FETCH_SIZE, then WRITE_SIZE; KiB per
+    dispatch) -> profiles/hbm_traffic.json.  Both counters are scaled by what they read for the calibration copy, whose
+    traffic is known: [32768,7168] BF16 rows through dispatch_copy_row_kernel = 458 752 KiB read and as much written."""
     import csv
     import re
 
     def averages(path, counter):
         sums, calls = {}, {}
         for row in csv.DictReader(open(path)):
-            if row.get("Counter_Name") != counter:
+            if row.get("Counter_Name") != counter or "dpep::" not in row["Kernel_Name"]:
                 continue
-            name = re.sub(r"\(.*", "", row["Kernel_Name"]).replace("void ", "").replace("dpep::(anonymous namespace)::", "").strip()
+            name = row["Kernel_Name"].replace("void ", "").replace("dpep::(anonymous namespace)::", "")
+            name = re.sub(r"\(.*", "", name).strip() + " @" + row["Grid_Size"]
             sums[name] = sums.get(name, 0.0) + float(row["Counter_Value"])
             calls[name] = calls.get(name, 0) + 1
-        return {name: sums[name] / calls[name] for name in sums}
+        return {name: sums[name] / calls[name] for name in sums}, calls
 
-    fetch, write = averages(fetch_csv, "FETCH_SIZE"), averages(write_csv, "WRITE_SIZE")
+    (fetch, calls), (write, _) = averages(fetch_csv, "FETCH_SIZE"), averages(write_csv, "WRITE_SIZE")
     known_kib = 32768 * 7168 * 2 / 1024
-    copy = "dispatch_copy_row_kernel"
-    if copy not in fetch or copy not in write:
-        raise SystemExit("the counter files hold no dispatch_copy_row_kernel: run bench.py with --calibrate-copy")
-    fetch_scale, write_scale = known_kib / fetch[copy], known_kib / write[copy]
+    copy = [name for name in fetch if name.startswith("dispatch_copy_row_kernel @") and name in write]
+    if len(copy) != 1:
+        raise SystemExit("the counter files must hold one shape of dispatch_copy_row_kernel: run bench.py with "
+                         "--calibrate-copy --no-extra-shapes")
+    fetch_scale, write_scale = known_kib / fetch[copy[0]], known_kib / write[copy[0]]
     kernels = {}
     for name in sorted(set(fetch) & set(write)):
         read_bytes, written = fetch[name] * fetch_scale * 1024, write[name] * write_scale * 1024
-        kernels[name] = dict(fetch_kib=fetch[name], write_kib=write[name], hbm_read_bytes=read_bytes, hbm_written_bytes=written,
-                             hbm_bytes=read_bytes + written)
-    table = dict(source="rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs) of `python3 bench.py --calibrate-copy ...`; "
-                 "KiB per dispatch, averaged over the dispatches of each kernel",
+        kernels[name] = dict(dispatches=calls[name], fetch_kib=fetch[name], write_kib=write[name], hbm_read_bytes=round(read_bytes),
+                             hbm_written_bytes=round(written), hbm_bytes=round(read_bytes + written))
+    table = dict(source="rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs) of `python3 bench.py --steps 5 --warmup 2 "
+                 "--kernel-iters 5 --kernel-warmup 2 --no-cpu-baseline --no-extra-shapes --calibrate-copy`; KiB per dispatch, "
+                 "averaged over the dispatches of each kernel and grid size (keys: '<kernel> @<grid size>'); most launches "
+                 "follow a 256 MiB cache flush, so inputs come from HBM",
                  fetch_scale=fetch_scale, write_scale=write_scale, calibration_kib=known_kib, kernels=kernels)
     json.dump(table, open(TRAFFIC_FILE, "w"), indent=1, sort_keys=True)
     print(f"wrote {TRAFFIC_FILE}: {len(kernels)} kernels, scale factors {fetch_scale:.3f} / {write_scale:.3f}")

@@ -60,8 +60,12 @@ struct Workspace {
 // told to stop, holds the number of the launch that wrote it last and needs no clearing.
 constexpr size_t kSyncBytes = 256;
 constexpr size_t kSyncFillStop = 64;
-constexpr int kMailboxTimeout = 2 + DPEP_MAX_LOCAL_EXPERTS;  // a layout kernel whose barrier wait ran out leaves its launch number here
-constexpr int kMailboxWords = 3 + DPEP_MAX_LOCAL_EXPERTS;
+// The host mailbox (pinned memory, 32-bit words): word 0 = number of rows and word 1 = sequence number of the layout
+// that reported last (one 8-byte store); word kMailboxTimeout = launch number of a layout kernel whose barrier wait
+// ran out; from word kMailboxCounts on, 16-byte aligned, the per-expert counts.
+constexpr int kMailboxTimeout = 2;
+constexpr int kMailboxCounts = 4;
+constexpr int kMailboxWords = kMailboxCounts + (DPEP_MAX_LOCAL_EXPERTS + 3) / 4 * 4;
 constexpr long long kLayoutBarrierTicks = 200000000;  // 2 s
 constexpr uint32_t kWorkspaceMagic = 0x44504550u;  // "DPEP"
 Workspace* as_workspace(void* ws);
@@ -111,5 +115,16 @@ __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cas
 // rows once.
 __device__ __forceinline__ void store16_nt(void* p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
 __device__ __forceinline__ u32x4 load16_nt(const void* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)); }
+
+// Counts of four consecutive local experts, first of them `first` (a multiple of 4), into the host mailbox as one
+// 16-byte store that goes through every cache (system scope).  One store per four experts instead of four: the
+// stores cross PCIe one by one, and a layout over 256 experts that sent a word at a time left the next launch
+// waiting behind them.  The caller waits with s_waitcnt vmcnt(0) before it publishes the sequence word.
+__device__ __forceinline__ void mailbox_store_counts(uint32_t* mailbox, int first, const int (&four)[4])
+{
+    const u32x4 v = {static_cast<uint32_t>(four[0]), static_cast<uint32_t>(four[1]), static_cast<uint32_t>(four[2]),
+                     static_cast<uint32_t>(four[3])};
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(mailbox + kMailboxCounts + first), "v"(v) : "memory");
+}
 
 }  // namespace dpep

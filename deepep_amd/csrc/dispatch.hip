@@ -245,7 +245,7 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_row_kernel(
 // row_to_route, workgroup 0 the per-expert outputs and the host mailbox.
 constexpr int kSmallRoutes = 2048;
 
-template <bool kQuant>
+template <bool kQuant, int kSlots>  // kSlots: compile-time bound of top-k (8 or DPEP_MAX_TOPK)
 __global__ __launch_bounds__(kMaxThreads) void layout_dispatch_small_kernel(
     const long long* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int num_topk,
     const u32x4* __restrict__ x, const float* __restrict__ scales, const float* __restrict__ weights, int units_per_row,
@@ -313,8 +313,6 @@ __global__ __launch_bounds__(kMaxThreads) void layout_dispatch_small_kernel(
                 counts[e] = mine[j];
                 psum[e] = offset + mine[j];
                 offsets[e + 1] = offset + mine[j];
-                if (mailbox != nullptr)
-                    __hip_atomic_store(mailbox + 2 + e, static_cast<uint32_t>(mine[j]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             }
         }
         offset += mine[j];
@@ -323,6 +321,7 @@ __global__ __launch_bounds__(kMaxThreads) void layout_dispatch_small_kernel(
         offsets[0] = 0;
         num_rows[0] = offset;  // the last thread's running offset is the total
     }
+    if (reporter && mailbox != nullptr && tid * 4 < num_local) mailbox_store_counts(mailbox, tid * 4, mine);
     if (reporter && mailbox != nullptr) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's counts have reached the host
     __syncthreads();
     if (reporter && mailbox != nullptr && tid == kMaxThreads - 1) {
@@ -331,22 +330,20 @@ __global__ __launch_bounds__(kMaxThreads) void layout_dispatch_small_kernel(
     }
     // earlier routes with the same expert, for each route of this token
     const int my_first = token * num_topk;
-    int want[DPEP_MAX_TOPK], seen[DPEP_MAX_TOPK];
+    int want[kSlots], seen[kSlots];
 #pragma unroll
-    for (int s = 0; s < DPEP_MAX_TOPK; ++s) {
-        want[s] = s < num_topk ? local_id[my_first + s] : -1;
+    for (int s = 0; s < kSlots; ++s) {
+        want[s] = s < num_topk ? local_id[my_first + s] : -2;  // -2 matches nothing
         seen[s] = 0;
     }
     for (int j = tid; j < my_first + num_topk; j += kMaxThreads) {
         const int e = local_id[j];
-        if (e < 0) continue;
 #pragma unroll
-        for (int s = 0; s < DPEP_MAX_TOPK; ++s)
-            if (s < num_topk && e == want[s] && j < my_first + s) ++seen[s];
+        for (int s = 0; s < kSlots; ++s) seen[s] += (e == want[s] && j < my_first + s) ? 1 : 0;
     }
 #pragma unroll
-    for (int s = 0; s < DPEP_MAX_TOPK; ++s)
-        if (seen[s] != 0) atomicAdd(&before[s], seen[s]);
+    for (int s = 0; s < kSlots; ++s)
+        if (seen[s] != 0 && want[s] >= 0) atomicAdd(&before[s], seen[s]);
     __syncthreads();
     if (tid < num_topk) {
         const int e = local_id[my_first + tid];
@@ -536,18 +533,20 @@ int dpep_layout_dispatch_small(void* ws, const int64_t* topk_idx, const void* x,
     const Split sp = choose_split(num_tokens, units, 8);
     const int n_routes = num_tokens * num_topk;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (quantize)
-        hipLaunchKernelGGL(layout_dispatch_small_kernel<true>, dim3(num_tokens * sp.parts), dim3(kMaxThreads), 0, s,
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(num_tokens * sp.parts), dim3(kMaxThreads), 0, s,
                            reinterpret_cast<const long long*>(topk_idx), n_routes, num_experts, expert_begin, num_local, num_topk,
-                           static_cast<const u32x4*>(x), nullptr, topk_weights, units, sp.per_part, sp.parts, 0, counts, psum, offsets,
-                           num_rows, route_to_row, row_to_route, static_cast<u32x4*>(out), out_scales, out_weights,
-                           w->mailbox_device, w->sequence);
-    else
-        hipLaunchKernelGGL(layout_dispatch_small_kernel<false>, dim3(num_tokens * sp.parts), dim3(kMaxThreads), 0, s,
-                           reinterpret_cast<const long long*>(topk_idx), n_routes, num_experts, expert_begin, num_local, num_topk,
-                           static_cast<const u32x4*>(x), scales, topk_weights, units, sp.per_part, sp.parts, scale_cols, counts, psum,
-                           offsets, num_rows, route_to_row, row_to_route, static_cast<u32x4*>(out), out_scales, out_weights,
-                           w->mailbox_device, w->sequence);
+                           static_cast<const u32x4*>(x), quantize ? nullptr : scales, topk_weights, units, sp.per_part, sp.parts,
+                           quantize ? 0 : scale_cols, counts, psum, offsets, num_rows, route_to_row, row_to_route,
+                           static_cast<u32x4*>(out), out_scales, out_weights, w->mailbox_device, w->sequence);
+    };
+    if (num_topk <= 8) {
+        if (quantize) launch(layout_dispatch_small_kernel<true, 8>);
+        else launch(layout_dispatch_small_kernel<false, 8>);
+    } else {
+        if (quantize) launch(layout_dispatch_small_kernel<true, DPEP_MAX_TOPK>);
+        else launch(layout_dispatch_small_kernel<false, DPEP_MAX_TOPK>);
+    }
     return launch_status("layout_dispatch_small");
 }
 

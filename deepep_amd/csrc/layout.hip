@@ -287,9 +287,6 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
             for (int w = 0; w < kWaves; ++w) lds.running[w][e] += offset;
             if (reporter) {
                 counts[e] = mine[j];
-                if (mailbox != nullptr)  // pinned host memory, written through every cache
-                    __hip_atomic_store(mailbox + 2 + e, static_cast<uint32_t>(mine[j]), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_SYSTEM);
                 psum[e] = offset + mine[j];
                 offsets[e + 1] = offset + mine[j];
             }
@@ -300,6 +297,7 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
         offsets[0] = 0;
         num_rows[0] = offset;
     }
+    if (reporter && mailbox != nullptr && tid * 4 < num_local) mailbox_store_counts(mailbox, tid * 4, mine);
     // The host polls the mailbox's sequence word: publish it (with the row count, one 8-byte store) after
     // every per-expert count of this workgroup has reached host memory.  The counts went out as write-through
     // stores, so each thread only has to wait until its own are acknowledged: no cache needs writing back, which

@@ -125,7 +125,7 @@ int dpep_layout_wait(void* ws, int32_t* counts_host, int num_local, int32_t* num
     }
     *num_rows_host = static_cast<int32_t>(box[0]);
     if (counts_host != nullptr)
-        for (int e = 0; e < num_local; ++e) counts_host[e] = static_cast<int32_t>(box[2 + e]);
+        for (int e = 0; e < num_local; ++e) counts_host[e] = static_cast<int32_t>(box[dpep::kMailboxCounts + e]);
     return DPEP_OK;
 }
 
