@@ -103,16 +103,21 @@ class Timer:
         torch.cuda.synchronize()
         return start.elapsed_time(stop) * 1000.0 / self.iters
 
-    def flushed(self, fn):
-        """Per-launch times with the caches flushed before every launch by a 256 MiB fill."""
+    def flushed(self, fn, read_sweep=False):
+        """Per-launch times with the caches flushed before every launch: by a 256 MiB fill (which leaves the caches full
+        of dirty lines that are written back while the timed kernel runs), or, read_sweep, by a read-only pass over
+        the same 256 MiB (which evicts as much and leaves nothing to write back)."""
         torch = self.torch
         if self.flush is None:
-            self.flush = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device="cuda")
+            self.flush = torch.zeros(FLUSH_BYTES, dtype=torch.uint8, device="cuda")
         pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(self.iters)]
         for _ in range(self.warmups):
             fn()
         for start, stop in pairs:
-            self.flush.zero_()
+            if read_sweep:
+                self.flush.view(torch.int64).sum()
+            else:
+                self.flush.zero_()
             start.record()
             fn()
             stop.record()
@@ -121,10 +126,13 @@ class Timer:
         pick = lambda q: times[min(len(times) - 1, int(q * len(times)))]
         return dict(mean=sum(times) / len(times), min=times[0], p50=pick(0.5), p95=pick(0.95))
 
-    def kernel(self, fn, nbytes, head_start=False, extra=None):
-        """One `kernels` entry: flushed statistics, the back-to-back figure, and GB/s of both against 8 TB/s."""
+    def kernel(self, fn, nbytes, head_start=False, extra=None, read_sweep=False):
+        """One `kernels` entry: flushed statistics, the back-to-back figure, and GB/s of both against 8 TB/s.
+        read_sweep: also the statistics after a read-only flush (`after_read_sweep_us`)."""
         warm = self.back_to_back(fn, head_start)
         cold = self.flushed(fn)
+        if read_sweep:
+            extra = dict(extra or {}, after_read_sweep_us=self.flushed(fn, read_sweep=True))
         entry = dict(
             bytes=nbytes,
             us=cold["mean"],
@@ -227,9 +235,9 @@ def megamoe_bench(torch, ops, timer, with_cpu):
     sets = []
     for _ in range(3):
         w1 = torch.randint(0, 256, (local, 2 * inter, hidden // 2), dtype=torch.uint8, device=dev)
-        s1 = torch.full((local, 2 * inter, ops.megamoe_prepared_scale_cols(hidden)), 119, dtype=torch.uint8, device=dev)
+        s1 = torch.full((local, 2 * inter, ops.megamoe_prepared_shape(2 * inter, hidden, True)[2]), 119, dtype=torch.uint8, device=dev)
         w2 = torch.randint(0, 256, (local, hidden, inter // 2), dtype=torch.uint8, device=dev)
-        s2 = torch.full((local, hidden, ops.megamoe_prepared_scale_cols(inter)), 119, dtype=torch.uint8, device=dev)
+        s2 = torch.full((local, hidden, ops.megamoe_prepared_shape(hidden, inter, False)[2]), 119, dtype=torch.uint8, device=dev)
         sets.append((w1, s1, w2, s2))
     ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local))
     y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
@@ -457,12 +465,12 @@ def main():
     bf16_dispatch_bytes = tokens * hidden * 2 + tokens * topk * 4 + rows * hidden * 2 + rows * 4
     copy_dispatch_bytes = tokens * (hidden + (hidden // 128) * 4) + tokens * topk * 4 + rows * (hidden + (hidden // 128) * 4 + 4)
     kernels = {
-        "layout": timer.kernel(lambda: ops.layout(ws, idxd, experts), nbytes["layout"], head_start=True),
-        "dispatch_fp8_quant": timer.kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), nbytes["dispatch"]),
-        "dispatch_fp8_copy": timer.kernel(lambda: ops.dispatch_copy(q_pre, s_pre, wd, r2row, r2route, rows), copy_dispatch_bytes),
-        "dispatch_bf16": timer.kernel(lambda: ops.dispatch_copy(xd, None, wd, r2row, r2route, rows), bf16_dispatch_bytes),
-        "combine": timer.kernel(lambda: ops.combine(grows, r2row, out=out_buf), nbytes["combine"]),
-        "combine_weighted": timer.kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), nbytes["combine"] + rows * 4),
+        "layout": timer.kernel(lambda: ops.layout(ws, idxd, experts), nbytes["layout"], head_start=True, read_sweep=True),
+        "dispatch_fp8_quant": timer.kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), nbytes["dispatch"], read_sweep=True),
+        "dispatch_fp8_copy": timer.kernel(lambda: ops.dispatch_copy(q_pre, s_pre, wd, r2row, r2route, rows), copy_dispatch_bytes, read_sweep=True),
+        "dispatch_bf16": timer.kernel(lambda: ops.dispatch_copy(xd, None, wd, r2row, r2route, rows), bf16_dispatch_bytes, read_sweep=True),
+        "combine": timer.kernel(lambda: ops.combine(grows, r2row, out=out_buf), nbytes["combine"], read_sweep=True),
+        "combine_weighted": timer.kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), nbytes["combine"] + rows * 4, read_sweep=True),
     }
 
     dominant = kernels["combine"]
@@ -490,7 +498,8 @@ def main():
             "bytes_per_step": moved,
             "kernel_timing": f"{args.kernel_warmup} warm-ups + {args.kernel_iters} launches per kernel and protocol; "
             "`us` / `GBps` / `frac_of_8TBps` are the cache-flushed mean (256 MiB fill before every launch), "
-            "`back_to_back_us` / `frac_back_to_back` the same launches queued without gaps",
+            "`back_to_back_us` / `frac_back_to_back` the same launches queued without gaps, `after_read_sweep_us` the "
+            "launches after a read-only pass over 256 MiB (caches evicted, no dirty lines left to write back)",
         },
         "roofline": {
             "kernel": "combine_kernel<0, false>",

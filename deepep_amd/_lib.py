@@ -37,7 +37,8 @@ SIGNATURES = {
     "dpep_mx_quant": (_I, (_P, _I, _I, _P, _P, _P)),
     "dpep_megamoe_schedule_check": (_I, (_I, _I, _I, _I)),
     "dpep_megamoe_workspace_bytes": (_Z, (_I, _I, _I, _I, _I, _I)),
-    "dpep_megamoe_prepared_scale_bytes": (_Z, (_I, _I, _I)),
+    "dpep_megamoe_padded_dim": (_I, (_I,)),
+    "dpep_megamoe_prepared_shape": (_I, (_I, _I, _I, ctypes.POINTER(_I), ctypes.POINTER(_I), ctypes.POINTER(_I))),
     "dpep_megamoe_prepare_weights": (_I, (_P, _P, _I, _I, _I, _I, _P, _P, _P)),
     "dpep_megamoe_forward": (_I, (_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
                                   _P, _P, _P)),

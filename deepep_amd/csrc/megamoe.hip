@@ -98,13 +98,23 @@ __device__ __forceinline__ int source_row(int physical_col, int n, int gate_up)
     return (tile & 1) * (n >> 1) + act_col;
 }
 
+// n, k: the raw matrix; np, kp: what the GEMM works on (padded_dim of each; for gate/up both halves are padded, so
+// np = 2 * padded_dim(n / 2)).  Padding columns and k blocks get zero codes (FP4 0.0) and the scale byte of 1.0.
 __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __restrict__ w,
-                                                              const uint8_t* __restrict__ s, int n, int k, int gate_up,
-                                                              uint8_t* __restrict__ w_out, uint8_t* __restrict__ s_out,
-                                                              long long packed_chunks, long long scale_pairs)
+                                                              const uint8_t* __restrict__ s, int n, int k, int np, int kp,
+                                                              int gate_up, uint8_t* __restrict__ w_out,
+                                                              uint8_t* __restrict__ s_out, long long packed_chunks,
+                                                              long long scale_pairs)
 {
     const long long id = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const int ktiles = k / 128;
+    const int ktiles = kp / 128;
+    // raw row of a physical (padded, interleaved) column, or -1 for a padding column
+    auto raw_row = [&](int physical_col) {
+        const int row = source_row(physical_col, np, gate_up);
+        if (!gate_up) return row < n ? row : -1;
+        const int half = np >> 1, in_half = row % half;
+        return in_half < (n >> 1) ? (row / half) * (n >> 1) + in_half : -1;
+    };
     if (id < packed_chunks) {
         // one 16-byte fragment; order [expert][block of 8 column tiles][k tile][column tile][k step][lane]: the
         // 16 KiB a workgroup copies per item are contiguous and its items follow each other in memory
@@ -112,34 +122,60 @@ __global__ __launch_bounds__(256) void prepare_weights_kernel(const uint8_t* __r
         long long rest = id >> 10;
         const int kt = rest % ktiles;
         rest /= ktiles;
-        const int nb = rest % (n / 256);
-        const long long e = rest / (n / 256);
+        const int nb = rest % (np / 256);
+        const long long e = rest / (np / 256);
         const int c = nb * 8 + (q >> 1), ks = kt * 2 + (q & 1);
-        const int row = source_row(c * 32 + (lane & 31), n, gate_up);
-        const uint8_t* src = w + (e * n + row) * (k / 2) + ks * 32 + (lane >> 5) * 16;
-        reinterpret_cast<u32x4*>(w_out)[id] = *reinterpret_cast<const u32x4*>(src);
+        const int row = raw_row(c * 32 + (lane & 31));
+        const int byte = ks * 32 + (lane >> 5) * 16;  // 16 bytes = 32 values of k, all inside the raw matrix or none
+        u32x4 fragment = {0u, 0u, 0u, 0u};
+        if (row >= 0 && byte * 2 < k) fragment = *reinterpret_cast<const u32x4*>(w + (e * n + row) * (k / 2) + byte);
+        reinterpret_cast<u32x4*>(w_out)[id] = fragment;
     }
     if (id < scale_pairs) {
         // Scales: per (expert, block of 8 column tiles, span of 4 k tiles) one 4 KiB block
         // [column tile 8][lane 64][k tile 4][2 bytes = k blocks (2*kb + g) of that k tile]; a span is what
-        // the GEMM copies in one go.  The last span is padded when k % 512 != 0.
+        // the GEMM copies in one go.  The last span is padded when kp % 512 != 0.
         const int spans = (ktiles + 3) / 4;
         const int kq = id & 3, lane = (id >> 2) & 63, c8 = (id >> 8) & 7;
         long long rest = id >> 11;
         const int span = rest % spans;
         rest /= spans;
-        const int nb = rest % (n / 256);
-        const long long e = rest / (n / 256);
+        const int nb = rest % (np / 256);
+        const long long e = rest / (np / 256);
         const int kt = span * 4 + kq;
         uint8_t lo = 127, hi = 127;
-        if (kt < ktiles) {
-            const int row = source_row((nb * 8 + c8) * 32 + (lane & 31), n, gate_up);
-            const uint8_t* src = s + (e * n + row) * (k / 32) + kt * 4 + (lane >> 5);
-            lo = src[0];
-            hi = src[2];
+        const int row = raw_row((nb * 8 + c8) * 32 + (lane & 31));
+        if (kt < ktiles && row >= 0) {
+            const int block = kt * 4 + (lane >> 5);  // k blocks of 32: this lane half's two of the k tile
+            const uint8_t* src = s + (e * n + row) * (k / 32);
+            if (block < k / 32) lo = src[block];
+            if (block + 2 < k / 32) hi = src[block + 2];
         }
         s_out[id * 2] = lo;
         s_out[id * 2 + 1] = hi;
+    }
+}
+
+// Rows [T, h] of e4m3 codes with [T, h/32] scale bytes -> [T, hp] and [T, hp/32]: zero codes and the scale byte of
+// 1.0 behind column h.  One thread per 16 output bytes (codes), then per scale byte.
+__global__ __launch_bounds__(256) void pad_activations_kernel(const uint8_t* __restrict__ codes,
+                                                              const uint8_t* __restrict__ scales, int h, int hp,
+                                                              uint8_t* __restrict__ codes_out,
+                                                              uint8_t* __restrict__ scales_out, long long code_units,
+                                                              long long scale_bytes)
+{
+    const long long id = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id < code_units) {
+        const long long row = id / (hp / 16);
+        const int unit = static_cast<int>(id % (hp / 16));
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (unit * 16 < h) v = *reinterpret_cast<const u32x4*>(codes + row * h + unit * 16);
+        reinterpret_cast<u32x4*>(codes_out)[id] = v;
+    }
+    if (id < scale_bytes) {
+        const long long row = id / (hp / 32);
+        const int block = static_cast<int>(id % (hp / 32));
+        scales_out[id] = block < h / 32 ? scales[row * (h / 32) + block] : static_cast<uint8_t>(127);
     }
 }
 
@@ -202,7 +238,8 @@ struct GemmParams {
     int n, k;
     uint8_t* act_codes;        // first GEMM: [rows, N/2] e4m3
     uint8_t* act_scales;       //             [rows, N/64] e8m0
-    uint16_t* out;             // second GEMM: [rows, N] bf16
+    uint16_t* out;             // second GEMM: [rows, out_cols] bf16
+    int out_cols;              //   columns that exist (<= N, a multiple of 8; the padding columns of N are not stored)
     // Zero rows of the final output.  When a launch has fewer tiles than workgroups, the workgroups left
     // without a tile stream zeros into the output rows of the tokens that no local expert serves (most tokens of a
     // rank's share), which the weighted reduce would otherwise have to write after the GEMMs: the stores cost the
@@ -634,10 +671,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 #pragma unroll
                     for (int it = 0; it < 2; ++it) {
                         const int r = it * 16 + (lane >> 2);
-                        if (r < tile_rows) {
+                        if (r < tile_rows && col < p.out_cols) {
                             const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
                             // cached store: the weighted reduce that follows reads these rows back at once
-                            *reinterpret_cast<u32x4*>(p.out + (out_row0 + r) * p.n + col) = chunk;
+                            *reinterpret_cast<u32x4*>(p.out + (out_row0 + r) * p.out_cols + col) = chunk;
                         }
                     }
                 }
@@ -757,6 +794,11 @@ __global__ __launch_bounds__(256) void shared_rows_kernel(const int* __restrict_
     if (id < static_cast<long long>(num_shared) * num_tokens)
         row_to_route[first + id] = static_cast<int>(id % num_tokens) * num_topk;
 }
+
+// What the GEMM works on for a logical dimension (hidden or intermediate): whole 256-column tiles and whole spans of
+// scales, at least 512 (a row's scale bytes fill one 16-byte copy).  Weights are padded when they are prepared,
+// activations by a copy of their own before the first GEMM; padding multiplies zero codes.
+int padded_dim(int dim) { return dim <= 512 ? 512 : (dim + 255) / 256 * 256; }
 
 int check_gemm(const char* what, int n, int k, int num_local)
 {
@@ -962,11 +1004,19 @@ int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktil
     return DPEP_OK;
 }
 
-size_t dpep_megamoe_prepared_scale_bytes(int num_local, int n, int k)
+int dpep_megamoe_padded_dim(int dim) { return dim < 1 ? 0 : dpep::padded_dim(dim); }
+
+int dpep_megamoe_prepared_shape(int n, int k, int gate_up, int* padded_n, int* padded_k, int* scale_cols)
 {
-    if (num_local < 1 || n < 1 || k < 1) return 0;
-    const size_t spans = (static_cast<size_t>(k) / 128 + 3) / 4;  // groups of four k tiles, the last one padded
-    return static_cast<size_t>(num_local) * n * spans * 16;
+    using namespace dpep;
+    DPEP_REQUIRE(padded_n && padded_k && scale_cols, "prepared_shape: NULL output");
+    DPEP_REQUIRE(k > 0 && k % 64 == 0, "prepared_shape: K=%d must be a positive multiple of 64", k);
+    DPEP_REQUIRE(n > 0 && n % (gate_up ? 256 : 64) == 0, "prepared_shape: N=%d must be a positive multiple of %d", n,
+                 gate_up ? 256 : 64);
+    *padded_n = gate_up ? 2 * padded_dim(n / 2) : padded_dim(n);
+    *padded_k = padded_dim(k);
+    *scale_cols = (*padded_k / 128 + 3) / 4 * 16;  // groups of four k tiles, the last one padded
+    return DPEP_OK;
 }
 
 int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scales, int num_local, int n, int k,
@@ -974,22 +1024,23 @@ int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scale
 {
     using namespace dpep;
     DPEP_REQUIRE(num_local >= 1, "prepare_weights: bad expert count %d", num_local);
-    DPEP_REQUIRE(k > 0 && k % 256 == 0, "prepare_weights: K=%d must be a positive multiple of 256", k);
-    DPEP_REQUIRE(n > 0 && n % kBN == 0, "prepare_weights: N=%d must be a positive multiple of %d", n, kBN);
+    int np = 0, kp = 0, scale_cols = 0;
+    if (int rc = dpep_megamoe_prepared_shape(n, k, gate_up, &np, &kp, &scale_cols)) return rc;
     DPEP_REQUIRE(w_packed && w_scales && out_packed && out_scales && aligned16(w_packed) && aligned16(out_packed),
                  "prepare_weights: NULL or misaligned buffer");
     DPEP_REQUIRE(w_packed != out_packed && w_scales != out_scales, "prepare_weights: cannot run in place");
-    const long long chunks = static_cast<long long>(num_local) * n * (k / 2) / 16;
-    const long long pairs = static_cast<long long>(dpep_megamoe_prepared_scale_bytes(num_local, n, k) / 2);
-    const unsigned blocks = static_cast<unsigned>((chunks + 255) / 256);
+    const long long chunks = static_cast<long long>(num_local) * np * (kp / 2) / 16;
+    const long long pairs = static_cast<long long>(num_local) * np * scale_cols / 2;
+    const long long threads = chunks > pairs ? chunks : pairs;
+    const unsigned blocks = static_cast<unsigned>((threads + 255) / 256);
     hipLaunchKernelGGL(prepare_weights_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), w_packed,
-                       w_scales, n, k, gate_up, out_packed, out_scales, chunks, pairs);
+                       w_scales, n, k, np, kp, gate_up, out_packed, out_scales, chunks, pairs);
     return launch_status("prepare_weights");
 }
 
 // Workspace carve-up shared by workspace_bytes and forward.
 struct MegaLayout {
-    size_t hist, meta, fill_state, route_to_row, row_to_route, act_codes, act_scales, out2, total;
+    size_t hist, meta, fill_state, route_to_row, row_to_route, x_codes, x_scales, act_codes, act_scales, out2, total;
 };
 
 static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int intermediate, int num_local, int num_shared)
@@ -1005,8 +1056,12 @@ static MegaLayout mega_layout(int num_tokens, int num_topk, int hidden, int inte
     l.fill_state = at;   at += up((1 + 4096) * 4);  // fillers of the first GEMM: count + progress of each (<= 1024 CUs x 4 waves)
     l.route_to_row = at; at += up(routes * 4);
     l.row_to_route = at; at += up((routes + shared_rows) * 4);
-    l.act_codes = at;    at += up(max_rows * intermediate);
-    l.act_scales = at;   at += up(max_rows * (intermediate / 32));
+    const size_t hp = dpep::padded_dim(hidden), ip = dpep::padded_dim(intermediate);
+    // padded copy of the input rows, only when hidden is not already what the GEMM works on
+    l.x_codes = at;      at += hp != static_cast<size_t>(hidden) ? up(static_cast<size_t>(num_tokens) * hp) : 0;
+    l.x_scales = at;     at += hp != static_cast<size_t>(hidden) ? up(static_cast<size_t>(num_tokens) * (hp / 32)) : 0;
+    l.act_codes = at;    at += up(max_rows * ip);
+    l.act_scales = at;   at += up(max_rows * (ip / 32));
     l.out2 = at;         at += up(max_rows * hidden * 2);
     l.total = at;
     return l;
@@ -1031,9 +1086,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     DPEP_REQUIRE(w != nullptr, "megamoe_forward: not a live workspace");
     DPEP_REQUIRE(num_tokens >= 1 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "megamoe_forward: bad B=%d K=%d",
                  num_tokens, num_topk);
-    DPEP_REQUIRE(hidden % 256 == 0 && intermediate % 256 == 0 && hidden >= 512 && intermediate >= 512,
-                 "megamoe_forward: hidden=%d and intermediate=%d must be multiples of 256, at least 512", hidden,
+    DPEP_REQUIRE(hidden >= 64 && hidden % 64 == 0 && intermediate >= 128 && intermediate % 128 == 0,
+                 "megamoe_forward: hidden=%d must be a positive multiple of 64, intermediate=%d of 128", hidden,
                  intermediate);
+    const int hp = padded_dim(hidden), ip = padded_dim(intermediate);
     DPEP_REQUIRE(num_local >= 1 && num_local <= kMaxMoeExperts && expert_begin >= 0 &&
                      expert_begin + num_local <= num_experts,
                  "megamoe_forward: bad expert range E=%d begin=%d L=%d (at most %d local experts)", num_experts,
@@ -1051,7 +1107,7 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
                  "megamoe_forward: misaligned buffer");
     // the GEMM's copies address activation rows with 32-bit byte offsets
     const long long max_rows = static_cast<long long>(num_tokens) * ((num_topk < num_local ? num_topk : num_local) + num_shared);
-    DPEP_REQUIRE(static_cast<long long>(num_tokens) * hidden < (1LL << 32) && max_rows * intermediate < (1LL << 32),
+    DPEP_REQUIRE(static_cast<long long>(num_tokens) * hp < (1LL << 32) && max_rows * ip < (1LL << 32),
                  "megamoe_forward: activation tensors of B=%d tokens exceed 4 GiB", num_tokens);
     const MegaLayout l = mega_layout(num_tokens, num_topk, hidden, intermediate, num_local, num_shared);
     DPEP_REQUIRE(l.total <= w->bytes, "megamoe_forward: workspace too small (%zu needed, %zu available)", l.total, w->bytes);
@@ -1075,6 +1131,15 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     GemmParams g1{};
     g1.a_codes = static_cast<const uint8_t*>(x_codes);
     g1.a_scales = x_scales;
+    if (hp != hidden) {
+        const long long units = static_cast<long long>(num_tokens) * (hp / 16), bytes = static_cast<long long>(num_tokens) * (hp / 32);
+        hipLaunchKernelGGL(pad_activations_kernel, dim3(static_cast<unsigned>((units + 255) / 256)), dim3(256), 0, s,
+                           static_cast<const uint8_t*>(x_codes), x_scales, hidden, hp, base + l.x_codes, base + l.x_scales, units,
+                           bytes);
+        if (int rc = launch_status("pad_activations")) return rc;
+        g1.a_codes = base + l.x_codes;
+        g1.a_scales = base + l.x_scales;
+    }
     g1.row_to_route = row_to_route;
     g1.topk = num_topk;
     g1.offsets = offsets;
@@ -1084,8 +1149,8 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g1.ws = s1;
     g1.w_shared = shared_w1;
     g1.ws_shared = shared_s1;
-    g1.n = 2 * intermediate;
-    g1.k = hidden;
+    g1.n = 2 * ip;
+    g1.k = hp;
     g1.act_codes = base + l.act_codes;
     g1.act_scales = base + l.act_scales;
     // Expected rows (the true counts stay on the device): tokens * topk / experts per routed expert, every
@@ -1123,9 +1188,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g2.ws = s2;
     g2.w_shared = shared_w2;
     g2.ws_shared = shared_s2;
-    g2.n = hidden;
-    g2.k = intermediate;
+    g2.n = hp;
+    g2.k = ip;
     g2.out = reinterpret_cast<uint16_t*>(base + l.out2);
+    g2.out_cols = hidden;
     g2.forced_rt = g1.forced_rt;
     if (int rc = launch_gemm2(g2, per_expert, s)) return rc;
     return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,

@@ -8,8 +8,9 @@ transform_weights_for_mega_moe :311-379, mega_moe :382-413, fp8_fp4_mega_moe :52
     ``num_experts / world_size`` experts and its inputs hold the flattened tokens of all source ranks
     (capacity ``world_size * num_max_tokens_per_rank`` rows).  The reference needs 2..128 real ranks;
   * prepared weights are this library's fragment order (``dpep_megamoe_prepare_weights``), not Ascend NZ;
-  * FP8xFP8 weights are not built; hidden and intermediate_hidden must be multiples of 256 with
-    intermediate_hidden >= 512 (the reference: multiples of 64 and 128, from 256);
+  * FP8xFP8 weights are not built.  hidden (multiples of 64) and intermediate_hidden (multiples of 128, from 256)
+    have the reference's limits; sizes that are not multiples of 256, and 256 itself, run padded to the next
+    one (at least 512): the weights when they are prepared, the input rows by a copy inside the forward;
   * shared experts run as extra experts that take every token (weight 1, added after the routed ones).
 """
 
@@ -57,9 +58,10 @@ def _pair(value, name):
 class _PreparedPair(tuple):
     """(weights, scales) in the kernel's streaming order; immutable after preparation."""
 
-    def __new__(cls, weight, scale, gate_up):
+    def __new__(cls, weight, scale, gate_up, logical):
         value = super().__new__(cls, (weight, scale))
         value.gate_up = gate_up
+        value.logical = tuple(logical)  # (experts, N, K) of the raw tensor; the prepared one may be padded
         value._versions = (weight._version, scale._version)
         return value
 
@@ -96,12 +98,12 @@ class SymmBuffer:
         _integer("num_max_tokens_per_rank", num_max_tokens_per_rank, 1, 65536)
         _integer("num_topk", num_topk, 1, min(32, num_experts))
         _integer("hidden", hidden, 1024, 8192)
-        _integer("intermediate_hidden", intermediate_hidden, 512, 4096)
+        _integer("intermediate_hidden", intermediate_hidden, 256, 4096)
         _integer("num_shared_experts", num_shared_experts, 0, 8)
         _integer("ranks_per_node", ranks_per_node, 0, size)
         _integer("timeout", timeout, 1, 300)
-        if hidden % 256 or intermediate_hidden % 256:
-            raise ValueError("hidden and intermediate_hidden must be divisible by 256 in this build")
+        if hidden % 64 or intermediate_hidden % 128:
+            raise ValueError("hidden must be divisible by 64; intermediate_hidden by 128")
         if activation != "swiglu" or mma_type not in {"fp8xfp4", "fp8xfp8"}:
             raise ValueError("Only SwiGLU with FP8xFP4/FP8xFP8 is implemented; no BF16xBF16")
         if mma_type != "fp8xfp4":
@@ -253,7 +255,7 @@ def transform_weights_for_mega_moe(l1_weights, l2_weights, activation: str = "sw
             out_w, out_s = ops.megamoe_prepare_weights(
                 weight.contiguous(), scale.contiguous().reshape(*weight.shape[:2], k // 32), gate_up
             )
-        prepared.append(_PreparedPair(out_w, out_s, gate_up))
+        prepared.append(_PreparedPair(out_w, out_s, gate_up, (weight.shape[0], weight.shape[1], k)))
     return tuple(prepared)
 
 
@@ -297,7 +299,9 @@ def _run(x, topk_idx, topk_weights, l1_weights, l2_weights, sym_buffer, *, share
     if data.device != b._device:
         raise ValueError("x must be on the buffer's creating device")
     bs = data.shape[0]
-    if tuple(w1.shape[:2]) != (b.num_local_experts, b.intermediate_hidden * 2) or tuple(topk_idx.shape) != (bs, b.num_topk):
+    if (l1_weights.logical != (b.num_local_experts, b.intermediate_hidden * 2, b.hidden)
+            or l2_weights.logical != (b.num_local_experts, b.hidden, b.intermediate_hidden)
+            or tuple(topk_idx.shape) != (bs, b.num_topk)):
         raise ValueError("Weight/routing shapes do not match the buffer configuration")
     if topk_idx.dtype != torch.int32:
         raise TypeError("topk_idx must be int32; convert explicitly before timing")
@@ -340,7 +344,7 @@ def _run(x, topk_idx, topk_weights, l1_weights, l2_weights, sym_buffer, *, share
             ops.megamoe_forward(
                 b._workspace, data.contiguous(), scales.contiguous(), topk_idx.contiguous(), topk_weights.contiguous(),
                 w1, s1, w2, s2, b.num_experts, b.group.rank() * b.num_local_experts, b.num_local_experts, y, counts,
-                shared=shared,
+                shared=shared, intermediate=b.intermediate_hidden,
             )
             if cumulative_stats is not None:
                 cumulative_stats.add_(counts)

@@ -370,15 +370,26 @@ def megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_loca
     return int(_lib.load().dpep_megamoe_workspace_bytes(num_tokens, num_topk, hidden, intermediate, num_local, num_shared))
 
 
-def megamoe_prepared_scale_cols(k: int) -> int:
-    """Bytes per output column of a prepared scale tensor: spans of k = 512 (16 bytes each), the last one padded."""
-    return (k // 128 + 3) // 4 * 16
+def megamoe_padded_dim(dim: int) -> int:
+    """What the grouped GEMM works on for a logical hidden / intermediate size (whole 256-column tiles, at least 512)."""
+    return int(_lib.load().dpep_megamoe_padded_dim(int(dim)))
+
+
+def megamoe_prepared_shape(n: int, k: int, gate_up: bool):
+    """(padded N, padded K, scale bytes per column) of the prepared form of a raw [L,N,K/2] weight tensor."""
+    import ctypes
+
+    out = [ctypes.c_int(0) for _ in range(3)]
+    status = _lib.load().dpep_megamoe_prepared_shape(int(n), int(k), int(bool(gate_up)), *(ctypes.byref(v) for v in out))
+    _lib.check(status, "megamoe_prepared_shape")
+    return tuple(v.value for v in out)
 
 
 def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
-    """Raw packed FP4 uint8 [L,N,K/2] + e8m0 uint8 [L,N,K/32] -> the kernel's streaming order.
+    """Raw packed FP4 uint8 [L,N,K/2] + e8m0 uint8 [L,N,K/32] -> the kernel's streaming order, padded to the sizes the
+    GEMM works on (``megamoe_prepared_shape``: zero codes and unit scales behind N and K).
 
-    Returns (packed [L,N,K/2], scales [L,N,megamoe_prepared_scale_cols(K)])."""
+    Returns (packed [L,Np,Kp/2], scales [L,Np,scale_cols])."""
     lib = _lib.load()
     _require("w_packed", w_packed, torch.uint8)
     if w_packed.ndim != 3:
@@ -386,10 +397,9 @@ def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
     experts, n, half_k = w_packed.shape
     k = half_k * 2
     _require("w_scales", w_scales.reshape(experts, n, -1), torch.uint8, (experts, n, k // 32), w_packed.device)
-    out_w = torch.empty_like(w_packed)
-    out_s = torch.empty((experts, n, megamoe_prepared_scale_cols(k)), dtype=torch.uint8, device=w_packed.device)
-    if out_s.numel() != lib.dpep_megamoe_prepared_scale_bytes(experts, n, k):
-        raise RuntimeError("prepared scale size disagrees with the library")
+    np_, kp, scale_cols = megamoe_prepared_shape(n, k, gate_up)
+    out_w = torch.empty((experts, np_, kp // 2), dtype=torch.uint8, device=w_packed.device)
+    out_s = torch.empty((experts, np_, scale_cols), dtype=torch.uint8, device=w_packed.device)
     with _on_device(w_packed.device):
         status = lib.dpep_megamoe_prepare_weights(
             _ptr(w_packed), _ptr(w_scales), experts, n, k, int(bool(gate_up)), _ptr(out_w), _ptr(out_s),
@@ -400,10 +410,12 @@ def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
 
 
 def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s2, num_experts, expert_begin,
-                    num_local, y, expert_token_nums, shared=None):
+                    num_local, y, expert_token_nums, shared=None, intermediate=None):
     """Fused W4A8 forward of one rank's local experts; writes y [B,H] BF16 and expert_token_nums [L] int32.
 
-    ``shared`` = (w1, s1, w2, s2) prepared weights of S shared experts, which every token passes through."""
+    ``intermediate`` = the experts' logical intermediate size; by default what the prepared ``w1`` holds (right unless
+    the weights were padded).  ``shared`` = (w1, s1, w2, s2) prepared weights of S shared experts, which every token
+    passes through."""
     lib = _lib.load()
     dev = ws.device
     _require("x_codes", x_codes, torch.float8_e4m3fn, device=dev)
@@ -414,12 +426,18 @@ def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s
     _require("topk_idx", topk_idx, torch.int32, (tokens, topk), dev)
     _require("topk_weights", topk_weights, torch.float32, (tokens, topk), dev)
     _require("w1", w1, torch.uint8, device=dev)
-    if w1.ndim != 3 or w1.shape[0] != num_local or w1.shape[2] * 2 != hidden or w1.shape[1] % 2:
+    if w1.ndim != 3 or w1.shape[0] != num_local or w1.shape[1] % 2:
         raise ValueError("w1 must be prepared [L, 2I, H/2]")
-    intermediate = w1.shape[1] // 2
-    _require("s1", s1, torch.uint8, (num_local, 2 * intermediate, megamoe_prepared_scale_cols(hidden)), dev)
-    _require("w2", w2, torch.uint8, (num_local, hidden, intermediate // 2), dev)
-    _require("s2", s2, torch.uint8, (num_local, hidden, megamoe_prepared_scale_cols(intermediate)), dev)
+    if intermediate is None:
+        intermediate = w1.shape[1] // 2
+    if hidden % 64 or intermediate % 128 or hidden < 64 or intermediate < 128:
+        raise ValueError("hidden must be a positive multiple of 64, intermediate of 128")
+    n1, k1, cols1 = megamoe_prepared_shape(2 * intermediate, hidden, True)
+    n2, k2, cols2 = megamoe_prepared_shape(hidden, intermediate, False)
+    _require("w1", w1, torch.uint8, (num_local, n1, k1 // 2), dev)
+    _require("s1", s1, torch.uint8, (num_local, n1, cols1), dev)
+    _require("w2", w2, torch.uint8, (num_local, n2, k2 // 2), dev)
+    _require("s2", s2, torch.uint8, (num_local, n2, cols2), dev)
     _require("y", y, torch.bfloat16, (tokens, hidden), dev)
     _require("expert_token_nums", expert_token_nums, torch.int32, (num_local,), dev)
     num_shared = 0
@@ -428,10 +446,10 @@ def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s
         sw1, ss1, sw2, ss2 = shared
         _require("shared w1", sw1, torch.uint8, device=dev)
         num_shared = sw1.shape[0]
-        _require("shared w1", sw1, torch.uint8, (num_shared, 2 * intermediate, hidden // 2), dev)
-        _require("shared s1", ss1, torch.uint8, (num_shared, 2 * intermediate, megamoe_prepared_scale_cols(hidden)), dev)
-        _require("shared w2", sw2, torch.uint8, (num_shared, hidden, intermediate // 2), dev)
-        _require("shared s2", ss2, torch.uint8, (num_shared, hidden, megamoe_prepared_scale_cols(intermediate)), dev)
+        _require("shared w1", sw1, torch.uint8, (num_shared, n1, k1 // 2), dev)
+        _require("shared s1", ss1, torch.uint8, (num_shared, n1, cols1), dev)
+        _require("shared w2", sw2, torch.uint8, (num_shared, n2, k2 // 2), dev)
+        _require("shared s2", ss2, torch.uint8, (num_shared, n2, cols2), dev)
     with _on_device(dev):
         status = lib.dpep_megamoe_forward(
             ws.handle, _ptr(x_codes), _ptr(x_scales), _ptr(topk_idx), _ptr(topk_weights), _ptr(w1), _ptr(s1), _ptr(w2),

@@ -174,17 +174,23 @@ int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktil
 size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, int intermediate, int num_local,
                                     int num_shared);
 
-/* Bytes of the prepared scale buffer of one weight tensor: the scales are stored in spans of four k tiles
- * (k = 512), the last span padded, so this equals L*N*K/32 when K % 512 == 0 and is larger otherwise.
+/* What the grouped GEMM works on for a logical hidden or intermediate size: whole 256-column tiles and whole spans of
+ * scales, at least 512 (dim <= 512 -> 512, else the next multiple of 256).  Prepared weights are padded to it when
+ * they are prepared (zero codes, scale 1.0), input rows by a copy inside the forward; 0 for dim < 1.
+ * (The reference accepts hidden % 64 == 0 and intermediate_hidden % 128 == 0, api.py:93-105.) */
+int dpep_megamoe_padded_dim(int dim);
+
+/* Shape of the prepared form of one raw weight tensor [L,N,K/2] + [L,N,K/32]: packed [L,padded_n,padded_k/2] and scales
+ * [L,padded_n,scale_cols] (the scales are stored in spans of four k tiles = k 512, the last span padded).
+ * N % 64 == 0 (gate_up: N = 2I with I % 128 == 0, both halves padded separately), K % 64 == 0.
  * (Part of the transform_weights_for_mega_moe contract below.) */
-size_t dpep_megamoe_prepared_scale_bytes(int num_local, int n, int k);
+int dpep_megamoe_prepared_shape(int n, int k, int gate_up, int* padded_n, int* padded_k, int* scale_cols);
 
 /* One-off weight re-layout (transform_weights_for_mega_moe, experiments/megamoe/python/.../api.py:311-379):
- * raw packed FP4 [L,N,K/2] + e8m0 [L,N,K/32]  ->  the tile order the GEMM kernel streams
- * (N % 256 == 0, K % 256 == 0).  Byte shuffle only; out_packed has the size of w_packed, out_scales has
- * dpep_megamoe_prepared_scale_bytes(L, N, K) bytes.  gate_up != 0 (first GEMM, N = 2I,
- * gate rows then up rows) interleaves gate and up in groups of 32 output columns so SwiGLU is lane-local
- * (the counterpart of _interleave_gate_up_128, api.py:285-293). */
+ * raw packed FP4 [L,N,K/2] + e8m0 [L,N,K/32]  ->  the tile order the GEMM kernel streams, padded as
+ * dpep_megamoe_prepared_shape says (out_packed and out_scales have those sizes).  Byte shuffle only.
+ * gate_up != 0 (first GEMM, N = 2I, gate rows then up rows) interleaves gate and up in groups of 32 output columns so
+ * SwiGLU is lane-local (the counterpart of _interleave_gate_up_128, api.py:285-293). */
 int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scales, int num_local, int n,
                                  int k, int gate_up, uint8_t* out_packed, uint8_t* out_scales, void* stream);
 
@@ -193,8 +199,9 @@ int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scale
  * layout -> gather rows -> GMM1 (MXFP8 x MXFP4) -> bf16 -> SwiGLU -> MXFP8 requant -> GMM2 -> bf16 ->
  * route-weighted fp32 reduce per token -> bf16.
  *   x_codes e4m3 [B,H], x_scales e8m0 [B,H/32], topk_idx int32 [B,K] (distinct, in [0,E)), topk_weights fp32 [B,K]
- *   w1/s1: prepared GMM1 weights [L,2I,H/2] and scales; w2/s2: prepared GMM2 weights [L,H,I/2] and scales
- *   (scale sizes: dpep_megamoe_prepared_scale_bytes)
+ *   H % 64 == 0, I % 128 == 0 (hidden / intermediate as the caller sees them)
+ *   w1/s1: prepared GMM1 weights of the raw [L,2I,H/2] and scales; w2/s2: prepared GMM2 weights of the raw [L,H,I/2]
+ *   and scales (sizes: dpep_megamoe_prepared_shape)
  *   shared_w1/s1/w2/s2: the same for num_shared shared experts ([S,2I,H/2] ...; sw1/sw2/ss1/ss2 of
  *   mega_moe_kernel_do), NULL when num_shared == 0.  A shared expert processes every token and its output is
  *   added with weight 1 after the routed experts' (golden.py:160-164).

@@ -28,8 +28,17 @@ def test_null_workspace_and_ranges(lib):
     assert lib.dpep_layout_workspace_bytes(-1, 2, 8) == 0
     assert lib.dpep_megamoe_workspace_bytes(0, 2, 512, 512, 4, 0) == 0
     assert lib.dpep_megamoe_workspace_bytes(16, 2, 512, 512, 4, -1) == 0
-    assert lib.dpep_megamoe_prepared_scale_bytes(2, 256, 768) == 2 * 256 * 2 * 16  # two spans of k = 512, the last padded
-    assert lib.dpep_megamoe_prepared_scale_bytes(2, 256, 1024) == 2 * 256 * 1024 // 32
+    assert [lib.dpep_megamoe_padded_dim(d) for d in (0, 64, 256, 512, 576, 768, 1088, 7168)] == [0, 512, 512, 512, 768, 768, 1280, 7168]
+    shape = [ctypes.c_int() for _ in range(3)]
+    refs = [ctypes.byref(v) for v in shape]
+    assert lib.dpep_megamoe_prepared_shape(256, 768, 0, *refs) == 0
+    assert [v.value for v in shape] == [512, 768, 32]  # two spans of k = 512, the last padded
+    assert lib.dpep_megamoe_prepared_shape(2 * 384, 1088, 1, *refs) == 0
+    assert [v.value for v in shape] == [1024, 1280, 48]  # gate and up halves padded to 512 each
+    assert lib.dpep_megamoe_prepared_shape(4096, 7168, 1, *refs) == 0 and [v.value for v in shape] == [4096, 7168, 224]
+    assert lib.dpep_megamoe_prepared_shape(100, 512, 0, *refs) == -1 and "N=100" in _message(lib)
+    assert lib.dpep_megamoe_prepared_shape(384, 512, 1, *refs) == -1 and "N=384" in _message(lib)  # I = 192
+    assert lib.dpep_megamoe_prepared_shape(256, 96, 0, *refs) == -1 and "K=96" in _message(lib)
 
 
 def test_payload_entry_points_check_arguments_first(lib):

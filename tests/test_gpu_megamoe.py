@@ -76,6 +76,7 @@ def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, ti
     ops.megamoe_forward(
         ws, torch.from_numpy(x_codes).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(x_scales).to(dev),
         torch.from_numpy(idx).to(dev), torch.from_numpy(weights).to(dev), w1, s1, w2, s2, experts, begin, local, y, counts,
+        intermediate=inter,
     )
     torch.cuda.synchronize()
     out = y.float().cpu().numpy(), counts.cpu().numpy()
@@ -92,6 +93,10 @@ def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, ti
         (96, 512, 768, 8, 6, 2, 1),      # some local experts may be empty
         (200, 768, 1280, 4, 0, 4, 3),    # K of both GEMMs not a multiple of 512 (padded last scale span)
         (128, 512, 512, 64, 16, 32, 2),  # many local experts, most with a handful of rows, some empty
+        (150, 1088, 384, 8, 0, 8, 2),    # hidden % 64, intermediate % 128 (the reference's granularity): padded to 1280 / 512
+        (96, 1024, 256, 4, 0, 4, 2),     # the reference's smallest intermediate size
+        (70, 576, 640, 4, 1, 2, 3),      # both padded, partial local range
+        (40, 64, 128, 2, 0, 2, 1),       # the smallest sizes the entry point takes
     ],
 )
 def test_megamoe_forward_matches_oracle(ops, tokens, hidden, inter, experts, begin, local, topk):
@@ -104,6 +109,33 @@ def test_megamoe_forward_matches_oracle(ops, tokens, hidden, inter, experts, beg
     assert err <= 2e-2, err
     untouched = ~((idx >= begin) & (idx < begin + local)).any(axis=1)
     assert not got[untouched].any()  # tokens without a local expert receive zeros
+
+
+@pytest.mark.parametrize("gate_up", [False, True])
+@pytest.mark.parametrize("n,k", [(320, 576), (256, 64), (1024, 1088), (512, 384)])
+def test_prepare_weights_pads_like_explicit_padding(ops, n, k, gate_up):
+    """The prepared form of a raw tensor whose sizes are not what the GEMM works on equals, byte for byte, the prepared
+    form of the same tensor padded by hand (zero codes, scale byte 127 = 1.0; gate and up halves padded separately)."""
+    if gate_up and n % 256:
+        pytest.skip("gate/up needs N = 2I with I % 128 == 0")
+    rng = np.random.default_rng(n + k)
+    experts = 2
+    packed = rng.integers(0, 256, (experts, n, k // 2), dtype=np.uint8)
+    scales = rng.integers(100, 140, (experts, n, k // 32), dtype=np.uint8)
+    np_, kp, _ = ops.megamoe_prepared_shape(n, k, gate_up)
+    assert kp == ops.megamoe_padded_dim(k) and kp % 256 == 0 and kp >= max(k, 512)
+    halves = 2 if gate_up else 1
+    big_packed = np.zeros((experts, np_, kp // 2), dtype=np.uint8)
+    big_scales = np.full((experts, np_, kp // 32), 127, dtype=np.uint8)
+    for h in range(halves):
+        src = slice(h * n // halves, (h + 1) * n // halves)
+        dst = slice(h * np_ // halves, h * np_ // halves + n // halves)
+        big_packed[:, dst, : k // 2] = packed[:, src]
+        big_scales[:, dst, : k // 32] = scales[:, src]
+    got = ops.megamoe_prepare_weights(torch.from_numpy(packed).cuda(), torch.from_numpy(scales).cuda(), gate_up)
+    want = ops.megamoe_prepare_weights(torch.from_numpy(big_packed).cuda(), torch.from_numpy(big_scales).cuda(), gate_up)
+    assert got[0].shape == want[0].shape == (experts, np_, kp // 2)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
 
 
 @pytest.mark.parametrize("tile_rows", [64, 128, 192])
@@ -239,6 +271,45 @@ def test_public_api_workflow():
         buf.destroy()
     with pytest.raises(RuntimeError, match="destroyed"):
         megamoe.fp8_fp4_mega_moe(y, p1, p2, buf)
+
+
+def test_public_api_padded_sizes_and_packed_int32_scales():
+    """hidden % 64 and intermediate_hidden % 128 as the reference allows them (api.py:93-105), through the public
+    classes; the raw E8M0 scales given once as bytes [E,N,K/64,2] and once packed four to an int32 [E,N,K/128]
+    (api.py:340-352 accepts both): same prepared bytes, same output."""
+    from deepep_amd import megamoe
+
+    tokens, hidden, inter, experts, topk = 50, 1152, 384, 4, 2
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, experts, topk, seed=9)
+    buf = megamoe.SymmBuffer(None, experts, tokens, topk, hidden, inter)
+    try:
+        as_bytes = [(torch.from_numpy(w).cuda(), torch.from_numpy(sc).cuda()) for w, sc in (l1, l2)]
+        as_int32 = [(w, sc.reshape(*w.shape[:2], -1).contiguous().view(torch.int32)) for w, sc in as_bytes]
+        assert tuple(as_int32[0][1].shape) == (experts, 2 * inter, hidden // 128)
+        p1, p2 = megamoe.transform_weights_for_mega_moe(*as_bytes)
+        q1, q2 = megamoe.transform_weights_for_mega_moe(*as_int32)
+        for a, b in ((p1, q1), (p2, q2)):
+            assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        assert tuple(p1[0].shape) == (experts, 1024, 1280 // 2) and tuple(p2[0].shape) == (experts, 1280, 512 // 2)
+        buf.x.view(torch.uint8).copy_(torch.from_numpy(x_codes))
+        buf.x_sf.view(torch.uint8).copy_(torch.from_numpy(x_scales))
+        buf.topk_idx.copy_(torch.from_numpy(idx))
+        buf.topk_weights.copy_(torch.from_numpy(weights))
+        buf.validate_inputs(tokens)
+        y = torch.full((tokens, hidden), float("nan"), dtype=torch.bfloat16, device="cuda")
+        megamoe.fp8_fp4_mega_moe(y, q1, q2, buf)
+        want = _oracle(x_codes, x_scales, l1, l2, idx, weights, 0)
+        got = y.float().cpu().numpy()
+        assert np.isfinite(got).all()
+        assert mm.relative_frobenius(got, want) <= 2e-2
+        # prepared from a narrower raw tensor (I = 256): padded to the same prepared shape, but not this buffer's weights
+        narrow, _ = megamoe.transform_weights_for_mega_moe(
+            (as_bytes[0][0][:, :512].contiguous(), as_bytes[0][1][:, :512].contiguous()), as_bytes[1])
+        assert narrow[0].shape == q1[0].shape
+        with pytest.raises(ValueError, match="do not match the buffer"):
+            megamoe.fp8_fp4_mega_moe(y, narrow, q2, buf)
+    finally:
+        buf.destroy()
 
 
 def test_megamoe_forward_in_hip_graph(ops):

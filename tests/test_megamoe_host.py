@@ -21,7 +21,7 @@ def test_check_routing_messages():
 
 def test_symm_buffer_argument_gates():
     for kwargs in (
-        dict(num_experts=0), dict(num_topk=0), dict(hidden=512), dict(hidden=1024 + 64), dict(intermediate_hidden=256),
+        dict(num_experts=0), dict(num_topk=0), dict(hidden=512), dict(hidden=1024 + 32), dict(intermediate_hidden=128), dict(intermediate_hidden=320),
         dict(num_topk=5), dict(num_experts=6, group=LocalGroup(0, 4)),
     ):
         args = dict(group=None, num_experts=4, num_max_tokens_per_rank=17, num_topk=2, hidden=1024, intermediate_hidden=512)
