@@ -219,21 +219,17 @@ def megamoe_cpu_baseline(hidden, inter):
     )
 
 
-def megamoe_bench(torch, ops, timer, with_cpu):
-    """W4A8 fused expert FFN for one EP64 rank's share: 64 source ranks x 256 tokens, 384 experts of which
-    6 are local, top-8 uniform routing (about 2048 rows), H=7168, I=2048.  Random codes and constant scale bytes: the
-    time does not depend on the values.  FLOPs = 2*R*H*2I + 2*R*I*H for the R rows that reach a local expert."""
+def megamoe_shape(torch, ops, timer, tokens, experts, local, topk, weight_sets, hidden=7168, inter=2048):
+    """One W4A8 forward shape: (back-to-back us, flushed statistics, rows that reach a local expert, FLOPs).  Random codes
+    and constant scale bytes: the time does not depend on the values.  FLOPs = 2*R*H*2I + 2*R*I*H for the R rows."""
     dev = "cuda"
-    tokens, hidden, inter, experts, local, topk = 64 * 256, 7168, 2048, 384, 6, 8
     gen = torch.Generator().manual_seed(0)
     idx = torch.multinomial(torch.ones(tokens, experts), topk, generator=gen).to(torch.int32).to(dev)
     w = torch.softmax(torch.randn(tokens, topk, generator=gen), -1).to(dev)
     x_codes = torch.randint(0, 120, (tokens, hidden), dtype=torch.uint8, generator=gen).to(dev).view(torch.float8_e4m3fn)
     x_scales = torch.full((tokens, hidden // 32), 127, dtype=torch.uint8, device=dev)
-    # Three weight sets used in turn (3 x 132 MB, more than the 256 MB memory-side cache), so that the GEMMs
-    # stream their weights from HBM as they do between the layers of a model.
     sets = []
-    for _ in range(3):
+    for _ in range(weight_sets):
         w1 = torch.randint(0, 256, (local, 2 * inter, hidden // 2), dtype=torch.uint8, device=dev)
         s1 = torch.full((local, 2 * inter, ops.megamoe_prepared_shape(2 * inter, hidden, True)[2]), 119, dtype=torch.uint8, device=dev)
         w2 = torch.randint(0, 256, (local, hidden, inter // 2), dtype=torch.uint8, device=dev)
@@ -254,6 +250,17 @@ def megamoe_bench(torch, ops, timer, with_cpu):
     rows = int(counts.sum().item())
     flops = 2.0 * rows * hidden * 2 * inter + 2.0 * rows * inter * hidden
     ws.destroy()
+    return us, cold, rows, flops
+
+
+def megamoe_bench(torch, ops, timer, with_cpu):
+    """W4A8 fused expert FFN, H=7168, I=2048.  The headline shape is one EP64 rank's share: 64 source ranks x 256 tokens,
+    384 experts of which 6 are local, top-8 uniform routing (about 2000 rows), with three weight sets used in turn
+    (3 x 132 MB, more than the 256 MB memory-side cache) so that the GEMMs stream their weights from HBM as they do
+    between the layers of a model.  `large_batch` is the same kernels where tile quantisation and fixed costs stop
+    mattering: 8192 tokens x top-8 over 32 local experts (65 536 rows)."""
+    hidden, inter = 7168, 2048
+    us, cold, rows, flops = megamoe_shape(torch, ops, timer, 64 * 256, 384, 6, 8, weight_sets=3)
     result = {
         "workload": "EP64 rank share: 16384 candidate tokens, 6 of 384 experts local, top-8, H=7168, I=2048, "
         "MXFP8 activations x MXFP4 weights (random codes, constant scale bytes), three weight sets in turn; layout + "
@@ -266,6 +273,14 @@ def megamoe_bench(torch, ops, timer, with_cpu):
         "roofline": {"bound": "mfma", "achieved": flops / us / 1e6, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
                      "note": "whole forward (4 launches), back to back; per-kernel GEMM times are in profiles/"},
+    }
+    big = Timer(torch, max(1, timer.iters // 5), max(1, timer.warmups // 5))
+    big.flush, big.cycles_per_us = timer.flush, timer.cycles_per_us
+    us, cold, rows, flops = megamoe_shape(torch, ops, big, 8192, 32, 32, 8, weight_sets=1)
+    result["large_batch"] = {
+        "workload": "8192 tokens x top-8, all 32 experts local (65 536 rows), one weight set (705 MB); whole forward",
+        "rows": rows, "us_forward": us, "flushed_us": cold, "gflop": flops / 1e9, "tflops_forward": flops / us / 1e6,
+        "frac_of_fp8_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
     }
     if with_cpu:
         result["cpu_baseline"] = megamoe_cpu_baseline(hidden, inter)

@@ -887,7 +887,7 @@ struct ScheduleFault {
 };
 
 template <int RT>
-bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, ScheduleFault* fault)
+bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, bool drain_at_switches, ScheduleFault* fault)
 {
     using Ring = GemmRing<RT>;
     constexpr int kAhead = Ring::kAhead, kCopies = Ring::kCopies;
@@ -912,7 +912,7 @@ bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, ScheduleFau
     auto advance = [&](bool in_prologue, int item) {
         if (++copy_kt == ktiles) {
             if (copy_tile + 1 < my_tiles) {
-                if (switch_needs_drain(in_prologue, ktiles, kAhead)) wait(0);
+                if (drain_at_switches && switch_needs_drain(in_prologue, ktiles, kAhead)) wait(0);
                 if (index_op >= done && ok) {
                     ok = false;
                     *fault = {item, 2};
@@ -988,16 +988,17 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
     return launch_status("mx_quant");
 }
 
-int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores)
+int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int without_drain)
 {
     using namespace dpep;
     DPEP_REQUIRE(tile_rows == 64 || tile_rows == 128 || tile_rows == 192, "schedule_check: tile_rows is 64, 128 or 192");
     DPEP_REQUIRE(tiles_per_workgroup >= 0 && ktiles >= 2 && ktiles % 2 == 0 && epilogue_stores >= 0,
                  "schedule_check: bad arguments");
     ScheduleFault fault = {0, 0};
-    const bool ok = tile_rows == 64    ? replay_workgroup<1>(tiles_per_workgroup, ktiles, epilogue_stores, &fault)
-                    : tile_rows == 128 ? replay_workgroup<2>(tiles_per_workgroup, ktiles, epilogue_stores, &fault)
-                                       : replay_workgroup<3>(tiles_per_workgroup, ktiles, epilogue_stores, &fault);
+    const bool drain = without_drain == 0;
+    const bool ok = tile_rows == 64    ? replay_workgroup<1>(tiles_per_workgroup, ktiles, epilogue_stores, drain, &fault)
+                    : tile_rows == 128 ? replay_workgroup<2>(tiles_per_workgroup, ktiles, epilogue_stores, drain, &fault)
+                                       : replay_workgroup<3>(tiles_per_workgroup, ktiles, epilogue_stores, drain, &fault);
     if (!ok)
         return fail(DPEP_EINVAL, "schedule_check: %s read before any wait covers them (item %d)",
                     fault.what == 1 ? "an item's copies are" : "the next tile's gather indices are", fault.item);

@@ -166,8 +166,10 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
  * rows and `ktiles` k tiles of 128 every asynchronous copy is covered by a counted wait before it is read, under
  * in-order completion of vector-memory operations: an item's operands before its MFMAs, the next tile's gather
  * indices before the copy cursor switches tiles).  epilogue_stores = stores a tile end issues (they only make the
- * counted waits stricter).  Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
-int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores);
+ * counted waits stricter).  without_drain != 0 replays the schedule WITHOUT the cursor's wait at tile switches (what a
+ * kernel that trusted every index fetch would do): the check then has to fail for tiles shorter than the copies run ahead,
+ * which is how the tests know that it can.  Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
+int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int without_drain);
 
 /* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480).
  * num_shared = number of shared experts (0..8) whose rows (every token, each) are held next to the routed ones. */

@@ -16,7 +16,7 @@ def test_schedule_holds_everywhere(tile_rows):
     lib = _lib.load()
     cases = 0
     for ktiles, tiles, epilogue in itertools.product((2, 4, 6, 8, 10, 14, 16, 56, 64), (0, 1, 2, 3, 5, 24, 100), (0, 48, 192)):
-        status = lib.dpep_megamoe_schedule_check(tile_rows, tiles, ktiles, epilogue)
+        status = lib.dpep_megamoe_schedule_check(tile_rows, tiles, ktiles, epilogue, 0)
         assert status == 0, (ktiles, tiles, epilogue, lib.dpep_last_error().decode())
         cases += 1
     assert cases == 9 * 7 * 3
@@ -24,6 +24,20 @@ def test_schedule_holds_everywhere(tile_rows):
 
 def test_schedule_check_rejects_bad_arguments():
     lib = _lib.load()
-    assert lib.dpep_megamoe_schedule_check(100, 10, 8, 0) == -1
-    assert lib.dpep_megamoe_schedule_check(128, 10, 7, 0) == -1
+    assert lib.dpep_megamoe_schedule_check(100, 10, 8, 0, 0) == -1
+    assert lib.dpep_megamoe_schedule_check(128, 10, 7, 0, 0) == -1
     assert b"schedule_check" in lib.dpep_last_error()
+
+
+@pytest.mark.parametrize("tile_rows,ahead", [(64, 5), (128, 4), (192, 3)])
+def test_replay_catches_a_schedule_without_the_wait_at_switches(tile_rows, ahead):
+    """The same replay with the cursor's wait at tile switches left out fails exactly where the rule says the wait is
+    needed: more than one tile per workgroup and either a switch inside the prologue (tiles no longer than the copies
+    run ahead) or tiles shorter than that.  Long tiles pass either way: a counted wait has covered the index fetch."""
+    lib = _lib.load()
+    for ktiles, tiles in itertools.product((2, 4, 6, 8, 16, 56), (1, 2, 3, 24)):
+        status = lib.dpep_megamoe_schedule_check(tile_rows, tiles, ktiles, 48, 1)
+        must_fail = tiles > 1 and ktiles <= ahead
+        assert (status != 0) == must_fail, (tile_rows, ktiles, tiles, lib.dpep_last_error().decode())
+        if must_fail:
+            assert b"gather indices" in lib.dpep_last_error()
