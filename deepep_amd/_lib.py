@@ -32,6 +32,7 @@ SIGNATURES = {
     "dpep_dispatch_quant_fp8": (_I, (_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_layout_dispatch_small": (_I, (_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P)),
     "dpep_cast_to_fp8": (_I, (_P, _I, _I, _P, _P, _P)),
+    "dpep_cast_back": (_I, (_P, _P, _I, _I, _I, _P, _P)),
     "dpep_combine": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_combine_fp16": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_mx_quant": (_I, (_P, _I, _I, _P, _P, _P)),

@@ -235,6 +235,38 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_row_kernel(
     if (part == 0 && weights != nullptr && threadIdx.x == 0) out_weights[row] = weights[route];
 }
 
+// ---- dequantiser: bf16(fp32(code) * scale) per block of 128 columns ---------------------------------------------
+// One thread per 16 codes (16 bytes in, 32 bytes out).  kByteScales: the scales are e8m0 bytes (four to an int32 in the
+// caller's tensor), value 2^(byte - 127) built by moving the byte into the exponent field; else fp32.  The last block of a
+// row may be short (hidden need only be a multiple of 16).
+template <bool kByteScales>
+__global__ __launch_bounds__(256) void cast_back_kernel(const u32x4* __restrict__ codes, const void* __restrict__ scales,
+                                                        int units_per_row, int scales_per_row, long long total_units,
+                                                        u32x4* __restrict__ out)
+{
+    const long long id = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total_units) return;
+    const long long row = id / units_per_row;
+    const int unit = static_cast<int>(id % units_per_row);
+    const long long at = row * scales_per_row + (unit >> 3);
+    const float scale = kByteScales ? __uint_as_float(static_cast<uint32_t>(static_cast<const uint8_t*>(scales)[at]) << 23)
+                                    : static_cast<const float*>(scales)[at];
+    const u32x4 q = load16_nt(codes + id);
+    u32x4 lo, hi;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int word = static_cast<int>(q[i]);
+        const float a = __fmul_rn(__builtin_amdgcn_cvt_f32_fp8(word, 0), scale);
+        const float b = __fmul_rn(__builtin_amdgcn_cvt_f32_fp8(word, 1), scale);
+        const float c = __fmul_rn(__builtin_amdgcn_cvt_f32_fp8(word, 2), scale);
+        const float d = __fmul_rn(__builtin_amdgcn_cvt_f32_fp8(word, 3), scale);
+        (i < 2 ? lo : hi)[(i & 1) * 2] = pack_bf16x2(a, b);
+        (i < 2 ? lo : hi)[(i & 1) * 2 + 1] = pack_bf16x2(c, d);
+    }
+    store16_nt(out + 2 * id, lo);
+    store16_nt(out + 2 * id + 1, hi);
+}
+
 // ---- small batches: routing layout and payload in ONE launch -------------------------------------------------
 // With at most kSmallRoutes routes (a decode step) the whole routing table fits a workgroup's LDS, and a workgroup
 // gets the rows of its own token faster by working them out itself than by waiting for a layout kernel: every
@@ -563,6 +595,26 @@ int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float
                        static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), nullptr, nullptr, 1, units,
                        sp.per_part, sp.parts, static_cast<u32x4*>(out), out_scales, nullptr);
     return launch_status("cast_to_fp8");
+}
+
+int dpep_cast_back(const void* codes, const void* scales, int scales_are_e8m0_bytes, int num_tokens, int hidden, void* out,
+                   void* stream)
+{
+    using namespace dpep;
+    DPEP_REQUIRE(num_tokens >= 0, "cast_back: bad T=%d", num_tokens);
+    DPEP_REQUIRE(hidden > 0 && hidden % 16 == 0, "cast_back: hidden=%d must be a positive multiple of 16", hidden);
+    if (num_tokens == 0) return DPEP_OK;
+    DPEP_REQUIRE(codes && scales && out && aligned16(codes) && aligned16(out), "cast_back: codes/out must be 16-byte aligned");
+    const int units = hidden / 16, blocks_per_row = (hidden + 127) / 128;
+    const long long total = static_cast<long long>(num_tokens) * units;
+    const unsigned grid = static_cast<unsigned>((total + 255) / 256);
+    if (scales_are_e8m0_bytes)
+        hipLaunchKernelGGL(cast_back_kernel<true>, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const u32x4*>(codes), scales, units, blocks_per_row, total, static_cast<u32x4*>(out));
+    else
+        hipLaunchKernelGGL(cast_back_kernel<false>, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const u32x4*>(codes), scales, units, blocks_per_row, total, static_cast<u32x4*>(out));
+    return launch_status("cast_back");
 }
 
 }  // extern "C"

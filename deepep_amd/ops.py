@@ -311,6 +311,29 @@ def cast_to_fp8(x):
     return out, scales
 
 
+def cast_back(codes, scales):
+    """per_token_cast_back on the device: (FP8 e4m3fn [T,H], scales) -> BF16 [T,H], bf16(fp32(code) * scale) per block of
+    128 columns.  scales: FP32 [T, ceil(H/128)], or int32 [T, ceil(H/128)/4] holding four e8m0 exponent bytes each."""
+    lib = _lib.load()
+    _require("codes", codes, torch.float8_e4m3fn)
+    if codes.ndim != 2 or codes.shape[1] % 16 or codes.shape[1] == 0:
+        raise ValueError("codes must be [T, H] with H a positive multiple of 16")
+    tokens, hidden = codes.shape
+    blocks = (hidden + 127) // 128
+    if scales.dtype == torch.int32:
+        if blocks % 4:
+            raise ValueError("int32 scales hold four blocks each: ceil(H/128) must be a multiple of 4")
+        _require("scales", scales, torch.int32, (tokens, blocks // 4), codes.device)
+    else:
+        _require("scales", scales, torch.float32, (tokens, blocks), codes.device)
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=codes.device)
+    with _on_device(codes.device):
+        status = lib.dpep_cast_back(_ptr(codes), _ptr(scales), int(scales.dtype == torch.int32), tokens, hidden, _ptr(out),
+                                    _stream(codes.device))
+    _lib.check(status, "cast_back")
+    return out
+
+
 def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
     """out[t] = round( sum_s fp32(y[row(t,s)]) (* row_weights[row]) ) in y's dtype (BF16 or FP16); optional
     weight-return channel."""

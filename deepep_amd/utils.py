@@ -20,15 +20,23 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 
 def per_token_cast_back(x_fp8: torch.Tensor, x_scales: torch.Tensor) -> torch.Tensor:
-    """bf16(fp32(q) * scale); int32 scales are four packed e8m0 bytes of which the low one is used."""
+    """bf16(fp32(q) * scale) per block of 128 columns (deep_ep/utils/math.py:64-79); an int32 scale holds the e8m0
+    exponent bytes of four consecutive blocks.  Device tensors go through the HIP kernel (``dpep_cast_back``); host
+    tensors are evaluated with torch, as the reference does on any device."""
     if x_fp8.numel() == 0:
         return x_fp8.to(torch.bfloat16)
     if x_fp8.dim() != 2:
         raise AssertionError("x_fp8 must be a 2D tensor")
     tokens, hidden = x_fp8.shape
-    if hidden % 128:
-        raise ValueError("hidden must be a multiple of 128")
+    blocks = (hidden + 127) // 128
+    if x_fp8.is_cuda and hidden % 16 == 0 and (x_scales.dtype != torch.int or blocks % 4 == 0):
+        from . import ops
+
+        scales = x_scales.contiguous()
+        scales = scales.view(tokens, -1) if scales.dtype == torch.int else scales.to(torch.float32).view(tokens, blocks)
+        return ops.cast_back(x_fp8.contiguous(), scales)
     if x_scales.dtype == torch.int:
         x_scales = (x_scales.view(dtype=torch.uint8).to(torch.int) << 23).view(dtype=torch.float)
-    values = x_fp8.to(torch.float32).view(tokens, -1, 128)
-    return (values * x_scales.view(tokens, -1, 1)).view(tokens, hidden).to(torch.bfloat16)
+    padded = torch.nn.functional.pad(x_fp8.to(torch.float32), (0, blocks * 128 - hidden))
+    values = padded.view(tokens, blocks, 128)
+    return (values * x_scales.view(tokens, -1, 1)).view(tokens, blocks * 128).to(torch.bfloat16)[:, :hidden].contiguous()

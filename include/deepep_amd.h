@@ -136,6 +136,13 @@ int dpep_layout_dispatch_small(void* ws, const int64_t* topk_idx, const void* x,
 /* Stand-alone per-128 quantiser (deep_ep/utils/math.py:45-61): x bf16 [T,H] -> fp8 [T,H], fp32 [T,H/128]. */
 int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float* out_scales, void* stream);
 
+/* The dequantiser the reference checks its FP8 path with: out = bf16(fp32(code) * scale), one scale per block of 128
+ * columns (per_token_cast_back, deep_ep/utils/math.py:64-79).  scales: fp32 [T, ceil(H/128)], or, scales_are_e8m0_bytes
+ * != 0, one exponent byte per block (the reference's int32 scale tensors hold four of them each, math.py:74-76).
+ * H % 16 == 0; the last block of a row may be short.  codes e4m3fn [T,H] -> out bf16 [T,H]. */
+int dpep_cast_back(const void* codes, const void* scales, int scales_are_e8m0_bytes, int num_tokens, int hidden, void* out,
+                   void* stream);
+
 /* Combine: out[t] = bf16_rne( sum over slots in order, skipping -1, of fp32(y[row]) (* w[row]) ).
  * Replaces combine() (csrc/ops/combine.cpp:198-326 -> combine_kernel, csrc/kernels/combine/combine.cpp:2965)
  * with row_weights == NULL, and aggregate() / the low-latency combine

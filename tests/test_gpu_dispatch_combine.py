@@ -216,6 +216,62 @@ def test_cast_to_fp8_every_bf16_magnitude(ops):
     np.testing.assert_array_equal(f32_bits(s), s_ref.view(np.uint32))
 
 
+def _finite_codes(shape, seed):
+    codes = np.random.default_rng(seed).integers(0, 256, shape, dtype=np.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x7E  # 0x7F / 0xFF are NaN in e4m3fn; checked apart
+    return codes
+
+
+def test_cast_back_every_code_and_scale_bit_exact(ops):
+    """The dequantiser (per_token_cast_back, deep_ep/utils/math.py:64-79): every finite e4m3fn code under scales from
+    2^-30 to 2^20 and non-powers of two, bit for bit against the oracle; NaN codes stay NaN."""
+    scales = np.array([2.0 ** -30, 1e-4 / 448, 0.001, 1 / 3, 1.0, 1.5, 448.0 / 7, 2.0 ** 20], dtype=np.float32)
+    codes = np.tile(np.arange(256, dtype=np.uint8), (scales.size, 1))  # row i: all codes, one 256-column row = 2 blocks
+    nan = (codes & 0x7F) == 0x7F
+    finite = np.where(nan, 0, codes).astype(np.uint8)
+    row_scales = np.stack([scales, scales[::-1]], axis=1).copy()  # a different scale for each of the two blocks
+    got = ops.cast_back(torch.from_numpy(finite).cuda().view(torch.float8_e4m3fn), torch.from_numpy(row_scales).cuda())
+    np.testing.assert_array_equal(bf16_bits(got), oquant.cast_back(finite, row_scales))
+    got_nan = ops.cast_back(torch.from_numpy(codes).cuda().view(torch.float8_e4m3fn), torch.from_numpy(row_scales).cuda())
+    assert torch.isnan(got_nan.float().cpu()).numpy()[nan].all()
+    np.testing.assert_array_equal(bf16_bits(got_nan)[~nan], oquant.cast_back(finite, row_scales)[~nan])
+
+
+@pytest.mark.parametrize("tokens,hidden", [(1, 128), (33, 7168), (5, 16), (7, 144), (12, 2064)])
+def test_cast_back_widths_and_packed_exponent_scales(ops, tokens, hidden):
+    """Widths that are not multiples of 128 (short last block, as the reference pads) and the int32 form of the scales
+    (four e8m0 exponent bytes each, math.py:74-76), against the same expression evaluated with torch on the host."""
+    from deepep_amd.utils import per_token_cast_back
+
+    blocks = (hidden + 127) // 128
+    codes = torch.from_numpy(_finite_codes((tokens, hidden), hidden)).view(torch.float8_e4m3fn)
+    scales = torch.rand(tokens, blocks, generator=torch.Generator().manual_seed(tokens)) * 4 + 1e-3
+    want = per_token_cast_back(codes, scales)  # host tensors: plain torch
+    got = per_token_cast_back(codes.cuda(), scales.cuda())  # device tensors: the HIP kernel
+    np.testing.assert_array_equal(bf16_bits(got), bf16_bits(want))
+    if blocks % 4 == 0:
+        exponents = torch.randint(100, 140, (tokens, blocks), generator=torch.Generator().manual_seed(1), dtype=torch.uint8)
+        packed = exponents.view(torch.int32)
+        want = per_token_cast_back(codes, packed)
+        got = per_token_cast_back(codes.cuda(), packed.cuda())
+        np.testing.assert_array_equal(bf16_bits(got), bf16_bits(want))
+        as_float = torch.pow(2.0, exponents.float() - 127)
+        np.testing.assert_array_equal(bf16_bits(got), bf16_bits(per_token_cast_back(codes, as_float)))
+
+
+def test_cast_back_restores_what_cast_to_fp8_made(ops):
+    """Round trip on the device: quantise, dequantise, compare with the oracle's round trip bit for bit and with the input
+    to the format's precision (2^-4 relative per element at most, e4m3 has 3 mantissa bits)."""
+    x, _, _, _ = cases.make_inputs("C2")
+    q, s = ops.cast_to_fp8(x.cuda())
+    back = ops.cast_back(q, s)
+    q_ref, s_ref = oquant.cast_to_fp8_torch(x)
+    np.testing.assert_array_equal(bf16_bits(back), oquant.cast_back(fp8_bits(q_ref), s_ref.numpy()))
+    err = (back.float().cpu() - x.float()).abs()
+    bound = x.float().abs().view(x.shape[0], -1, 128).amax(-1, keepdim=True).expand(-1, -1, 128).reshape(x.shape) / 16
+    assert (err <= bound + 1e-6).all()
+
+
 @pytest.mark.parametrize("name,tokens", [("C1", None), ("C2", None), ("C3", 700), ("C4", 4096)])
 def test_dispatch_quant_fp8_fused_equals_quantize_then_copy(ops, ws, name, tokens):
     x, idx, w, cfg = cases.make_inputs(name, tokens=tokens)
