@@ -235,6 +235,25 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_row_kernel(
     if (part == 0 && weights != nullptr && threadIdx.x == 0) out_weights[row] = weights[route];
 }
 
+// Stand-alone quantiser for rows whose width is not a multiple of 128: the last block of a row is short and is
+// quantised as if padded with zeros (per_token_cast_to_fp8 pads, deep_ep/utils/math.py:52-53).  One thread per 16 values
+// of the padded row, so the eight lanes of a block are always all present; padding units load and store nothing.
+__global__ __launch_bounds__(256) void cast_to_fp8_short_block_kernel(const u32x4* __restrict__ x, int units_per_row,
+                                                                      int blocks_per_row, long long padded_units,
+                                                                      u32x4* __restrict__ out, float* __restrict__ out_scales)
+{
+    const long long id = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= padded_units) return;  // padded_units is a multiple of 8: whole blocks leave together
+    const long long row = id / (blocks_per_row * 8);
+    const int unit = static_cast<int>(id % (blocks_per_row * 8));
+    const bool real = unit < units_per_row;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const u32x4* src = x + (row * units_per_row + unit) * 2;
+    const Quant16 q = quantize16(real ? load16(src) : zero, real ? load16(src + 1) : zero);
+    if (real) store16_nt(out + row * units_per_row + unit, q.codes);
+    if ((unit & 7) == 0) out_scales[row * blocks_per_row + (unit >> 3)] = q.scale;
+}
+
 // ---- dequantiser: bf16(fp32(code) * scale) per block of 128 columns ---------------------------------------------
 // One thread per 16 codes (16 bytes in, 32 bytes out).  kByteScales: the scales are e8m0 bytes (four to an int32 in the
 // caller's tensor), value 2^(byte - 127) built by moving the byte into the exponent field; else fp32.  The last block of a
@@ -586,10 +605,18 @@ int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float
 {
     using namespace dpep;
     DPEP_REQUIRE(num_tokens >= 0, "cast_to_fp8: bad T=%d", num_tokens);
-    DPEP_REQUIRE(hidden > 0 && hidden % 128 == 0, "cast_to_fp8: hidden=%d must be a positive multiple of 128", hidden);
+    DPEP_REQUIRE(hidden > 0 && hidden % 16 == 0, "cast_to_fp8: hidden=%d must be a positive multiple of 16", hidden);
     if (num_tokens == 0) return DPEP_OK;
     DPEP_REQUIRE(x && out && out_scales && aligned16(x) && aligned16(out), "cast_to_fp8: x/out must be 16-byte aligned");
     const int units = hidden / 16;
+    if (hidden % 128 != 0) {
+        const int blocks = (hidden + 127) / 128;
+        const long long padded = static_cast<long long>(num_tokens) * blocks * 8;
+        hipLaunchKernelGGL(cast_to_fp8_short_block_kernel, dim3(static_cast<unsigned>((padded + 255) / 256)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), units, blocks, padded,
+                           static_cast<u32x4*>(out), out_scales);
+        return launch_status("cast_to_fp8");
+    }
     const Split sp = choose_split(num_tokens, units, 8);
     hipLaunchKernelGGL(dispatch_quant_row_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0,
                        static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), nullptr, nullptr, 1, units,

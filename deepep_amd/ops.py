@@ -297,14 +297,15 @@ def dispatch_quant_fp8(x, topk_weights, route_to_row, row_to_route, num_rows: Op
 
 
 def cast_to_fp8(x):
-    """per_token_cast_to_fp8 on the device: BF16 [T,H] -> (FP8 [T,H], FP32 [T,H/128])."""
+    """per_token_cast_to_fp8 on the device: BF16 [T,H] -> (FP8 [T,H], FP32 [T,ceil(H/128)]); a short last block is
+    quantised as if padded with zeros, as the reference does."""
     lib = _lib.load()
     _require("x", x, torch.bfloat16)
-    if x.ndim != 2 or x.shape[1] % 128:
-        raise ValueError("x must be [T, H] with H a multiple of 128")
+    if x.ndim != 2 or x.shape[1] % 16 or x.shape[1] == 0:
+        raise ValueError("x must be [T, H] with H a positive multiple of 16")
     tokens, hidden = x.shape
     out = torch.empty((tokens, hidden), dtype=torch.float8_e4m3fn, device=x.device)
-    scales = torch.empty((tokens, hidden // 128), dtype=torch.float32, device=x.device)
+    scales = torch.empty((tokens, (hidden + 127) // 128), dtype=torch.float32, device=x.device)
     with _on_device(x.device):
         status = lib.dpep_cast_to_fp8(_ptr(x), tokens, hidden, _ptr(out), _ptr(scales), _stream(x.device))
     _lib.check(status, "cast_to_fp8")

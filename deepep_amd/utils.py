@@ -12,8 +12,8 @@ from . import ops
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Quantise each group of 128 values to E4M3 with FP32 scales, on the GPU (HIP kernel).
 
-    Bit-identical to the reference's torch expression on CPU.  ``x`` must be a contiguous BF16
-    [T, H] GPU tensor with H a multiple of 128 (the reference zero-pads other widths)."""
+    Bit-identical to the reference's torch expression on CPU.  ``x`` must be a contiguous BF16 [T, H] GPU tensor with
+    H a multiple of 16; a last block shorter than 128 is quantised as if padded with zeros, as in the reference."""
     if x.dim() != 2:
         raise AssertionError("x must be a 2D tensor")
     return ops.cast_to_fp8(x)

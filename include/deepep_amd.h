@@ -133,7 +133,8 @@ int dpep_layout_dispatch_small(void* ws, const int64_t* topk_idx, const void* x,
                                int32_t* offsets, int32_t* route_to_row, int32_t* row_to_route, int32_t* num_rows, void* out,
                                float* out_scales, float* out_weights, void* stream);
 
-/* Stand-alone per-128 quantiser (deep_ep/utils/math.py:45-61): x bf16 [T,H] -> fp8 [T,H], fp32 [T,H/128]. */
+/* Stand-alone per-128 quantiser (deep_ep/utils/math.py:45-61): x bf16 [T,H] -> fp8 [T,H], fp32 [T,ceil(H/128)].
+ * H % 16 == 0; a last block shorter than 128 is quantised as if padded with zeros (math.py:52-53). */
 int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float* out_scales, void* stream);
 
 /* The dequantiser the reference checks its FP8 path with: out = bf16(fp32(code) * scale), one scale per block of 128

@@ -216,6 +216,21 @@ def test_cast_to_fp8_every_bf16_magnitude(ops):
     np.testing.assert_array_equal(f32_bits(s), s_ref.view(np.uint32))
 
 
+@pytest.mark.parametrize("tokens,hidden", [(3, 16), (9, 144), (17, 2064), (5, 7168 + 64), (4, 112)])
+def test_cast_to_fp8_short_last_block(ops, tokens, hidden):
+    """Widths that are not multiples of 128: the last block is quantised as if padded with zeros
+    (deep_ep/utils/math.py:52-53), bit for bit against the reference expression on the padded row."""
+    gen = torch.Generator().manual_seed(hidden)
+    x = (torch.randn(tokens, hidden, generator=gen) * 3).bfloat16()
+    x[0, -16:] = 0  # a short block of zeros: amax floor 1e-4
+    padded = torch.nn.functional.pad(x, (0, (-hidden) % 128))
+    q_ref, s_ref = oquant.cast_to_fp8_torch(padded)
+    q, s = ops.cast_to_fp8(x.cuda())
+    assert tuple(s.shape) == (tokens, (hidden + 127) // 128)
+    np.testing.assert_array_equal(fp8_bits(q), fp8_bits(q_ref)[:, :hidden])
+    np.testing.assert_array_equal(f32_bits(s), f32_bits(s_ref))
+
+
 def _finite_codes(shape, seed):
     codes = np.random.default_rng(seed).integers(0, 256, shape, dtype=np.uint8)
     codes[(codes & 0x7F) == 0x7F] = 0x7E  # 0x7F / 0xFF are NaN in e4m3fn; checked apart
