@@ -42,12 +42,12 @@ struct Workspace {
     uint32_t* mailbox_device;  // the same memory as the kernels address it
     uint32_t sequence;         // of the most recent layout launch
     int mailbox_local;         // its number of local experts
-    // One-launch layout: its barrier between workgroups (device memory, zero between launches), the bound of the
-    // barrier's wait in 100 MHz ticks, and two switches for tests (take two launches instead; expect more
-    // arrivals than there are workgroups, so that the wait runs out).
-    void* barrier;  // kSyncBytes of device memory behind the caller's bytes, see below
-    long long barrier_ticks;
-    int barrier_extra_arrivals;
+    // One-launch layout: the memory its workgroups exchange histograms through, the bound of a workgroup's wait for the
+    // others' histograms in 100 MHz ticks, and two switches for tests (take two launches instead; expect more
+    // histogram rows than there are workgroups, so that the wait runs out).
+    void* sync;  // kSyncBytes of device memory behind the caller's bytes, see below
+    long long exchange_ticks;
+    int exchange_extra_rows;
     int layout_one_launch;
     uint32_t layout_launches;  // number of the most recent layout launch (never 0)
     uint32_t timeout_seen;     // number of the last timed-out launch the host has been told about
@@ -55,18 +55,22 @@ struct Workspace {
     int gemm_zero_fill;        // 1 (default): idle workgroups of the first GEMM zero rows of unserved tokens; 0: the reduce does
     int gemm_tile_rows;  // 0: the grouped GEMM chooses its tile height; 64 / 128 / 192: forced (tests)
 };
-// Small words the kernels synchronise through, zero when the workspace is created and left zero by every launch:
-// the layout's barrier at offset 0 (two counters); the word at kSyncFillStop, through which the MegaMoE fillers are
-// told to stop, holds the number of the launch that wrote it last and needs no clearing.
-constexpr size_t kSyncBytes = 256;
+// Device memory the kernels synchronise through, behind the caller's bytes, zero when the workspace is created:
+// at offset 0 the one-launch layout's epoch (64 bits: the highest tag any launch has used; a launch tags what it
+// publishes with epoch + 1 and raises the epoch when it ends, so a replayed HIP graph gets a fresh tag too); at
+// kSyncFillStop the word through which the MegaMoE fillers are told to stop (it holds the number of the launch that wrote
+// it last and needs no clearing); from kSyncTagged on the tagged per-workgroup histograms of the one-launch layout.
 constexpr size_t kSyncFillStop = 64;
+constexpr size_t kSyncTagged = 256;
+constexpr size_t kSyncTaggedWords = 4096 + DPEP_MAX_LOCAL_EXPERTS;  // (workgroups + 1) * experts never exceeds this
+constexpr size_t kSyncBytes = kSyncTagged + kSyncTaggedWords * 8;
 // The host mailbox (pinned memory, 32-bit words): word 0 = number of rows and word 1 = sequence number of the layout
 // that reported last (one 8-byte store); word kMailboxTimeout = launch number of a layout kernel whose barrier wait
 // ran out; from word kMailboxCounts on, 16-byte aligned, the per-expert counts.
 constexpr int kMailboxTimeout = 2;
 constexpr int kMailboxCounts = 4;
 constexpr int kMailboxWords = kMailboxCounts + (DPEP_MAX_LOCAL_EXPERTS + 3) / 4 * 4;
-constexpr long long kLayoutBarrierTicks = 200000000;  // 2 s
+constexpr long long kLayoutExchangeTicks = 200000000;  // 2 s
 constexpr uint32_t kWorkspaceMagic = 0x44504550u;  // "DPEP"
 Workspace* as_workspace(void* ws);
 

@@ -15,11 +15,12 @@
 //            its expert's next free row plus the number of lower lanes in the mask.  The carry between steps
 //            lives in LDS.  There is no separate scan launch.
 // Inputs whose chunks fit a wave's registers (at most kKeep steps of 64 routes) take ONE launch: the workgroups
-// (at most 65, far fewer than there are CUs, so all are resident together) count, meet at a barrier in device
-// memory, and assign from the ids they still hold.  The barrier's wait is bounded; a launch whose wait runs out
-// assigns nothing (its histograms may be stale): it reports no rows, marks every route as having none, and leaves
-// its number in the workspace's mailbox, where the host finds it; later layouts on that workspace take two
-// launches.  Larger inputs take two launches anyway.
+// (at most 65, far fewer than there are CUs, so all are resident together) count, publish their histograms as
+// self-validating words (count + the launch's tag in one 64-bit store), read each other's as soon as they appear, and
+// assign from the ids they still hold: no barrier, no counter that anybody has to reset.  The wait for the others'
+// words is bounded; a launch whose wait runs out assigns nothing (a histogram is missing): it reports no rows, marks
+// every route as having none, and leaves its number in the workspace's mailbox, where the host finds it; later layouts
+// on that workspace take two launches.  Larger inputs take two launches anyway.
 #include <mutex>
 
 #include "common.h"
@@ -35,6 +36,7 @@ constexpr int kMinChunk = 256;        // routes per wavefront, lower bound (mult
 constexpr int kPrefetch = 8;          // 64-route steps whose ids are fetched at once
 constexpr int kKeep = 16;             // 64-route steps of a chunk that the one-launch kernel holds in registers
 constexpr int kColumnBatch = 16;      // histogram loads in flight per thread
+static_assert(kSyncTaggedWords >= static_cast<size_t>(kBlockHistInts), "the tagged histograms need a word per (workgroup, expert)");
 
 __device__ __forceinline__ uint64_t lanes_below()
 {
@@ -75,20 +77,9 @@ struct LayoutLds {
     unsigned long long match[kWaves][DPEP_MAX_LOCAL_EXPERTS];
     int partial[kThreads * 2];
     int wave_sums[kWaves];
+    int timed_out;  // one-launch kernel: some thread's wait for another workgroup's histogram ran out
+    unsigned long long tag;  // one-launch kernel: the tag of this launch, read once per workgroup
 };
-
-// kCoherent: the access goes past the caches (in the one-launch kernel other CUs read what this one has just written).
-template <bool kCoherent>
-__device__ __forceinline__ void store_int(int* dst, int value)
-{
-    if (kCoherent) __hip_atomic_store(dst, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *dst = value;
-}
-template <bool kCoherent>
-__device__ __forceinline__ int load_int(const int* src)
-{
-    return kCoherent ? __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *src;
-}
 
 __device__ __forceinline__ void clear_wave_lds(LayoutLds& lds, int num_local)
 {
@@ -106,7 +97,6 @@ __device__ __forceinline__ void count_step(int e, int* __restrict__ mine)
 }
 
 // The waves' histograms (lds.running) out to wave_hist, and their sum to block_hist.  Called by all threads.
-template <bool kCoherent>
 __device__ __forceinline__ void publish_histograms(LayoutLds& lds, int num_local, int num_chunks,
                                                    int* __restrict__ wave_hist, int* __restrict__ block_hist)
 {
@@ -118,9 +108,9 @@ __device__ __forceinline__ void publish_histograms(LayoutLds& lds, int num_local
             const int g = blockIdx.x * kWaves + w;
             const int count = lds.running[w][e];
             sum += count;
-            if (g < num_chunks) store_int<kCoherent>(wave_hist + static_cast<size_t>(g) * num_local + e, count);
+            if (g < num_chunks) wave_hist[static_cast<size_t>(g) * num_local + e] = count;
         }
-        store_int<kCoherent>(block_hist + static_cast<size_t>(blockIdx.x) * num_local + e, sum);
+        block_hist[static_cast<size_t>(blockIdx.x) * num_local + e] = sum;
     }
 }
 
@@ -169,7 +159,7 @@ __global__ __launch_bounds__(kThreads) void layout_count_kernel(const IdxT* __re
 #pragma unroll
         for (int i = 0; i < kPrefetch; ++i) count_step(experts[i], lds.running[wave]);
     }
-    publish_histograms<false>(lds, num_local, num_chunks, wave_hist, block_hist);
+    publish_histograms(lds, num_local, num_chunks, wave_hist, block_hist);
 }
 
 // For one expert, over the workgroups {first, first+stride, ...}: the sum of all block_hist rows and of those
@@ -179,7 +169,6 @@ struct ColumnSums {
     int before;
 };
 
-template <bool kCoherent>
 __device__ __forceinline__ ColumnSums column_sums(const int* __restrict__ block_hist, int num_local, int e, int first,
                                                   int stride, int num_blocks)
 {
@@ -189,7 +178,7 @@ __device__ __forceinline__ ColumnSums column_sums(const int* __restrict__ block_
 #pragma unroll
         for (int j = 0; j < kColumnBatch; ++j) {
             const int b = b0 + j * stride;
-            v[j] = b < num_blocks ? load_int<kCoherent>(block_hist + static_cast<size_t>(b) * num_local + e) : 0;
+            v[j] = b < num_blocks ? block_hist[static_cast<size_t>(b) * num_local + e] : 0;
         }
 #pragma unroll
         for (int j = 0; j < kColumnBatch; ++j) {
@@ -200,16 +189,93 @@ __device__ __forceinline__ ColumnSums column_sums(const int* __restrict__ block_
     return sums;
 }
 
+// Words of the one-launch kernel's exchange (see "one launch" below): tag above kCountBits, count below.
+constexpr int kCountBits = 24;
+constexpr unsigned long long kCountMask = (1ull << kCountBits) - 1ull;
+
+__device__ __forceinline__ unsigned long long load_word(const unsigned long long* src)
+{
+    return __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The workgroup's histogram (sum of its waves') out to its row of `tagged`.  Called by all threads, after a workgroup
+// barrier behind the counting.
+__device__ __forceinline__ void publish_tagged(LayoutLds& lds, int num_local, unsigned long long* __restrict__ tagged,
+                                               unsigned long long tag)
+{
+    for (int e = threadIdx.x; e < num_local; e += kThreads) {
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) sum += lds.running[w][e];
+        __hip_atomic_store(tagged + static_cast<size_t>(blockIdx.x) * num_local + e,
+                           (tag << kCountBits) | static_cast<unsigned long long>(sum), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// column_sums over tagged rows {first, first+stride, ...} below `rows`: every word is re-read until it carries `tag`.
+// Sets lds_timed_out and gives up when that takes longer than limit_ticks.
+__device__ __forceinline__ ColumnSums tagged_column_sums(const unsigned long long* __restrict__ tagged, int num_local, int e,
+                                                         int first, int stride, int rows, unsigned long long tag,
+                                                         long long limit_ticks, int* lds_timed_out)
+{
+    ColumnSums sums = {0, 0};
+    long long start = 0;
+    for (int b0 = first; b0 < rows; b0 += kColumnBatch * stride) {
+        unsigned long long v[kColumnBatch];
+        for (int spins = 0;; ++spins) {
+            bool all = true;
+#pragma unroll
+            for (int j = 0; j < kColumnBatch; ++j) {
+                const int b = b0 + j * stride;
+                v[j] = b < rows ? load_word(tagged + static_cast<size_t>(b) * num_local + e) : tag << kCountBits;
+            }
+#pragma unroll
+            for (int j = 0; j < kColumnBatch; ++j) all = all && (v[j] >> kCountBits) == tag;
+            if (all) break;
+            if ((spins & 15) == 15) {
+                const long long now = wall_clock64();
+                if (start == 0) start = now;
+                if (now - start > limit_ticks) {
+                    *lds_timed_out = 1;
+                    return sums;
+                }
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+#pragma unroll
+        for (int j = 0; j < kColumnBatch; ++j) {
+            const int count = static_cast<int>(v[j] & kCountMask);
+            sums.total += count;
+            sums.before += b0 + j * stride < static_cast<int>(blockIdx.x) ? count : 0;
+        }
+    }
+    return sums;
+}
+
+// Where the one-launch kernel's workgroups find each other's histograms.
+struct TaggedSource {
+    const unsigned long long* tagged;
+    unsigned long long tag;
+    int rows;
+    long long limit_ticks;
+    uint32_t* timeouts;  // host mailbox word that receives launch_id when the wait runs out
+    uint32_t launch_id;
+};
+
 // From the histograms to every wave's first row per expert (lds.running).  The launch's last workgroup owns no
 // chunk: it is the reporter, which writes the per-expert outputs and reports to the host, so that the wait for the
 // host stores (a PCIe round trip) delays no workgroup that still has routes to assign.  Called by all threads.
-// num_blocks = workgroups that own chunks.  kCoherent: the histograms were written by other CUs of this launch.
-template <bool kCoherent>
-__device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restrict__ wave_hist,
+// num_blocks = workgroups that own chunks.  kTagged: the one-launch kernel (the workgroup's own wave histograms are
+// still in lds.running, the others' arrive as tagged words from `source`); else the count launch left everything in
+// wave_hist / block_hist.  Returns false if the wait for the tagged words ran out: every count is then reported as zero.
+template <bool kTagged>
+__device__ __forceinline__ bool expert_bases(LayoutLds& lds, const int* __restrict__ wave_hist,
                                              const int* __restrict__ block_hist, int num_local, int padded_local,
                                              int num_chunks, int num_blocks, int* __restrict__ counts,
                                              int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows,
-                                             uint32_t* __restrict__ mailbox, uint32_t sequence, bool valid = true)
+                                             uint32_t* __restrict__ mailbox, uint32_t sequence,
+                                             const TaggedSource* source = nullptr)
 {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const bool reporter = blockIdx.x == gridDim.x - 1;
@@ -218,15 +284,21 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
             const int g = blockIdx.x * kWaves + w;
-            own[w] = g < num_chunks ? load_int<kCoherent>(wave_hist + static_cast<size_t>(g) * num_local + e) : 0;
+            if (kTagged) own[w] = lds.running[w][e];  // (the reporter's are zero: it counted nothing)
+            else own[w] = g < num_chunks ? wave_hist[static_cast<size_t>(g) * num_local + e] : 0;
         }
     };
-    // (valid == false: the histograms cannot be trusted, every count is reported as zero)
+    auto sums_of = [&](int e, int first, int stride) {
+        if (kTagged)
+            return tagged_column_sums(source->tagged, num_local, e, first, stride, source->rows, source->tag,
+                                      source->limit_ticks, &lds.timed_out);
+        return column_sums(block_hist, num_local, e, first, stride, num_blocks);
+    };
     auto finish = [&](int e, int total, int before, const int (&own)[kWaves]) {  // the waves one after the other
-        lds.totals[e] = valid ? total : 0;
+        lds.totals[e] = total;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            lds.running[w][e] = valid ? before : 0;
+            lds.running[w][e] = before;
             before += own[w];
         }
     };
@@ -234,7 +306,7 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
         for (int e = tid; e < num_local; e += kThreads) {
             int own[kWaves];
             own_rows(e, own);
-            const ColumnSums sums = column_sums<kCoherent>(block_hist, num_local, e, 0, 1, num_blocks);
+            const ColumnSums sums = sums_of(e, 0, 1);
             finish(e, sums.total, sums.before, own);
         }
     } else {
@@ -245,7 +317,7 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
         int own[kWaves] = {0, 0, 0, 0};
         if (tid < num_local) own_rows(tid, own);
         if (p < parts && e < num_local) {
-            const ColumnSums sums = column_sums<kCoherent>(block_hist, num_local, e, p, parts, num_blocks);
+            const ColumnSums sums = sums_of(e, p, parts);
             lds.partial[tid * 2] = sums.total;
             lds.partial[tid * 2 + 1] = sums.before;
         }
@@ -260,6 +332,18 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
         }
     }
     __syncthreads();
+    const bool valid = !kTagged || lds.timed_out == 0;
+    if (!valid) {
+        // A histogram is missing: every count is reported as zero, and the host is told (this store is acknowledged
+        // before the reporter publishes the mailbox's sequence word below, so the host never sees one without the other).
+        if (tid == 0) __hip_atomic_store(source->timeouts, source->launch_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        for (int e = tid; e < num_local; e += kThreads) {
+            lds.totals[e] = 0;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) lds.running[w][e] = 0;
+        }
+        __syncthreads();
+    }
 
     // Exclusive scan of totals over experts: four consecutive experts per thread, then a workgroup scan.
     int mine[4], local_sum = 0;
@@ -308,6 +392,7 @@ __device__ __forceinline__ void expert_bases(LayoutLds& lds, const int* __restri
         const unsigned long long word = (static_cast<unsigned long long>(sequence) << 32) | static_cast<uint32_t>(offset);
         __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
+    return valid;
 }
 
 template <typename IdxT>
@@ -337,79 +422,51 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
     }
 }
 
-// Barrier of the one-launch kernel, in device memory, all zero between launches.
-struct GridBarrier {
-    unsigned arrived;
-    unsigned departed;
-};
-
-// All threads call it.  Returns false if the wait ran out (the other workgroups did not all arrive in time).
-// What the workgroups exchange (the histograms) is written and read with device-scope accesses that go past
-// the per-CU and per-XCD caches, so the barrier only has to order them: every thread waits until its own stores are
-// acknowledged before its workgroup's arrival is counted.  Acquire/release fences here would write back and
-// invalidate whole caches, which costs more than the launch this barrier saves.
-__device__ __forceinline__ bool grid_arrive_and_wait(GridBarrier* bar, unsigned needed, long long limit_ticks, int* in_time_flag)
-{
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned seen = __hip_atomic_fetch_add(&bar->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-        const long long start = wall_clock64();
-        bool in_time = true;
-        while (seen < needed) {
-            __builtin_amdgcn_s_sleep(1);
-            if (wall_clock64() - start > limit_ticks) {
-                in_time = false;
-                break;
-            }
-            seen = __hip_atomic_load(&bar->arrived, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        *in_time_flag = in_time;
-    }
-    __syncthreads();
-    return *in_time_flag != 0;
-}
-
-// The last workgroup to leave clears the barrier for the next launch: by then none is waiting on it any more.
-__device__ __forceinline__ void grid_depart(GridBarrier* bar)
-{
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const unsigned left = __hip_atomic_fetch_add(&bar->departed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (left == gridDim.x - 1) {
-            __hip_atomic_store(&bar->arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&bar->departed, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-}
-
-// Count, barrier, assign in one launch; every wave keeps the ids of its chunk (at most kKeep steps) in registers.
-// `needed` is the number of workgroups (the reporter included), `limit_ticks` the bound of the wait (100 MHz ticks).
+// ---- one launch: histograms exchanged as tagged words -------------------------------------------------------------
+// A published histogram entry is one 64-bit word: the launch's tag in the upper kTagBits, the count below.  A reader
+// knows from the word itself whether it belongs to this launch, so there is nothing to wait for but the data, and
+// nothing to clear afterwards.  Tags only grow: a launch uses epoch + 1, where the epoch (device memory) is the highest
+// tag any launch on this workspace has used, read by every workgroup before it publishes and raised with an atomic max
+// when the workgroup ends.  No workgroup can end before every workgroup has read the epoch (it ends only after it has
+// seen everybody's words, which are published after that read), so all workgroups of a launch agree on the tag; a
+// launch that ran out of time may use two tags, and the atomic max still leaves the epoch above both.  Replays of a
+// captured launch therefore get fresh tags without any host involvement.  40 tag bits last 10^12 launches.
+// Count, exchange, assign in one launch; every wave keeps the ids of its chunk (at most kKeep steps) in registers.
+// `rows` = histogram rows to wait for (the workgroups that own chunks; one more in a test that wants the wait to run out),
+// `limit_ticks` the bound of that wait (100 MHz ticks).
 template <typename IdxT>
 __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     const IdxT* __restrict__ idx, int n_routes, int num_experts, int expert_begin, int num_local, int padded_local,
-    int chunk, int num_chunks, int* __restrict__ wave_hist, int* __restrict__ block_hist, int* __restrict__ counts,
-    int* __restrict__ psum, int* __restrict__ offsets, int* __restrict__ num_rows, int* __restrict__ route_to_row,
-    int* __restrict__ row_to_route, uint32_t* __restrict__ mailbox, uint32_t sequence, GridBarrier* __restrict__ bar,
-    unsigned needed, long long limit_ticks, uint32_t* __restrict__ timeouts, uint32_t launch_id)
+    int chunk, int num_chunks, int* __restrict__ counts, int* __restrict__ psum, int* __restrict__ offsets,
+    int* __restrict__ num_rows, int* __restrict__ route_to_row, int* __restrict__ row_to_route,
+    uint32_t* __restrict__ mailbox, uint32_t sequence, unsigned long long* __restrict__ epoch,
+    unsigned long long* __restrict__ tagged, int rows, long long limit_ticks, uint32_t* __restrict__ timeouts,
+    uint32_t launch_id)
 {
     __shared__ LayoutLds lds;
-    __shared__ int in_time_flag;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = blockIdx.x * kWaves + wave;
     const int begin = g < num_chunks ? g * chunk : 0;
     const int end = g < num_chunks ? min(begin + chunk, n_routes) : 0;
+    // One thread reads the epoch for the whole workgroup (asked for together with the ids): every thread must use the
+    // same tag, and the tag must be final before anything this workgroup publishes can be seen.
+    if (threadIdx.x == 0) {
+        lds.tag = load_word(epoch) + 1ull;
+        lds.timed_out = 0;
+    }
     int experts[kKeep];
     fetch_experts(experts, idx, begin, end, n_routes, num_experts, expert_begin, num_local);
     clear_wave_lds(lds, num_local);
 #pragma unroll
     for (int i = 0; i < kKeep; ++i) count_step(experts[i], lds.running[wave]);
-    publish_histograms<true>(lds, num_local, num_chunks, wave_hist, block_hist);
-    const bool in_time = grid_arrive_and_wait(bar, needed, limit_ticks, &in_time_flag);
-    if (!in_time && threadIdx.x == 0)  // this launch's results are not valid
-        __hip_atomic_store(timeouts, launch_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    expert_bases<true>(lds, wave_hist, block_hist, num_local, padded_local, num_chunks, gridDim.x - 1, counts, psum, offsets,
-                       num_rows, mailbox, sequence, in_time);
+    __syncthreads();
+    const unsigned long long tag = lds.tag;
+    // (the reporter owns no chunk and publishes nothing: row gridDim.x - 1 is only ever waited for by a test that wants
+    // the wait to run out)
+    if (blockIdx.x != gridDim.x - 1) publish_tagged(lds, num_local, tagged, tag);
+    const TaggedSource source = {tagged, tag, rows, limit_ticks, timeouts, launch_id};
+    const bool in_time = expert_bases<true>(lds, nullptr, nullptr, num_local, padded_local, num_chunks, gridDim.x - 1, counts,
+                                            psum, offsets, num_rows, mailbox, sequence, &source);
     if (in_time) {
 #pragma unroll
         for (int i = 0; i < kKeep; ++i)
@@ -417,11 +474,11 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
                 assign_step(experts[i], begin + i * kWave + lane, end, lds.match[wave], lds.running[wave], route_to_row,
                             row_to_route);
     } else {
-        // Some workgroup's histogram may be missing or left over from an earlier launch: rows computed from it
-        // could lie anywhere.  No route gets a row (and the counts above are all zero).
+        // Some workgroup's histogram is missing: rows computed without it could lie anywhere.  No route gets a row
+        // (and the counts above are all zero).
         for (int route = begin + lane; route < end; route += kWave) route_to_row[route] = -1;
     }
-    grid_depart(bar);
+    if (threadIdx.x == 0) __hip_atomic_fetch_max(epoch, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 int padded_experts(int num_local)
@@ -493,14 +550,14 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
     const int n_routes = num_tokens * num_topk;
     const size_t need = dpep_layout_workspace_bytes(num_tokens, num_topk, num_local);
     DPEP_REQUIRE(need <= w->bytes, "layout: workspace too small (%zu needed, %zu available)", need, w->bytes);
-    // A one-launch layout whose barrier wait ran out left its number in the mailbox.  If nobody has been told yet
+    // A one-launch layout whose wait for the other workgroups' histograms ran out left its number in the mailbox.  If nobody has been told yet
     // (the launch reported to no host wait: MegaMoE's internal layout), this call is; either way the workspace
     // takes two launches from then on.
     if (const uint32_t timed_out = w->mailbox_host[kMailboxTimeout]; timed_out != w->timeout_seen) {
         w->timeout_seen = timed_out;
         w->layout_one_launch = 0;
-        return fail(DPEP_ERUNTIME, "layout: an earlier layout kernel on this workspace ran out of time at its barrier "
-                                   "between workgroups and reported no rows; layouts on this workspace take two launches from now on");
+        return fail(DPEP_ERUNTIME, "layout: an earlier layout kernel on this workspace ran out of time waiting for the "
+                                   "other workgroups' histograms and reported no rows; layouts on this workspace take two launches from now on");
     }
     w->layout_launches = w->layout_launches == 0xffffffffu ? 1u : w->layout_launches + 1u;  // never 0
     const int padded = padded_experts(num_local);
@@ -515,11 +572,12 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
     }
     uint32_t* mailbox = report_to_host ? w->mailbox_device : nullptr;
     if (blocks > 0 && chunk <= kKeep * kWave && w->layout_one_launch) {
+        char* sync = static_cast<char*>(w->sync);
         hipLaunchKernelGGL(layout_fused_kernel<IdxT>, dim3(blocks + 1), dim3(kThreads), 0, stream, idx, n_routes, num_experts,
-                           expert_begin, num_local, padded, chunk, num_chunks, wave_hist, block_hist, counts, psum, offsets,
-                           num_rows, route_to_row, row_to_route, mailbox, w->sequence,
-                           static_cast<GridBarrier*>(w->barrier), static_cast<unsigned>(blocks + 1 + w->barrier_extra_arrivals),
-                           w->barrier_ticks, w->mailbox_device + kMailboxTimeout, w->layout_launches);
+                           expert_begin, num_local, padded, chunk, num_chunks, counts, psum, offsets, num_rows, route_to_row,
+                           row_to_route, mailbox, w->sequence, reinterpret_cast<unsigned long long*>(sync),
+                           reinterpret_cast<unsigned long long*>(sync + kSyncTagged), blocks + w->exchange_extra_rows,
+                           w->exchange_ticks, w->mailbox_device + kMailboxTimeout, w->layout_launches);
         return launch_status("layout_fused");
     }
     return enqueue_count_and_assign<IdxT>(idx, n_routes, num_experts, expert_begin, num_local, padded, chunk, num_chunks, wave_hist,

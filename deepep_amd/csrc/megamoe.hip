@@ -1162,7 +1162,7 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     // Without shared experts most tokens of a share have no row: workgroups of the first GEMM that get no tile
     // zero those rows of y meanwhile, and the weighted reduce skips what they got through.
     int* fill_state = reinterpret_cast<int*>(base + l.fill_state);
-    int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->barrier) + kSyncFillStop);
+    int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->sync) + kSyncFillStop);
     w->gemm_launches = w->gemm_launches >= 0x7fffffffu ? 1u : w->gemm_launches + 1u;  // never 0
     g1.launch_id = static_cast<int>(w->gemm_launches);
     g1.forced_rt = w->gemm_tile_rows / 64;

@@ -40,9 +40,9 @@ int dpep_workspace_create(size_t bytes, void** ws)
     DPEP_REQUIRE(bytes > 0, "workspace_create: bytes must be positive");
     *ws = nullptr;
     void* base = nullptr;
-    const size_t barrier_at = (bytes + 255) / 256 * 256;  // the layout's barrier words follow the caller's bytes
-    DPEP_HIP(hipMalloc(&base, barrier_at + dpep::kSyncBytes));
-    if (hipError_t cleared = hipMemset(static_cast<char*>(base) + barrier_at, 0, dpep::kSyncBytes); cleared != hipSuccess) {
+    const size_t sync_at = (bytes + 255) / 256 * 256;  // the kernels' synchronisation memory follows the caller's bytes
+    DPEP_HIP(hipMalloc(&base, sync_at + dpep::kSyncBytes));
+    if (hipError_t cleared = hipMemset(static_cast<char*>(base) + sync_at, 0, dpep::kSyncBytes); cleared != hipSuccess) {
         (void)hipFree(base);
         return dpep::fail(DPEP_ERUNTIME, "workspace_create: %s", hipGetErrorString(cleared));
     }
@@ -69,9 +69,9 @@ int dpep_workspace_create(size_t bytes, void** ws)
     w->mailbox_device = static_cast<uint32_t*>(mailbox_device);
     w->sequence = 0;
     w->mailbox_local = 0;
-    w->barrier = static_cast<char*>(base) + barrier_at;
-    w->barrier_ticks = dpep::kLayoutBarrierTicks;
-    w->barrier_extra_arrivals = 0;
+    w->sync = static_cast<char*>(base) + sync_at;
+    w->exchange_ticks = dpep::kLayoutExchangeTicks;
+    w->exchange_extra_rows = 0;
     w->layout_one_launch = 1;
     w->gemm_tile_rows = 0;
     w->gemm_launches = 0;
@@ -120,7 +120,7 @@ int dpep_layout_wait(void* ws, int32_t* counts_host, int num_local, int32_t* num
     if (const uint32_t timed_out = box[dpep::kMailboxTimeout]; timed_out != w->timeout_seen) {
         w->timeout_seen = timed_out;
         w->layout_one_launch = 0;
-        return dpep::fail(DPEP_ERUNTIME, "layout_wait: the layout kernel ran out of time at its barrier between workgroups "
+        return dpep::fail(DPEP_ERUNTIME, "layout_wait: the layout kernel ran out of time waiting for the other workgroups' histograms "
                                          "and reported no rows; layouts on this workspace take two launches from now on");
     }
     *num_rows_host = static_cast<int32_t>(box[0]);
@@ -135,12 +135,12 @@ int dpep_workspace_tune(void* ws, const char* key, long long value)
     DPEP_REQUIRE(w != nullptr && key != nullptr, "workspace_tune: not a live workspace");
     if (strcmp(key, "layout_one_launch") == 0) {
         w->layout_one_launch = value != 0;
-    } else if (strcmp(key, "layout_barrier_ticks") == 0) {
-        DPEP_REQUIRE(value > 0, "workspace_tune: layout_barrier_ticks must be positive");
-        w->barrier_ticks = value;
-    } else if (strcmp(key, "layout_barrier_extra_arrivals") == 0) {
-        DPEP_REQUIRE(value >= 0 && value <= 1, "workspace_tune: layout_barrier_extra_arrivals is 0 or 1");
-        w->barrier_extra_arrivals = static_cast<int>(value);
+    } else if (strcmp(key, "layout_exchange_ticks") == 0) {
+        DPEP_REQUIRE(value > 0, "workspace_tune: layout_exchange_ticks must be positive");
+        w->exchange_ticks = value;
+    } else if (strcmp(key, "layout_exchange_extra_rows") == 0) {
+        DPEP_REQUIRE(value >= 0 && value <= 1, "workspace_tune: layout_exchange_extra_rows is 0 or 1");
+        w->exchange_extra_rows = static_cast<int>(value);
     } else if (strcmp(key, "gemm_zero_fill") == 0) {
         w->gemm_zero_fill = value != 0;
     } else if (strcmp(key, "gemm_tile_rows") == 0) {

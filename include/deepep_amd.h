@@ -41,10 +41,10 @@ int dpep_workspace_destroy(void* ws);
 int dpep_workspace_capacity(void* ws, size_t* bytes);
 /* Switches of a workspace for tests and diagnosis; no counterpart in the reference.  Keys:
  *   "layout_one_launch"             0: dpep_layout always takes two launches (count, assign); 1 (default): one
- *                                   launch with a barrier between its workgroups where the input is small enough
- *   "layout_barrier_ticks"          bound of that barrier's wait in 10 ns ticks (default 2 s)
- *   "layout_barrier_extra_arrivals" 1: the barrier expects one workgroup more than there are, so that its wait
- *                                   runs out (exercises the error path)
+ *                                   launch whose workgroups exchange their histograms, where the input is small enough
+ *   "layout_exchange_ticks"         bound of a workgroup's wait for the others' histograms in 10 ns ticks (default 2 s)
+ *   "layout_exchange_extra_rows"    1: the workgroups wait for one histogram more than there are workgroups, so that
+ *                                   the wait runs out (exercises the error path)
  *   "gemm_zero_fill"                1 (default): workgroups of dpep_megamoe_forward's first GEMM that get no tile zero
  *                                   the output rows of tokens no local expert serves; 0: the weighted reduce writes them
  *   "gemm_tile_rows"                0 (default): dpep_megamoe_forward chooses the row-tile height of its grouped GEMMs

@@ -68,21 +68,21 @@ LAYOUT_SHAPES = [
 @pytest.mark.parametrize("one_launch", [True, False])
 @pytest.mark.parametrize("tokens,topk,experts,begin,local", LAYOUT_SHAPES)
 def test_layout_matches_oracle(ops, ws, tokens, topk, experts, begin, local, one_launch):
-    """Both forms of the layout (one launch with a barrier between workgroups; count and assign launches)."""
+    """Both forms of the layout (one launch whose workgroups exchange histograms; count and assign launches)."""
     rng = np.random.default_rng(tokens * 31 + topk)
     idx = rng.integers(-1, experts + 1, size=(tokens, topk))  # includes -1 and == E (both invalid)
     ws.tune("layout_one_launch", one_launch)
     try:
         _check_layout(ops, ws, idx, experts, begin, local)
-        _check_layout(ops, ws, idx[::-1].copy(), experts, begin, local)  # the barrier is clear again for the next launch
+        _check_layout(ops, ws, idx[::-1].copy(), experts, begin, local)  # the next launch on the workspace gets a tag of its own
     finally:
         ws.tune("layout_one_launch", 1)
 
 
-def test_layout_barrier_wait_that_runs_out_is_reported(ops):
-    """The barrier's wait is bounded: told to expect one workgroup more than the launch has, with a bound of
-    100 us, every workgroup gives up and the kernel ends normally.  Such a launch assigns nothing (its histograms may
-    be stale, so any row computed from them could lie anywhere): every route is left without a row, every count is
+def test_layout_wait_for_histograms_that_runs_out_is_reported(ops):
+    """A workgroup's wait for the others' histograms is bounded: told to wait for one histogram more than the launch
+    has workgroups, with a bound of 100 us, every workgroup gives up and the kernel ends normally.  Such a launch assigns
+    nothing (a histogram is missing, so any row computed without it could lie anywhere): every route is left without a row, every count is
     zero, and the host gets an error instead of results.  The workspace stays usable: later layouts take two launches."""
     workspace = ops.Workspace(1 << 20)
     try:
@@ -90,15 +90,15 @@ def test_layout_barrier_wait_that_runs_out_is_reported(ops):
         want = olayout.layout(idx.cpu().numpy(), 16)
         good = ops.layout(workspace, idx, 16)  # leaves valid histograms of this very input behind
         ops.layout_wait(workspace)
-        workspace.tune("layout_barrier_extra_arrivals", 1)
-        workspace.tune("layout_barrier_ticks", 10_000)
+        workspace.tune("layout_exchange_extra_rows", 1)
+        workspace.tune("layout_exchange_ticks", 10_000)
         lay = ops.layout(workspace, idx, 16)
-        with pytest.raises(RuntimeError, match="barrier"):
+        with pytest.raises(RuntimeError, match="histograms"):
             ops.layout_wait(workspace)
         torch.cuda.synchronize()
         assert (lay["route_to_row"] == -1).all() and not lay["counts"].any() and not lay["psum"].any()
         assert not lay["offsets"].any() and int(lay["num_rows"].item()) == 0
-        workspace.tune("layout_barrier_extra_arrivals", 0)
+        workspace.tune("layout_exchange_extra_rows", 0)
         again = ops.layout(workspace, idx, 16)  # two launches now; the earlier failure has been reported already
         _, rows = ops.layout_wait(workspace)
         assert rows == want["num_rows"]
@@ -116,12 +116,12 @@ def test_layout_timeout_nobody_waited_for_is_reported_by_the_next_call(ops):
     workspace = ops.Workspace(1 << 20)
     try:
         idx = torch.randint(0, 16, (512, 4), device="cuda")
-        workspace.tune("layout_barrier_extra_arrivals", 1)
-        workspace.tune("layout_barrier_ticks", 10_000)
+        workspace.tune("layout_exchange_extra_rows", 1)
+        workspace.tune("layout_exchange_ticks", 10_000)
         ops.layout(workspace, idx, 16)
         torch.cuda.synchronize()
-        workspace.tune("layout_barrier_extra_arrivals", 0)
-        with pytest.raises(RuntimeError, match="barrier"):
+        workspace.tune("layout_exchange_extra_rows", 0)
+        with pytest.raises(RuntimeError, match="histograms"):
             ops.layout(workspace, idx, 16)
         lay = ops.layout(workspace, idx, 16)
         _, rows = ops.layout_wait(workspace)
