@@ -854,14 +854,15 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
         for (int j = 1; j * bm < mean + 6.0 * sigma; ++j) m_tiles += 0.5 * erfc((j * bm - mean) / (sigma * 1.4142135623730951));
         const double tiles = p.num_local * m_tiles * n_tiles;
         const double rounds = ceil(tiles / cus - 0.02);  // a stray tile in one launch out of fifty does not count
-        // Microseconds per tile, fitted to kernel traces on an MI355X over shares from 32 to 512 rows per expert,
-        // 4 to 32 experts and two problem sizes (it reproduced the measured order of the three heights in 14 of 16
-        // cases, and was within 7 % in the other two): a fixed part (prologue, epilogue) plus a part per k tile;
-        // an expert with a single row tile streams its weight tile from HBM with nobody to share it with, which
-        // adds about 0.3 us per k tile whatever the height.
-        constexpr double kFixed[3] = {4.2, 2.9, 7.9}, kPerItem[3] = {0.53, 0.87, 1.29};
+        // Microseconds, fitted to kernel traces on an MI355X over shares from 32 to 2048 rows per expert, 4 to 32
+        // experts and two problem sizes (it reproduced the measured order of the three heights in 14 of 16 small cases,
+        // was within 7 % in the other two, and in the many-round cases of a large batch): once per launch the part of the
+        // first tile that nothing overlaps (the 192-row kernel's three-stage ring starts slowly), per tile its epilogue
+        // and switch, per k tile the main loop; an expert with a single row tile streams its weight tile from HBM with
+        // nobody to share it with, which adds about 0.3 us per k tile whatever the height.
+        constexpr double kFirst[3] = {0.0, 0.0, 4.7}, kPerTile[3] = {4.2, 2.9, 3.2}, kPerItem[3] = {0.53, 0.87, 1.22};
         const double per_item = kPerItem[rt - 1] + (m_tiles <= 1.2 ? 0.3 : 0.0);
-        const double cost = (rounds < 1.0 ? 1.0 : rounds) * (kFixed[rt - 1] + (p.k / kBK) * per_item);
+        const double cost = kFirst[rt - 1] + (rounds < 1.0 ? 1.0 : rounds) * (kPerTile[rt - 1] + (p.k / kBK) * per_item);
         if (cost < best_cost - 1e-9) {
             best_cost = cost;
             best = rt;
