@@ -356,7 +356,7 @@ def test_roundtrip_identity_multiplicity(ops, ws):
 
 
 def test_full_size_prefill_properties(ops, ws):
-    # BASELINE prefill shape (T=4096, H=7168, E=256, K=8, Zipf): checks that do not need the oracle to
+    # the prefill shape at full size (T=4096, H=7168, E=256, K=8, Zipf): checks that do not need the oracle to
     # materialise 470 MB: row checksums of the FP8 payload against the token checksums, and the combine
     # of the dispatched BF16 rows against count * x on integer-valued input.
     x, idx, w, cfg = cases.make_inputs("C3")
