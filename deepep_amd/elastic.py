@@ -12,7 +12,9 @@ tuples and exception types.  What is different, deliberately:
     tables; payload rows are written straight into torch-allocated outputs;
   * ``use_fp8_dispatch=True`` with a BF16 ``x`` quantises per 128 elements inside the dispatch
     kernel and returns ``(fp8, scales)`` (the reference moves pre-quantised tuples only — which this
-    class also accepts).
+    class also accepts);
+  * a synchronous call (``async_with_compute_stream=False``) is queued on the caller's current stream; only
+    asynchronous calls use the communication stream (see ``_Enqueue``).
 """
 
 from __future__ import annotations
@@ -144,6 +146,53 @@ class EPHandle:
         self.num_compute_units = value
 
 
+class _Enqueue:
+    """Where one call's kernels go, and what the caller gets to wait on.
+
+    The reference always launches on its communication stream and, unless ``async_with_compute_stream`` is set, makes
+    the caller's stream wait for it before the call returns (deep_ep/backends/mesh_clos/elastic.py:905-1003).  On one GPU
+    that round trip through a second stream buys nothing for a synchronous call, and its events and stream switches cost
+    more host time than a decode step's kernels take; so a synchronous call is queued on the caller's own current stream
+    (nothing to wait for afterwards, no tensor crosses a stream) and only an asynchronous one goes to the communication
+    stream, behind an event on the caller's stream, and hands back an event that keeps its tensors alive.
+    One buffer's calls share its workspace: a call queued on another stream than the previous one waits for that stream.
+    """
+
+    def __init__(self, runtime, previous_event=None, asynchronous=False):
+        self.runtime, self.previous_event, self.asynchronous = runtime, previous_event, asynchronous
+        self._scope = None
+
+    def __enter__(self):
+        runtime, api = self.runtime, gpu_api()
+        if self.previous_event is not None:
+            self.previous_event.current_stream_wait()
+        if self.asynchronous:
+            producer = EventHandle()
+            self._scope = api.stream(runtime.stream)
+            self._scope.__enter__()
+            producer.current_stream_wait()
+            target = runtime.stream
+        else:
+            target = api.current_stream(runtime.device)
+        last = getattr(runtime, "last_stream", None)
+        if last is not None and last != target:
+            target.wait_stream(last)
+        runtime.last_stream = target
+        return self
+
+    def event(self, retained):
+        """What the call returns as its event; asynchronous calls record it on the communication stream (call inside
+        the ``with`` block)."""
+        if self.asynchronous:
+            return EventOverlap._holding(EventHandle(), retained)
+        return EventOverlap()
+
+    def __exit__(self, *exc):
+        if self._scope is not None:
+            self._scope.__exit__(*exc)
+        return False
+
+
 class _Runtime:
     """Process-local owner of the HBM workspace and the communication stream (the single-GPU
     counterpart of deep_ep/_runtime.py:67-308 without SHMEM bootstrap)."""
@@ -162,6 +211,7 @@ class _Runtime:
         # does); the HBM actually taken is bounded by what the single-GPU kernels use, the layout scratch.
         self.workspace = native.Workspace(min(num_bytes, WORKSPACE_ALLOCATION_CAP), self.torch_device)
         self.stream = gpu_api().Stream(device=self.torch_device)
+        self.last_stream = None  # the stream the buffer's most recent kernels were queued on
         self.closed = False
 
     def ensure_alive(self):
@@ -171,6 +221,8 @@ class _Runtime:
     def close(self):
         if not self.closed:
             self.stream.synchronize()
+            if self.last_stream is not None:
+                self.last_stream.synchronize()
             self.workspace.destroy()
             self.closed = True
             self.notify_inflight = None
@@ -311,12 +363,14 @@ class ElasticBuffer:
         return max(MIN_WORKSPACE_BYTES, (scratch + (2 << 20) - 1) // (2 << 20) * (2 << 20))
 
     def barrier(self, use_comm_stream: bool = True, with_cpu_sync: bool = False, sequential: bool = True) -> None:
-        """Host-synchronous barrier: with one rank it drains the communication stream."""
+        """Host-synchronous barrier: with one rank it drains the streams the buffer's kernels were queued on."""
         if type(use_comm_stream) is not bool or with_cpu_sync is not True or sequential is not True:
             raise NotImplementedError("Only the host-synchronous sequential barrier is implemented")
         runtime = self._live_runtime()
         runtime.ensure_alive()
         runtime.stream.synchronize()
+        if getattr(runtime, "last_stream", None) is not None:
+            runtime.last_stream.synchronize()
 
     @staticmethod
     def capture() -> EventHandle:
@@ -538,13 +592,9 @@ class ElasticBuffer:
                  "topk_weights must be contiguous FP32 [T,K] on the buffer GPU without grad"),
             )
 
-            # ---- launch: everything from here runs on the communication stream --------------
+            # ---- launch -----------------------------------------------------------------------
             try:
-                if previous_event is not None:
-                    previous_event.current_stream_wait()
-                producer = EventHandle()
-                with gpu_api().stream(runtime.stream):
-                    producer.current_stream_wait()
+                with _Enqueue(runtime, previous_event, async_with_compute_stream) as queue:
 
                     def payload(rows):
                         if fuse_quant:
@@ -586,9 +636,7 @@ class ElasticBuffer:
                     handle._routing_versions = {
                         name: (getattr(handle, name).data_ptr(), getattr(handle, name)._version) for name in _ROUTING
                     }
-                    event = EventOverlap._holding(EventHandle(), retained)
-                if not async_with_compute_stream:
-                    event.current_stream_wait(release_handle=True)
+                    event = queue.event(retained)
                 runtime.notify_inflight = None
                 return (out, out_scales) if fp8 else out, None, out_weights, handle, event
             except Exception:
@@ -662,9 +710,7 @@ class ElasticBuffer:
             if runtime.notify_failed:
                 raise RuntimeError("A previous communication launch failed; restart the distributed job")
             try:
-                producer = EventHandle()
-                with gpu_api().stream(runtime.stream):
-                    producer.current_stream_wait()
+                with _Enqueue(runtime) as queue:
                     # The payload kernel does not depend on R.  Batches of up to SMALL_BATCH_ROUTES routes (every
                     # low-latency batch with the usual top-k) take one launch for layout and payload; larger ones
                     # queue the payload kernel right behind the layout.  (Experts repeated within a token are
@@ -700,8 +746,7 @@ class ElasticBuffer:
                     handle.num_tokens, handle.num_topk, handle.hidden = tokens, topk, width
                     retained = (hidden, scales, topk_weights, indices, out, out_scales, row_weights, send_counts,
                                 layout["route_to_row"], layout["row_to_route"], layout["meta"])
-                    event = EventOverlap._holding(EventHandle(), retained)
-                event.current_stream_wait(release_handle=True)
+                    event = queue.event(retained)
                 runtime.notify_inflight = None
                 return (out, out_scales) if scales is not None else out, None, None, handle, event
             except Exception:
@@ -737,13 +782,9 @@ class ElasticBuffer:
             if runtime.notify_failed:
                 raise RuntimeError("A previous communication launch failed; restart the distributed job")
             try:
-                producer = EventHandle()
-                with gpu_api().stream(runtime.stream):
-                    producer.current_stream_wait()
+                with _Enqueue(runtime) as queue:
                     output, _ = runtime.native.combine(x, handle.route_to_row, handle.source_weights, None)
-                    retained = (x, output, handle.route_to_row, handle.source_weights, handle.topk_idx)
-                    event = EventOverlap._holding(EventHandle(), retained)
-                event.current_stream_wait(release_handle=True)
+                    event = queue.event((x, output, handle.route_to_row, handle.source_weights, handle.topk_idx))
                 runtime.notify_inflight = None
                 return output, None, event
             except Exception:
@@ -844,20 +885,13 @@ class ElasticBuffer:
                 (not weighted or handle.source_weights is not None, ValueError, "Low-latency handle carries no saved route weights"),
             )
             try:
-                if previous_event is not None:
-                    previous_event.current_stream_wait()
-                producer = EventHandle()
-                with gpu_api().stream(runtime.stream):
-                    producer.current_stream_wait()
+                with _Enqueue(runtime, previous_event, async_with_compute_stream) as queue:
                     output, output_weights = native.combine(
                         x, handle.route_to_row, handle.source_weights if weighted else None, topk_weights
                     )
-                    retained = (x, topk_weights, output, output_weights, handle.topk_idx) + tuple(
+                    event = queue.event((x, topk_weights, output, output_weights, handle.topk_idx) + tuple(
                         getattr(handle, name) for name in _ROUTING
-                    )
-                    event = EventOverlap._holding(EventHandle(), retained)
-                if not async_with_compute_stream:
-                    event.current_stream_wait(release_handle=True)
+                    ))
                 runtime.notify_inflight = None
                 return output, output_weights, event
             except Exception:
