@@ -127,7 +127,7 @@ class SymmBuffer:
         self._workspace = None
         self._plan_bs = None
         self._closed = False
-        self._stream = torch.cuda.Stream(device=self._device)
+        self._last_stream = None  # the stream the most recent call was queued on
         self.allocate_inputs()
 
     # -- lifetime ----------------------------------------------------------------------------------
@@ -204,7 +204,8 @@ class SymmBuffer:
         with self._lock:
             if self._closed:
                 return
-            self._stream.synchronize()
+            if self._last_stream is not None:
+                self._last_stream.synchronize()
             if self._workspace is not None:
                 self._workspace.destroy()
             self._workspace = self._plan_bs = None
@@ -330,28 +331,27 @@ def _run(x, topk_idx, topk_weights, l1_weights, l2_weights, sym_buffer, *, share
                 raise ValueError("Cumulative stats must not alias inputs, output or timer")
     with b._lock:
         b._ensure_alive()
+        # The call is queued on the caller's current stream (every call is synchronous with it: the reference makes the
+        # caller wait for its own stream before it returns).  Calls of one owner share its workspace, so a call that
+        # arrives on another stream than the previous one waits for that stream first.
         caller = torch.cuda.current_stream(b._device)
-        b._stream.wait_stream(caller)
-        # calls of one owner are serialised on its own stream
-        with torch.cuda.stream(b._stream):
-            b._prepare(bs)
-            if scales is None:
-                data, scales = ops.mx_quant(data.contiguous())  # BF16 override: quantised here, not a BF16 GEMM
-            if scales.dtype != torch.uint8:
-                scales = scales.view(torch.uint8)
-            y = out if out is not None else torch.empty((bs, b.hidden), dtype=torch.bfloat16, device=b._device)
-            counts = torch.empty((b.num_local_experts,), dtype=torch.int32, device=b._device)
-            ops.megamoe_forward(
-                b._workspace, data.contiguous(), scales.contiguous(), topk_idx.contiguous(), topk_weights.contiguous(),
-                w1, s1, w2, s2, b.num_experts, b.group.rank() * b.num_local_experts, b.num_local_experts, y, counts,
-                shared=shared, intermediate=b.intermediate_hidden,
-            )
-            if cumulative_stats is not None:
-                cumulative_stats.add_(counts)
-                cumulative_stats.record_stream(b._stream)
-        caller.wait_stream(b._stream)
-        for tensor in (y, counts):
-            tensor.record_stream(caller)
+        if b._last_stream is not None and b._last_stream != caller:
+            caller.wait_stream(b._last_stream)
+        b._last_stream = caller
+        b._prepare(bs)
+        if scales is None:
+            data, scales = ops.mx_quant(data.contiguous())  # BF16 override: quantised here, not a BF16 GEMM
+        if scales.dtype != torch.uint8:
+            scales = scales.view(torch.uint8)
+        y = out if out is not None else torch.empty((bs, b.hidden), dtype=torch.bfloat16, device=b._device)
+        counts = torch.empty((b.num_local_experts,), dtype=torch.int32, device=b._device)
+        ops.megamoe_forward(
+            b._workspace, data.contiguous(), scales.contiguous(), topk_idx.contiguous(), topk_weights.contiguous(),
+            w1, s1, w2, s2, b.num_experts, b.group.rank() * b.num_local_experts, b.num_local_experts, y, counts,
+            shared=shared, intermediate=b.intermediate_hidden,
+        )
+        if cumulative_stats is not None:
+            cumulative_stats.add_(counts)
         return y, counts
 
 
