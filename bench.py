@@ -342,6 +342,10 @@ def rank_share_kernels(torch, ops, cases, timer):
                    "which `bytes` (the survey's algorithmic figure) leaves out"}),
     }
     entries["combine_weighted"]["GBps_with_zero_fill"] = (combine_bytes + zero_fill) / entries["combine_weighted"]["us"] / 1e3
+    entries["combine_weighted_served_only"] = timer.kernel(
+        lambda: ops.combine(y, r2row, recv_w, out=out, served_only=True), combine_bytes, head_start=True,
+        extra={"note": "rows of unserved tokens are skipped (dpep_combine_served): what the rank does for its share of an EP "
+               "job, where those tokens get their rows from other ranks"})
     ws.destroy()
     return {"workload": f"EP64 rank share: {tokens} candidate tokens, {local} of {experts} experts local, top-{topk} uniform, "
             f"H={hidden}, {rows} rows, {served} served tokens", "kernels": entries}

@@ -35,6 +35,7 @@ SIGNATURES = {
     "dpep_cast_back": (_I, (_P, _P, _I, _I, _I, _P, _P)),
     "dpep_combine": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_combine_fp16": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
+    "dpep_combine_served": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_mx_quant": (_I, (_P, _I, _I, _P, _P, _P)),
     "dpep_megamoe_schedule_check": (_I, (_I, _I, _I, _I, _I)),
     "dpep_megamoe_workspace_bytes": (_Z, (_I, _I, _I, _I, _I, _I)),

@@ -26,7 +26,7 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ row_weights, const int* __restrict__ route_to_row,
     int num_topk, int vec_per_row, int vec_per_part, int parts, u32x4* __restrict__ out,
     const float* __restrict__ return_in, float* __restrict__ return_out, const int* __restrict__ shared_first_row,
-    int num_shared, int num_tokens, const int* __restrict__ fill_state, int num_rows)
+    int num_shared, int num_tokens, const int* __restrict__ fill_state, int num_rows, int leave_unserved)
 {
     __shared__ int rows[DPEP_MAX_TOPK + kBatch];
     __shared__ float wts[DPEP_MAX_TOPK + kBatch];
@@ -54,6 +54,7 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     const int v_begin = part * vec_per_part;
     const int v_end = min(v_begin + vec_per_part, vec_per_row);
     if (!any_row) {
+        if (leave_unserved) return;  // the caller wants only the tokens that own a row written
         // (MegaMoE) rows that idle workgroups of the first GEMM have already zeroed: filler f of n took tokens
         // f, f + n, ... and got through fill_state[1 + f] of them
         if (kWeights == 2 && fill_state != nullptr) {
@@ -101,16 +102,19 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     }
 }
 
-// Route-weighted reduce for sparse shares (most tokens own no row, none owns a shared expert's): one WAVE per
-// token, so that a token without rows costs one short-lived wave instead of a workgroup with a barrier, and four
-// times as many tokens are in flight per CU (the kernel above spends its time on the chain of dependent loads
-// each of its workgroups starts with).  Same arithmetic in the same order as combine_kernel<2>: slots
-// ascending, separate fp32 multiply and add, one RNE rounding to BF16.
+// The reduce for sparse shares (most tokens own no row, none owns a shared expert's): one WAVE per token, so that a
+// token without rows costs one short-lived wave instead of a workgroup with a barrier, and four times as many tokens
+// are in flight per CU (the kernel above spends its time on the chain of dependent loads each of its workgroups
+// starts with).  Same arithmetic in the same order as combine_kernel: slots ascending, separate fp32 multiply and
+// add (no multiply at all without weights), one RNE rounding to BF16.  kWeights as above; kCached: the rows were
+// written by the kernel right before this one (the second GEMM) and are read through the caches.
 constexpr int kSparseBatch = 8;  // 16-byte vectors per lane in flight per slot
 constexpr int kSparseWaves = 4;  // tokens (= waves) per workgroup
+template <int kWeights, bool kCached>
 __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
-    const u32x4* __restrict__ y, const float* __restrict__ route_weights, const int* __restrict__ route_to_row,
-    int num_topk, int vec_per_row, u32x4* __restrict__ out, int num_tokens, const int* __restrict__ fill_state)
+    const u32x4* __restrict__ y, const float* __restrict__ weights, const int* __restrict__ route_to_row, int num_topk,
+    int vec_per_row, u32x4* __restrict__ out, int num_tokens, const int* __restrict__ fill_state,
+    const float* __restrict__ return_in, float* __restrict__ return_out, int num_rows, int leave_unserved)
 {
     const int lane = threadIdx.x & 63;
     const int token = blockIdx.x * kSparseWaves + (threadIdx.x >> 6);
@@ -118,12 +122,17 @@ __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
     int row = -1;
     float weight = 0.0f;
     if (lane < num_topk) {
-        row = route_to_row[static_cast<size_t>(token) * num_topk + lane];
-        weight = route_weights[static_cast<size_t>(token) * num_topk + lane];
+        const size_t route = static_cast<size_t>(token) * num_topk + lane;
+        row = route_to_row[route];
+        if (row >= num_rows) row = -1;  // a row the caller's y does not hold
+        if (kWeights == 1) weight = row >= 0 ? weights[row] : 0.0f;
+        if (kWeights == 2) weight = weights[route];
+        if (return_out != nullptr) return_out[route] = row >= 0 ? return_in[row] : 0.0f;
     }
     const uint64_t valid = __ballot(row >= 0);
     u32x4* dst = out + static_cast<size_t>(token) * vec_per_row;
     if (valid == 0ull) {
+        if (leave_unserved) return;
         if (fill_state != nullptr) {  // rows that idle workgroups of the first GEMM have already zeroed
             const int fillers = fill_state[0];
             if (fillers > 0 && token / fillers < fill_state[1 + token % fillers]) return;
@@ -147,15 +156,19 @@ __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
 #pragma unroll
             for (int b = 0; b < kSparseBatch; ++b) {
                 const int v = v0 + b * 64 + lane;
-                if (v < vec_per_row) val[b] = load16(src + v);  // rows the second GEMM has just written: cached
+                if (v < vec_per_row) val[b] = kCached ? load16(src + v) : load16_nt(src + v);
             }
 #pragma unroll
             for (int b = 0; b < kSparseBatch; ++b) {
                 if (v0 + b * 64 + lane >= vec_per_row) continue;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float lo = __fmul_rn(bf16_to_f32(val[b][i] & 0xffffu), w);
-                    const float hi = __fmul_rn(bf16_to_f32(val[b][i] >> 16), w);
+                    float lo = bf16_to_f32(val[b][i] & 0xffffu);
+                    float hi = bf16_to_f32(val[b][i] >> 16);
+                    if (kWeights != 0) {
+                        lo = __fmul_rn(lo, w);
+                        hi = __fmul_rn(hi, w);
+                    }
                     acc[b][2 * i] = __fadd_rn(acc[b][2 * i], lo);
                     acc[b][2 * i + 1] = __fadd_rn(acc[b][2 * i + 1], hi);
                 }
@@ -199,11 +212,11 @@ template <int kWeights, bool kHalf = false>
 void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, const float* weights, const int32_t* route_to_row,
                     int num_topk, int vec, void* out, const float* return_in, float* return_out,
                     int num_rows, const int32_t* shared_first_row = nullptr, int num_shared = 0, int num_tokens = 0,
-                    const int32_t* fill_state = nullptr)
+                    const int32_t* fill_state = nullptr, int leave_unserved = 0)
 {
     hipLaunchKernelGGL((combine_kernel<kWeights, kHalf>), dim3(g.blocks), dim3(g.threads), 0, stream, static_cast<const u32x4*>(y),
                        weights, route_to_row, num_topk, vec, g.per_part, g.parts, static_cast<u32x4*>(out), return_in,
-                       return_out, shared_first_row, num_shared, num_tokens, fill_state, num_rows);
+                       return_out, shared_first_row, num_shared, num_tokens, fill_state, num_rows, leave_unserved);
 }
 
 }  // namespace
@@ -215,9 +228,9 @@ int combine_routes(const void* y, const float* route_weights, const int32_t* rou
 {
     const int vec = hidden / 8;
     if (num_shared == 0 && 2LL * num_rows_hint < num_tokens) {  // a sparse share: most tokens own no row
-        hipLaunchKernelGGL(combine_sparse_kernel, dim3((num_tokens + kSparseWaves - 1) / kSparseWaves), dim3(64 * kSparseWaves), 0, stream,
-                           static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk, vec, static_cast<u32x4*>(out),
-                           num_tokens, fill_state);
+        hipLaunchKernelGGL((combine_sparse_kernel<2, true>), dim3((num_tokens + kSparseWaves - 1) / kSparseWaves),
+                           dim3(64 * kSparseWaves), 0, stream, static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk,
+                           vec, static_cast<u32x4*>(out), num_tokens, fill_state, nullptr, nullptr, 0x7fffffff, 0);
         return launch_status("combine_routes_sparse");
     }
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
@@ -233,7 +246,8 @@ namespace {
 
 template <bool kHalf>
 int combine_entry(const char* what, const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens,
-                  int num_topk, int num_rows, int hidden, void* out, const float* return_in, float* return_out, void* stream)
+                  int num_topk, int num_rows, int hidden, void* out, const float* return_in, float* return_out, void* stream,
+                  int leave_unserved = 0)
 {
     DPEP_REQUIRE(num_tokens >= 0 && num_topk >= 1 && num_topk <= DPEP_MAX_TOPK, "%s: bad T=%d K=%d", what, num_tokens,
                  num_topk);
@@ -248,12 +262,28 @@ int combine_entry(const char* what, const void* y, const float* row_weights, con
     DPEP_REQUIRE(route_to_row != nullptr && out != nullptr && aligned16(out), "%s: NULL or misaligned buffer", what);
     DPEP_REQUIRE(num_rows == 0 || (y != nullptr && aligned16(y)), "%s: y must be 16-byte aligned", what);
     const int vec = hidden / 8;
-    const CombineGrid g = combine_grid(num_tokens, num_rows, vec);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (!kHalf && leave_unserved && 2LL * num_rows < num_tokens) {
+        // a sparse share whose unserved tokens are skipped: a wave per token (with the zero rows to write as well, the
+        // workgroup-per-part kernel below measured faster: 53 against 56 us at 16384 tokens of which 2000 own rows)
+        const dim3 grid((num_tokens + kSparseWaves - 1) / kSparseWaves), block(64 * kSparseWaves);
+        if (row_weights != nullptr)
+            hipLaunchKernelGGL((combine_sparse_kernel<1, false>), grid, block, 0, s, static_cast<const u32x4*>(y), row_weights,
+                               route_to_row, num_topk, vec, static_cast<u32x4*>(out), num_tokens, nullptr, return_in, return_out,
+                               num_rows, 1);
+        else
+            hipLaunchKernelGGL((combine_sparse_kernel<0, false>), grid, block, 0, s, static_cast<const u32x4*>(y), nullptr,
+                               route_to_row, num_topk, vec, static_cast<u32x4*>(out), num_tokens, nullptr, return_in, return_out,
+                               num_rows, 1);
+        return launch_status(what);
+    }
+    const CombineGrid g = combine_grid(num_tokens, num_rows, vec);
     if (row_weights != nullptr)
-        launch_combine<1, kHalf>(g, s, y, row_weights, route_to_row, num_topk, vec, out, return_in, return_out, num_rows);
+        launch_combine<1, kHalf>(g, s, y, row_weights, route_to_row, num_topk, vec, out, return_in, return_out, num_rows, nullptr, 0,
+                                 0, nullptr, leave_unserved);
     else
-        launch_combine<0, kHalf>(g, s, y, nullptr, route_to_row, num_topk, vec, out, return_in, return_out, num_rows);
+        launch_combine<0, kHalf>(g, s, y, nullptr, route_to_row, num_topk, vec, out, return_in, return_out, num_rows, nullptr, 0, 0,
+                                 nullptr, leave_unserved);
     return launch_status(what);
 }
 
@@ -267,6 +297,13 @@ int dpep_combine(const void* y, const float* row_weights, const int32_t* route_t
 {
     return dpep::combine_entry<false>("combine", y, row_weights, route_to_row, num_tokens, num_topk, num_rows, hidden, out,
                                       return_in, return_out, stream);
+}
+
+int dpep_combine_served(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
+                        int num_rows, int hidden, void* out, const float* return_in, float* return_out, void* stream)
+{
+    return dpep::combine_entry<false>("combine_served", y, row_weights, route_to_row, num_tokens, num_topk, num_rows, hidden,
+                                      out, return_in, return_out, stream, /*leave_unserved=*/1);
 }
 
 int dpep_combine_fp16(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens, int num_topk,

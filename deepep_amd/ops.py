@@ -335,9 +335,10 @@ def cast_back(codes, scales):
     return out
 
 
-def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
+def combine(y, route_to_row, row_weights=None, return_values=None, out=None, served_only=False):
     """out[t] = round( sum_s fp32(y[row(t,s)]) (* row_weights[row]) ) in y's dtype (BF16 or FP16); optional
-    weight-return channel."""
+    weight-return channel.  ``served_only`` (BF16, needs ``out``): tokens without any row keep what ``out`` held instead
+    of being zero-filled (one rank's share of an EP job produces nothing for the tokens it does not serve)."""
     lib = _lib.load()
     if not isinstance(y, torch.Tensor) or y.dtype not in (torch.bfloat16, torch.float16):
         raise ValueError("y must be a BF16 or FP16 tensor")
@@ -359,10 +360,16 @@ def combine(y, route_to_row, row_weights=None, return_values=None, out=None):
         _require("return_values", return_values, torch.float32, (rows,), dev)
         returned = torch.empty((tokens, topk), dtype=torch.float32, device=dev)
     if out is None:
+        if served_only:
+            raise ValueError("served_only needs the caller's out (rows of unserved tokens are left as they are)")
         out = torch.empty((tokens, hidden), dtype=y.dtype, device=dev)
     else:
         _require("out", out, y.dtype, (tokens, hidden), dev)
     entry = lib.dpep_combine if y.dtype == torch.bfloat16 else lib.dpep_combine_fp16
+    if served_only:
+        if y.dtype != torch.bfloat16:
+            raise ValueError("served_only is available for BF16 rows")
+        entry = lib.dpep_combine_served
     with _on_device(dev):
         status = entry(
             _ptr(y), _ptr(row_weights), _ptr(route_to_row), tokens, topk, rows, hidden, _ptr(out),

@@ -157,6 +157,14 @@ int dpep_combine(const void* y, const float* row_weights, const int32_t* route_t
                  int num_topk, int num_rows, int hidden, void* out, const float* return_in,
                  float* return_out, void* stream);
 
+/* dpep_combine that writes only the tokens that own at least one row and leaves the others' rows of `out` untouched.
+ * For one rank's receive share of an EP job most candidate tokens own no row here, and in the reference nothing is
+ * produced for them on this rank at all (a rank returns rows only for the routes it served,
+ * csrc/kernels/combine/combine.cpp:2965); dpep_combine zero-fills them, which is what a single-rank caller needs. */
+int dpep_combine_served(const void* y, const float* row_weights, const int32_t* route_to_row, int num_tokens,
+                        int num_topk, int num_rows, int hidden, void* out, const float* return_in,
+                        float* return_out, void* stream);
+
 /* The same combine for IEEE half rows and output (the low-latency path accepts BF16 or FP16 expert outputs and
  * returns the same dtype: deep_ep/backends/mesh_clos/elastic.py:596-606; oracle expected_combine,
  * tests/elastic/test_ep_low_latency.py:449-463): fp32 accumulation in slot order, one RNE rounding to half. */

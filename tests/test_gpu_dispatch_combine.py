@@ -605,3 +605,25 @@ def test_decode_step_in_hip_graph(ops):
     finally:
         torch.cuda.synchronize()
         workspace.destroy()
+
+
+@pytest.mark.parametrize("weighted", [False, True])
+def test_combine_served_only_leaves_unserved_tokens_untouched(ops, ws, weighted):
+    """One rank's share: tokens without a local route keep what the output held (the reference produces nothing for them
+    on this rank), tokens with one get exactly what the zero-filling combine gives them."""
+    x, idx, w, cfg = cases.make_inputs("C4", tokens=3000)
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    gen = torch.Generator().manual_seed(9)
+    y = torch.randn(rows, cfg["hidden"], generator=gen).bfloat16().cuda()
+    row_w = torch.rand(rows, generator=gen).cuda() if weighted else None
+    back = torch.rand(rows, generator=gen).cuda()
+    full, full_back = ops.combine(y, got["route_to_row"], row_w, back)
+    sentinel = torch.full((idx.shape[0], cfg["hidden"]), 7.0, dtype=torch.bfloat16, device="cuda")
+    part, part_back = ops.combine(y, got["route_to_row"], row_w, back, out=sentinel.clone(), served_only=True)
+    served = torch.from_numpy((want["route_to_row"] >= 0).any(axis=1)).cuda()
+    assert 0 < int(served.sum()) < idx.shape[0]
+    assert torch.equal(part[served].view(torch.int16), full[served].view(torch.int16))
+    assert torch.equal(part[~served], sentinel[~served]) and not full[~served].any()
+    assert torch.equal(part_back, full_back)
+    with pytest.raises(ValueError, match="served_only"):
+        ops.combine(y, got["route_to_row"], row_w, served_only=True)
