@@ -219,7 +219,7 @@ def megamoe_cpu_baseline(hidden, inter):
     )
 
 
-def megamoe_shape(torch, ops, timer, tokens, experts, local, topk, weight_sets, hidden=7168, inter=2048):
+def megamoe_shape(torch, ops, timer, tokens, experts, local, topk, weight_sets, hidden=7168, inter=2048, served_only=False):
     """One W4A8 forward shape: (back-to-back us, flushed statistics, rows that reach a local expert, FLOPs).  Random codes
     and constant scale bytes: the time does not depend on the values.  FLOPs = 2*R*H*2I + 2*R*I*H for the R rows."""
     dev = "cuda"
@@ -236,6 +236,7 @@ def megamoe_shape(torch, ops, timer, tokens, experts, local, topk, weight_sets, 
         s2 = torch.full((local, hidden, ops.megamoe_prepared_shape(hidden, inter, False)[2]), 119, dtype=torch.uint8, device=dev)
         sets.append((w1, s1, w2, s2))
     ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local))
+    ws.tune("megamoe_served_only", int(served_only))
     y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
     counts = torch.empty((local,), dtype=torch.int32, device=dev)
     calls = [0]
@@ -273,6 +274,13 @@ def megamoe_bench(torch, ops, timer, with_cpu):
         "roofline": {"bound": "mfma", "achieved": flops / us / 1e6, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
                      "note": "whole forward (4 launches), back to back; per-kernel GEMM times are in profiles/"},
+    }
+    us, cold, rows, flops = megamoe_shape(torch, ops, timer, 64 * 256, 384, 6, 8, weight_sets=3, served_only=True)
+    result["served_only"] = {
+        "workload": "the same rank share with the rows of y left untouched whose token no local expert serves (what the rank "
+        "owes an EP job: other ranks produce those rows); nothing is zero-filled, by the GEMM's idle workgroups or the reduce",
+        "rows": rows, "us_forward": us, "flushed_us": cold, "tflops_forward": flops / us / 1e6,
+        "frac_of_fp8_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
     }
     big = Timer(torch, max(1, timer.iters // 5), max(1, timer.warmups // 5))
     big.flush, big.cycles_per_us = timer.flush, timer.cycles_per_us

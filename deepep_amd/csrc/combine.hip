@@ -224,18 +224,18 @@ void launch_combine(const CombineGrid& g, hipStream_t stream, const void* y, con
 // Route-weighted reduce used by the MegaMoE forward: out[t] = bf16( sum_s w[t,s] * float(y[row(t,s)]) ).
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
                    int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
-                   const int32_t* fill_state, hipStream_t stream)
+                   const int32_t* fill_state, int leave_unserved, hipStream_t stream)
 {
     const int vec = hidden / 8;
     if (num_shared == 0 && 2LL * num_rows_hint < num_tokens) {  // a sparse share: most tokens own no row
         hipLaunchKernelGGL((combine_sparse_kernel<2, true>), dim3((num_tokens + kSparseWaves - 1) / kSparseWaves),
                            dim3(64 * kSparseWaves), 0, stream, static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk,
-                           vec, static_cast<u32x4*>(out), num_tokens, fill_state, nullptr, nullptr, 0x7fffffff, 0);
+                           vec, static_cast<u32x4*>(out), num_tokens, fill_state, nullptr, nullptr, 0x7fffffff, leave_unserved);
         return launch_status("combine_routes_sparse");
     }
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
     launch_combine<2>(g, stream, y, route_weights, route_to_row, num_topk, vec, out, nullptr, nullptr, 0x7fffffff,
-                      shared_first_row, num_shared, num_tokens, fill_state);
+                      shared_first_row, num_shared, num_tokens, fill_state, leave_unserved);
     return launch_status("combine_routes");
 }
 

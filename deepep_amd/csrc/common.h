@@ -53,6 +53,7 @@ struct Workspace {
     uint32_t timeout_seen;     // number of the last timed-out launch the host has been told about
     uint32_t gemm_launches;    // number of the most recent MegaMoE forward (never 0)
     int gemm_zero_fill;        // 1 (default): idle workgroups of the first GEMM zero rows of unserved tokens; 0: the reduce does
+    int megamoe_served_only;   // 1: rows of y whose token no local expert serves are left untouched; 0 (default): zeroed
     int gemm_tile_rows;  // 0: the grouped GEMM chooses its tile height; 64 / 128 / 192: forced (tests)
 };
 // Device memory the kernels synchronise through, behind the caller's bytes, zero when the workspace is created:

@@ -23,7 +23,7 @@ int layout_i32(void* ws, const int32_t* idx, int num_tokens, int num_topk, int n
                int32_t* row_to_route, int32_t* num_rows, hipStream_t stream);
 int combine_routes(const void* y, const float* route_weights, const int32_t* route_to_row, int num_tokens, int num_topk,
                    int num_rows_hint, int hidden, void* out, const int32_t* shared_first_row, int num_shared,
-                   const int32_t* fill_state, hipStream_t stream);
+                   const int32_t* fill_state, int leave_unserved, hipStream_t stream);
 
 namespace {
 
@@ -1167,7 +1167,10 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     w->gemm_launches = w->gemm_launches >= 0x7fffffffu ? 1u : w->gemm_launches + 1u;  // never 0
     g1.launch_id = static_cast<int>(w->gemm_launches);
     g1.forced_rt = w->gemm_tile_rows / 64;
-    const bool fill = num_shared == 0 && w->gemm_zero_fill;
+    // (served-only: rows of y whose token no local expert serves are nobody's business, neither the fillers' nor the
+    // reduce's; with shared experts every token is served)
+    const bool served_only = num_shared == 0 && w->megamoe_served_only;
+    const bool fill = num_shared == 0 && w->gemm_zero_fill && !served_only;
     if (fill) {
         g1.fill_out = static_cast<u32x4*>(y);
         g1.fill_route_to_row = route_to_row;
@@ -1198,7 +1201,8 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     if (int rc = launch_gemm2(g2, per_expert, s)) return rc;
     return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,
                           static_cast<int>(expected_rows),
-                          hidden, y, num_shared > 0 ? num_rows : nullptr, num_shared, fill ? fill_state : nullptr, s);
+                          hidden, y, num_shared > 0 ? num_rows : nullptr, num_shared, fill ? fill_state : nullptr,
+                          served_only ? 1 : 0, s);
 }
 
 }  // extern "C"

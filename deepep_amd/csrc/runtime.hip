@@ -76,6 +76,7 @@ int dpep_workspace_create(size_t bytes, void** ws)
     w->gemm_tile_rows = 0;
     w->gemm_launches = 0;
     w->gemm_zero_fill = 1;
+    w->megamoe_served_only = 0;
     w->layout_launches = 0;
     w->timeout_seen = 0;
     *ws = w;
@@ -143,6 +144,8 @@ int dpep_workspace_tune(void* ws, const char* key, long long value)
         w->exchange_extra_rows = static_cast<int>(value);
     } else if (strcmp(key, "gemm_zero_fill") == 0) {
         w->gemm_zero_fill = value != 0;
+    } else if (strcmp(key, "megamoe_served_only") == 0) {
+        w->megamoe_served_only = value != 0;
     } else if (strcmp(key, "gemm_tile_rows") == 0) {
         DPEP_REQUIRE(value == 0 || value == 64 || value == 128 || value == 192,
                      "workspace_tune: gemm_tile_rows is 0 (automatic), 64, 128 or 192");

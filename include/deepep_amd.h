@@ -47,6 +47,9 @@ int dpep_workspace_capacity(void* ws, size_t* bytes);
  *                                   the wait runs out (exercises the error path)
  *   "gemm_zero_fill"                1 (default): workgroups of dpep_megamoe_forward's first GEMM that get no tile zero
  *                                   the output rows of tokens no local expert serves; 0: the weighted reduce writes them
+ *   "megamoe_served_only"           1: dpep_megamoe_forward leaves the rows of y whose token no local expert serves
+ *                                   untouched (one rank's share of an EP job, where other ranks produce those rows);
+ *                                   0 (default): they are zeroed
  *   "gemm_tile_rows"                0 (default): dpep_megamoe_forward chooses the row-tile height of its grouped GEMMs
  *                                   from the expected rows per expert; 64, 128 or 192: that height for both */
 int dpep_workspace_tune(void* ws, const char* key, long long value);

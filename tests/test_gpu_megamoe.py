@@ -530,3 +530,30 @@ def test_forward_is_reproducible_whoever_zeroes_which_row(ops):
                 assert torch.equal(y.view(torch.int16), first.view(torch.int16))
     finally:
         workspace.destroy()
+
+
+def test_forward_served_only_leaves_unserved_rows_untouched(ops):
+    """One rank's share with `megamoe_served_only`: rows of y whose token no local expert serves keep what they held
+    (other ranks produce them in an EP job), served rows are bit for bit those of the zero-filling forward."""
+    tokens, hidden, inter, experts, begin, local, topk = 900, 512, 512, 64, 8, 4, 2
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=4)
+    dev = "cuda"
+    w1, s1 = ops.megamoe_prepare_weights(torch.from_numpy(l1[0]).to(dev), torch.from_numpy(l1[1]).reshape(local, 2 * inter, -1).to(dev), True)
+    w2, s2 = ops.megamoe_prepare_weights(torch.from_numpy(l2[0]).to(dev), torch.from_numpy(l2[1]).reshape(local, hidden, -1).to(dev), False)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local))
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+    args = (torch.from_numpy(x_codes).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(x_scales).to(dev),
+            torch.from_numpy(idx).to(dev), torch.from_numpy(weights).to(dev), w1, s1, w2, s2, experts, begin, local)
+    try:
+        full = torch.full((tokens, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.megamoe_forward(ws, *args, full, counts)
+        ws.tune("megamoe_served_only", 1)
+        part = torch.full((tokens, hidden), 5.0, dtype=torch.bfloat16, device=dev)
+        ops.megamoe_forward(ws, *args, part, counts)
+        torch.cuda.synchronize()
+        served = torch.from_numpy(((idx >= begin) & (idx < begin + local)).any(axis=1)).to(dev)
+        assert 0 < int(served.sum()) < tokens
+        assert torch.equal(part[served].view(torch.int16), full[served].view(torch.int16))
+        assert (part[~served] == 5.0).all() and not full[~served].any()
+    finally:
+        ws.destroy()
