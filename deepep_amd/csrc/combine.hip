@@ -102,19 +102,70 @@ __global__ __launch_bounds__(kMaxThreads) void combine_kernel(
     }
 }
 
+// One wave reduces the 16-byte vectors [vec_begin, vec_end) of one token: lane s holds the row and weight of the
+// token's slot s (row < 0: no row), valid = the lanes that hold a row; rows are row_stride vectors apart.  Slots ascending, separate fp32 multiply and add, one
+// rounding to BF16.  kSparseBatch = 16-byte vectors per lane in flight per slot.
+template <int kWeights, bool kCached, int kSparseBatch>
+__device__ __forceinline__ void reduce_token_rows(const u32x4* __restrict__ y, int row, float weight, uint64_t valid,
+                                                  int row_stride, int vec_begin, int vec_end, u32x4* __restrict__ dst, int lane)
+{
+    for (int v0 = vec_begin; v0 < vec_end; v0 += 64 * kSparseBatch) {
+        float acc[kSparseBatch][8];
+#pragma unroll
+        for (int b = 0; b < kSparseBatch; ++b)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[b][i] = 0.0f;
+        for (uint64_t rest = valid; rest != 0ull; rest &= rest - 1ull) {
+            const int slot = __builtin_ctzll(rest);
+            const int r = __builtin_amdgcn_readlane(row, slot);
+            const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight), slot));
+            const u32x4* src = y + static_cast<size_t>(r) * row_stride;
+            u32x4 val[kSparseBatch];
+#pragma unroll
+            for (int b = 0; b < kSparseBatch; ++b) {
+                const int v = v0 + b * 64 + lane;
+                if (v < vec_end) val[b] = kCached ? load16(src + v) : load16_nt(src + v);
+            }
+#pragma unroll
+            for (int b = 0; b < kSparseBatch; ++b) {
+                if (v0 + b * 64 + lane >= vec_end) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float lo = bf16_to_f32(val[b][i] & 0xffffu);
+                    float hi = bf16_to_f32(val[b][i] >> 16);
+                    if (kWeights != 0) {
+                        lo = __fmul_rn(lo, w);
+                        hi = __fmul_rn(hi, w);
+                    }
+                    acc[b][2 * i] = __fadd_rn(acc[b][2 * i], lo);
+                    acc[b][2 * i + 1] = __fadd_rn(acc[b][2 * i + 1], hi);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < kSparseBatch; ++b) {
+            const int v = v0 + b * 64 + lane;
+            if (v >= vec_end) continue;
+            u32x4 packed;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) packed[i] = pack_bf16x2(acc[b][2 * i], acc[b][2 * i + 1]);
+            store16_nt(dst + v, packed);
+        }
+    }
+}
+
 // The reduce for sparse shares (most tokens own no row, none owns a shared expert's): one WAVE per token, so that a
 // token without rows costs one short-lived wave instead of a workgroup with a barrier, and four times as many tokens
 // are in flight per CU (the kernel above spends its time on the chain of dependent loads each of its workgroups
 // starts with).  Same arithmetic in the same order as combine_kernel: slots ascending, separate fp32 multiply and
 // add (no multiply at all without weights), one RNE rounding to BF16.  kWeights as above; kCached: the rows were
 // written by the kernel right before this one (the second GEMM) and are read through the caches.
-constexpr int kSparseBatch = 8;  // 16-byte vectors per lane in flight per slot
 constexpr int kSparseWaves = 4;  // tokens (= waves) per workgroup
 template <int kWeights, bool kCached>
 __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
     const u32x4* __restrict__ y, const float* __restrict__ weights, const int* __restrict__ route_to_row, int num_topk,
     int vec_per_row, u32x4* __restrict__ out, int num_tokens, const int* __restrict__ fill_state,
-    const float* __restrict__ return_in, float* __restrict__ return_out, int num_rows, int leave_unserved)
+    const float* __restrict__ return_in, float* __restrict__ return_out, int num_rows)
 {
     const int lane = threadIdx.x & 63;
     const int token = blockIdx.x * kSparseWaves + (threadIdx.x >> 6);
@@ -132,7 +183,6 @@ __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
     const uint64_t valid = __ballot(row >= 0);
     u32x4* dst = out + static_cast<size_t>(token) * vec_per_row;
     if (valid == 0ull) {
-        if (leave_unserved) return;
         if (fill_state != nullptr) {  // rows that idle workgroups of the first GEMM have already zeroed
             const int fillers = fill_state[0];
             if (fillers > 0 && token / fillers < fill_state[1 + token % fillers]) return;
@@ -141,30 +191,70 @@ __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
         for (int v = lane; v < vec_per_row; v += 64) store16_nt(dst + v, zero);
         return;
     }
-    for (int v0 = 0; v0 < vec_per_row; v0 += 64 * kSparseBatch) {
-        float acc[kSparseBatch][8];
+    reduce_token_rows<kWeights, kCached, 8>(y, row, weight, valid, vec_per_row, 0, vec_per_row, dst, lane);
+}
+
+// Sparse shares whose unserved tokens are left alone (one rank's part of an EP job: the rows of tokens it does not
+// serve belong to other ranks).  A workgroup takes 64 / top-k consecutive tokens: every wave loads their (at most 64)
+// routes itself, one per lane, so that the tokens without a row (most of them) cost a lane of one load instead of a wave
+// each, and nothing goes through LDS or a barrier.  The four waves share every row, a quarter of its vectors each, and walk
+// the block's rows (set bits of the ballot, i.e. tokens ascending, slots ascending) with the loads of the next row in
+// flight while the current one is accumulated: a workgroup with several rows pays one memory round trip, not one per row.
+// Same arithmetic as combine_kernel: slots ascending, separate fp32 multiply and add, one rounding to BF16.
+constexpr int kServedWaves = 4;
+constexpr int kServedBatch = 4;  // 16-byte vectors per lane and row in flight
+template <int kWeights, bool kCached>
+__global__ __launch_bounds__(64 * kServedWaves) void combine_served_kernel(
+    const u32x4* __restrict__ y, const float* __restrict__ weights, const int* __restrict__ route_to_row, int num_topk,
+    int tokens_per_block, int vec_per_row, u32x4* __restrict__ out, int num_tokens, const float* __restrict__ return_in,
+    float* __restrict__ return_out, int num_rows)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int token0 = blockIdx.x * tokens_per_block;
+    const int tokens = min(tokens_per_block, num_tokens - token0);
+    int row = -1;
+    float weight = 0.0f;
+    if (lane < tokens * num_topk) {
+        const size_t route = static_cast<size_t>(token0) * num_topk + lane;
+        row = route_to_row[route];
+        if (row >= num_rows) row = -1;  // a row the caller's y does not hold
+        if (kWeights == 1) weight = row >= 0 ? weights[row] : 0.0f;
+        if (kWeights == 2) weight = weights[route];
+        if (return_out != nullptr && wave == 0) return_out[route] = row >= 0 ? return_in[row] : 0.0f;
+    }
+    const uint64_t valid = __ballot(row >= 0);
+    if (valid == 0ull) return;
+    const int token_of_lane = lane / num_topk;
+    const int quarter = (vec_per_row + kServedWaves - 1) / kServedWaves;
+    const int vec_begin = wave * quarter, vec_end = min(vec_begin + quarter, vec_per_row);
+    for (int v0 = vec_begin; v0 < vec_end; v0 += 64 * kServedBatch) {
+        u32x4 buffer[2][kServedBatch];
+        float acc[kServedBatch][8];
+        auto clear = [&]() {
 #pragma unroll
-        for (int b = 0; b < kSparseBatch; ++b)
+            for (int b = 0; b < kServedBatch; ++b)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[b][i] = 0.0f;
-        for (uint64_t rest = valid; rest != 0ull; rest &= rest - 1ull) {
-            const int slot = __builtin_ctzll(rest);
-            const int r = __builtin_amdgcn_readlane(row, slot);
-            const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight), slot));
-            const u32x4* src = y + static_cast<size_t>(r) * vec_per_row;
-            u32x4 val[kSparseBatch];
+                for (int i = 0; i < 8; ++i) acc[b][i] = 0.0f;
+        };
+        auto issue = [&](u32x4 (&into)[kServedBatch], int at) {
+            const u32x4* src = y + static_cast<size_t>(__builtin_amdgcn_readlane(row, at)) * vec_per_row;
 #pragma unroll
-            for (int b = 0; b < kSparseBatch; ++b) {
+            for (int b = 0; b < kServedBatch; ++b) {
                 const int v = v0 + b * 64 + lane;
-                if (v < vec_per_row) val[b] = kCached ? load16(src + v) : load16_nt(src + v);
+                if (v < vec_end) into[b] = kCached ? load16(src + v) : load16_nt(src + v);
             }
+        };
+        // accumulates the row of lane `at`; stores the token when `next` (-1: none) belongs to another one
+        auto consume = [&](const u32x4 (&from)[kServedBatch], int at, int next) {
+            const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, weight), at));
 #pragma unroll
-            for (int b = 0; b < kSparseBatch; ++b) {
-                if (v0 + b * 64 + lane >= vec_per_row) continue;
+            for (int b = 0; b < kServedBatch; ++b) {
+                if (v0 + b * 64 + lane >= vec_end) continue;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float lo = bf16_to_f32(val[b][i] & 0xffffu);
-                    float hi = bf16_to_f32(val[b][i] >> 16);
+                    float lo = bf16_to_f32(from[b][i] & 0xffffu);
+                    float hi = bf16_to_f32(from[b][i] >> 16);
                     if (kWeights != 0) {
                         lo = __fmul_rn(lo, w);
                         hi = __fmul_rn(hi, w);
@@ -173,17 +263,50 @@ __global__ __launch_bounds__(64 * kSparseWaves) void combine_sparse_kernel(
                     acc[b][2 * i + 1] = __fadd_rn(acc[b][2 * i + 1], hi);
                 }
             }
-        }
+            const int token = __builtin_amdgcn_readlane(token_of_lane, at);
+            if (next >= 0 && __builtin_amdgcn_readlane(token_of_lane, next) == token) return;
+            u32x4* dst = out + static_cast<size_t>(token0 + token) * vec_per_row;
 #pragma unroll
-        for (int b = 0; b < kSparseBatch; ++b) {
-            const int v = v0 + b * 64 + lane;
-            if (v >= vec_per_row) continue;
-            u32x4 packed;
+            for (int b = 0; b < kServedBatch; ++b) {
+                const int v = v0 + b * 64 + lane;
+                if (v >= vec_end) continue;
+                u32x4 packed;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) packed[i] = pack_bf16x2(acc[b][2 * i], acc[b][2 * i + 1]);
-            store16_nt(dst + v, packed);
+                for (int i = 0; i < 4; ++i) packed[i] = pack_bf16x2(acc[b][2 * i], acc[b][2 * i + 1]);
+                store16_nt(dst + v, packed);
+            }
+            clear();
+        };
+        clear();
+        uint64_t rest = valid;
+        int at = __builtin_ctzll(rest);
+        rest &= rest - 1ull;
+        issue(buffer[0], at);
+        for (;;) {
+            int next = rest != 0ull ? __builtin_ctzll(rest) : -1;
+            rest &= rest - 1ull;
+            if (next >= 0) issue(buffer[1], next);
+            consume(buffer[0], at, next);
+            if (next < 0) break;
+            at = next;
+            next = rest != 0ull ? __builtin_ctzll(rest) : -1;
+            rest &= rest - 1ull;
+            if (next >= 0) issue(buffer[0], next);
+            consume(buffer[1], at, next);
+            if (next < 0) break;
+            at = next;
         }
     }
+}
+
+template <int kWeights, bool kCached>
+void launch_combine_served(hipStream_t stream, const void* y, const float* weights, const int32_t* route_to_row, int num_tokens,
+                           int num_topk, int vec, void* out, const float* return_in, float* return_out, int num_rows)
+{
+    const int tokens_per_block = 64 / num_topk;  // top-k is at most 32
+    hipLaunchKernelGGL((combine_served_kernel<kWeights, kCached>), dim3((num_tokens + tokens_per_block - 1) / tokens_per_block),
+                       dim3(64 * kServedWaves), 0, stream, static_cast<const u32x4*>(y), weights, route_to_row, num_topk,
+                       tokens_per_block, vec, static_cast<u32x4*>(out), num_tokens, return_in, return_out, num_rows);
 }
 
 struct CombineGrid {
@@ -227,10 +350,15 @@ int combine_routes(const void* y, const float* route_weights, const int32_t* rou
                    const int32_t* fill_state, int leave_unserved, hipStream_t stream)
 {
     const int vec = hidden / 8;
+    if (num_shared == 0 && leave_unserved && 2LL * num_rows_hint < num_tokens) {
+        launch_combine_served<2, true>(stream, y, route_weights, route_to_row, num_tokens, num_topk, vec, out, nullptr, nullptr,
+                                       0x7fffffff);
+        return launch_status("combine_routes_served");
+    }
     if (num_shared == 0 && 2LL * num_rows_hint < num_tokens) {  // a sparse share: most tokens own no row
         hipLaunchKernelGGL((combine_sparse_kernel<2, true>), dim3((num_tokens + kSparseWaves - 1) / kSparseWaves),
                            dim3(64 * kSparseWaves), 0, stream, static_cast<const u32x4*>(y), route_weights, route_to_row, num_topk,
-                           vec, static_cast<u32x4*>(out), num_tokens, fill_state, nullptr, nullptr, 0x7fffffff, leave_unserved);
+                           vec, static_cast<u32x4*>(out), num_tokens, fill_state, nullptr, nullptr, 0x7fffffff);
         return launch_status("combine_routes_sparse");
     }
     const CombineGrid g = combine_grid(num_tokens, num_rows_hint, vec);
@@ -264,17 +392,14 @@ int combine_entry(const char* what, const void* y, const float* row_weights, con
     const int vec = hidden / 8;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (!kHalf && leave_unserved && 2LL * num_rows < num_tokens) {
-        // a sparse share whose unserved tokens are skipped: a wave per token (with the zero rows to write as well, the
-        // workgroup-per-part kernel below measured faster: 53 against 56 us at 16384 tokens of which 2000 own rows)
-        const dim3 grid((num_tokens + kSparseWaves - 1) / kSparseWaves), block(64 * kSparseWaves);
+        // a sparse share whose unserved tokens are skipped (with the zero rows to write as well, the workgroup-per-part
+        // kernel below measured faster than a wave per token: 53 against 56 us at 16384 tokens of which 2000 own rows)
         if (row_weights != nullptr)
-            hipLaunchKernelGGL((combine_sparse_kernel<1, false>), grid, block, 0, s, static_cast<const u32x4*>(y), row_weights,
-                               route_to_row, num_topk, vec, static_cast<u32x4*>(out), num_tokens, nullptr, return_in, return_out,
-                               num_rows, 1);
+            launch_combine_served<1, false>(s, y, row_weights, route_to_row, num_tokens, num_topk, vec, out, return_in, return_out,
+                                            num_rows);
         else
-            hipLaunchKernelGGL((combine_sparse_kernel<0, false>), grid, block, 0, s, static_cast<const u32x4*>(y), nullptr,
-                               route_to_row, num_topk, vec, static_cast<u32x4*>(out), num_tokens, nullptr, return_in, return_out,
-                               num_rows, 1);
+            launch_combine_served<0, false>(s, y, nullptr, route_to_row, num_tokens, num_topk, vec, out, return_in, return_out,
+                                            num_rows);
         return launch_status(what);
     }
     const CombineGrid g = combine_grid(num_tokens, num_rows, vec);

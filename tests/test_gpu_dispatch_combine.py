@@ -627,3 +627,27 @@ def test_combine_served_only_leaves_unserved_tokens_untouched(ops, ws, weighted)
     assert torch.equal(part_back, full_back)
     with pytest.raises(ValueError, match="served_only"):
         ops.combine(y, got["route_to_row"], row_w, served_only=True)
+
+
+@pytest.mark.parametrize("topk", [1, 6, 32])
+def test_combine_served_only_any_topk(ops, topk):
+    """The served-only reduce deals 256 // top-k tokens to a workgroup: top-k values that do not divide 256, a ragged last
+    workgroup and tokens with several rows give what the zero-filling combine gives on the served tokens."""
+    gen = torch.Generator().manual_seed(100 + topk)
+    tokens, hidden = 1003, 1024
+    routes = tokens * topk
+    rows = max(routes // 12, 8)
+    route_to_row = torch.full((routes,), -1, dtype=torch.int32)
+    route_to_row[torch.randperm(routes, generator=gen)[:rows]] = torch.randperm(rows, generator=gen).int()
+    route_to_row = route_to_row.view(tokens, topk).cuda()
+    y = torch.randn(rows, hidden, generator=gen).bfloat16().cuda()
+    row_w = torch.rand(rows, generator=gen).cuda()
+    back = torch.rand(rows, generator=gen).cuda()
+    full, full_back = ops.combine(y, route_to_row, row_w, back)
+    sentinel = torch.full((tokens, hidden), -3.0, dtype=torch.bfloat16, device="cuda")
+    part, part_back = ops.combine(y, route_to_row, row_w, back, out=sentinel.clone(), served_only=True)
+    served = (route_to_row >= 0).any(dim=1)
+    assert 0 < int(served.sum()) < tokens
+    assert torch.equal(part[served].view(torch.int16), full[served].view(torch.int16))
+    assert torch.equal(part[~served], sentinel[~served])
+    assert torch.equal(part_back, full_back)
