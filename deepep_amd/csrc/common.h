@@ -60,8 +60,11 @@ struct Workspace {
 // at offset 0 the one-launch layout's epoch (64 bits: the highest tag any launch has used; a launch tags what it
 // publishes with epoch + 1 and raises the epoch when it ends, so a replayed HIP graph gets a fresh tag too); at
 // kSyncFillStop the word through which the MegaMoE fillers are told to stop (it holds the number of the launch that wrote
-// it last and needs no clearing); from kSyncTagged on the tagged per-workgroup histograms of the one-launch layout.
+// it last and needs no clearing); at kSyncReporterTag the tag the one-launch layout's reporter workgroup has settled on
+// (64 bits; it publishes no histogram, so this is how the others know that it has read the epoch); from kSyncTagged on the
+// tagged per-workgroup histograms of the one-launch layout.
 constexpr size_t kSyncFillStop = 64;
+constexpr size_t kSyncReporterTag = 128;
 constexpr size_t kSyncTagged = 256;
 constexpr size_t kSyncTaggedWords = 4096 + DPEP_MAX_LOCAL_EXPERTS;  // (workgroups + 1) * experts never exceeds this
 constexpr size_t kSyncBytes = kSyncTagged + kSyncTaggedWords * 8;

@@ -427,10 +427,12 @@ __global__ __launch_bounds__(kThreads) void layout_assign_kernel(
 // knows from the word itself whether it belongs to this launch, so there is nothing to wait for but the data, and
 // nothing to clear afterwards.  Tags only grow: a launch uses epoch + 1, where the epoch (device memory) is the highest
 // tag any launch on this workspace has used, read by every workgroup before it publishes and raised with an atomic max
-// when the workgroup ends.  No workgroup can end before every workgroup has read the epoch (it ends only after it has
-// seen everybody's words, which are published after that read), so all workgroups of a launch agree on the tag; a
-// launch that ran out of time may use two tags, and the atomic max still leaves the epoch above both.  Replays of a
-// captured launch therefore get fresh tags without any host involvement.  40 tag bits last 10^12 launches.
+// when the workgroup ends.  No workgroup can end before every workgroup has read the epoch: it ends only after it has
+// seen the words of everybody who owns a chunk, which are published after that read, and the tag of the reporter, which
+// owns none, in a word of its own (the reporter stores it right after its read; the others look for it as the last
+// thing they do, when it has long been there).  So all workgroups of a launch agree on the tag; a launch that ran
+// out of time may use two tags, and the atomic max still leaves the epoch above both.  Replays of a captured launch
+// therefore get fresh tags without any host involvement.  40 tag bits last 10^12 launches.
 // Count, exchange, assign in one launch; every wave keeps the ids of its chunk (at most kKeep steps) in registers.
 // `rows` = histogram rows to wait for (the workgroups that own chunks; one more in a test that wants the wait to run out),
 // `limit_ticks` the bound of that wait (100 MHz ticks).
@@ -450,9 +452,12 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     const int end = g < num_chunks ? min(begin + chunk, n_routes) : 0;
     // One thread reads the epoch for the whole workgroup (asked for together with the ids): every thread must use the
     // same tag, and the tag must be final before anything this workgroup publishes can be seen.
+    unsigned long long* reporter_tag = epoch + kSyncReporterTag / sizeof(unsigned long long);
+    const bool reporter = blockIdx.x == gridDim.x - 1;
     if (threadIdx.x == 0) {
         lds.tag = load_word(epoch) + 1ull;
         lds.timed_out = 0;
+        if (reporter) __hip_atomic_store(reporter_tag, lds.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     int experts[kKeep];
     fetch_experts(experts, idx, begin, end, n_routes, num_experts, expert_begin, num_local);
@@ -463,10 +468,12 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     const unsigned long long tag = lds.tag;
     // (the reporter owns no chunk and publishes nothing: row gridDim.x - 1 is only ever waited for by a test that wants
     // the wait to run out)
-    if (blockIdx.x != gridDim.x - 1) publish_tagged(lds, num_local, tagged, tag);
+    if (!reporter) publish_tagged(lds, num_local, tagged, tag);
     const TaggedSource source = {tagged, tag, rows, limit_ticks, timeouts, launch_id};
     const bool in_time = expert_bases<true>(lds, nullptr, nullptr, num_local, padded_local, num_chunks, gridDim.x - 1, counts,
                                             psum, offsets, num_rows, mailbox, sequence, &source);
+    // (asked for here, needed only at the very end: the load travels while the routes are assigned)
+    unsigned long long reporter_seen = threadIdx.x == 0 && !reporter ? load_word(reporter_tag) : 0ull;
     if (in_time) {
 #pragma unroll
         for (int i = 0; i < kKeep; ++i)
@@ -478,7 +485,24 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
         // (and the counts above are all zero).
         for (int route = begin + lane; route < end; route += kWave) route_to_row[route] = -1;
     }
-    if (threadIdx.x == 0) __hip_atomic_fetch_max(epoch, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) {
+        // The epoch may only move once the reporter has read it (a reporter that read the raised epoch would wait for
+        // words nobody publishes).  Tags only grow, so any value from this launch's tag on means that it has; the wait
+        // is bounded like the others, and a reporter that comes later still reports the launch as failed.
+        if (!reporter) {
+            long long start = 0;
+            for (int spins = 0; reporter_seen < tag; ++spins) {
+                if ((spins & 15) == 15) {
+                    const long long now = wall_clock64();
+                    if (start == 0) start = now;
+                    if (now - start > limit_ticks) break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+                reporter_seen = load_word(reporter_tag);
+            }
+        }
+        __hip_atomic_fetch_max(epoch, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 int padded_experts(int num_local)
