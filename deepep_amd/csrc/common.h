@@ -122,6 +122,12 @@ __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cas
 // Streaming (non-temporal) 16-byte accesses: the byte movers write rows nobody reads again soon, and combine reads
 // rows once.
 __device__ __forceinline__ void store16_nt(void* p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
+// Write-through 16-byte store (device scope): the line goes to memory without waiting in the L2 for an eviction.  For
+// the combine's output, which shares HBM with eight times as many reads, this measured 1 % faster than the streaming store.
+__device__ __forceinline__ void store16_through(void* p, u32x4 v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
 __device__ __forceinline__ u32x4 load16_nt(const void* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)); }
 
 // Counts of four consecutive local experts, first of them `first` (a multiple of 4), into the host mailbox as one
