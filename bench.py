@@ -347,7 +347,7 @@ def rank_share_kernels(torch, ops, cases, timer):
             lambda: ops.combine(y, r2row, recv_w, out=out), combine_bytes,
             extra={"zero_fill_bytes": zero_fill,
                    "note": "rows of unserved tokens are zero-filled, not skipped: the kernel also writes zero_fill_bytes, "
-                   "which `bytes` (the survey's algorithmic figure) leaves out"}),
+                   "which `bytes` (rows read plus served rows written) leaves out"}),
     }
     entries["combine_weighted"]["GBps_with_zero_fill"] = (combine_bytes + zero_fill) / entries["combine_weighted"]["us"] / 1e3
     entries["combine_weighted_served_only"] = timer.kernel(
