@@ -313,6 +313,27 @@ def test_combine_matches_oracle(ops, ws, name, tokens, weighted):
     np.testing.assert_array_equal(f32_bits(returned), ocombine.return_weights(ret.numpy(), want["route_to_row"]).view(np.uint32))
 
 
+@pytest.mark.parametrize("hidden,topk", [(8, 2), (520, 3), (1096, 8), (7176, 12), (2048, 32)])
+def test_combine_dense_ragged_widths_and_long_topk(ops, hidden, topk):
+    """Dense routing takes column parts of 64 16-byte vectors, a wave each: widths that end in a short part (or are
+    shorter than one part), and more slots than one batch of loads holds, against the oracle."""
+    gen = torch.Generator().manual_seed(hidden + topk)
+    tokens, experts = 130, 40
+    idx = torch.stack([torch.randperm(experts, generator=gen)[:topk] for _ in range(tokens)])
+    idx[5, :] = -1
+    idx[9, 0] = experts  # invalid id
+    want = olayout.layout(idx.numpy(), experts)
+    rows = want["num_rows"]
+    assert rows >= tokens  # dense: at least a row per token
+    y = torch.randn(rows, hidden, generator=gen).bfloat16()
+    w_rows = torch.rand(rows, generator=gen)
+    r2r = torch.from_numpy(want["route_to_row"]).cuda()
+    for weights in (None, w_rows):
+        out, _ = ops.combine(y.cuda(), r2r, None if weights is None else weights.cuda())
+        ref = ocombine.combine(bf16_bits(y), want["route_to_row"], None if weights is None else weights.numpy())
+        np.testing.assert_array_equal(bf16_bits(out), ref)
+
+
 def test_combine_reference_bounded_integer_fixture(ops, ws):
     # tests/elastic/test_combine.py:496-515: exact sums base*count + sum((e%3-1)+(s%3-1))
     tokens, hidden, experts, topk, generation = 333, 7168, 64, 8, 2
