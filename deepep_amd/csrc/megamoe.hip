@@ -495,8 +495,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                              lds0 + Cfg::kOffColScales + slot * Cfg::kColScaleSlot + wave * 1024, copy_kt & 3);
         if (kGather) copy4_to_lds_unless(index_src, lds_index + ((copy_ordinal + 1) & 1) * (kGemmThreads * 4) + wave * 256, copy_kt);
     };
-    auto advance_copy_cursor = [&](bool in_prologue) {
-        copy_stage = copy_stage + 1 == kStages ? 0 : copy_stage + 1;
+    // The cursor moves on after an item's copies: the next ring stage (advance_copy_stage), then the next k tile or tile.
+    auto finish_copy_cursor = [&](bool in_prologue = false) {
         if (++copy_kt == ktiles) {
             if (copy_tile + stride < total_tiles) {
                 // The next tile's indices were fetched with this tile's first item, so switching needs no global
@@ -513,6 +513,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                 copy_kt = ktiles - 1;  // past the last tile: keep re-copying its last item (never read)
             }
         }
+    };
+    auto advance_copy_cursor = [&](bool in_prologue) {
+        copy_stage = copy_stage + 1 == kStages ? 0 : copy_stage + 1;
+        finish_copy_cursor(in_prologue);
     };
     auto issue_item = [&]() {
 #pragma unroll
@@ -718,10 +722,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             // A wave issues in order and owns its SIMD alone, so whatever is not an MFMA should sit in the
             // shadow of one.  First k step: its MFMAs are followed, one piece each, by the LDS reads of the
             // second k step's fragments and, once the barrier has passed, by the copies of the item kAhead
-            // ahead.  Second k step: the remaining copies and the reads of the next item's scales and first
-            // fragments (whose registers the first k step has released).
+            // ahead.  Second k step: the remaining copies in its first half, then the item's scale / index copies and
+            // the copy cursor's arithmetic, and all along the reads of the next item's scales and first fragments
+            // (whose registers the first k step has released).
             shift_scales(parity);
-            constexpr int kSlots = kMfmas / 2 + kMfmas - 1;  // MFMAs after the barrier that are followed by another
+            constexpr int kSlots = kMfmas;  // MFMAs behind the barrier that deal out the item's copies
             // enough read groups per MFMA that the second k step's fragments have all left LDS before the barrier
             constexpr int kReadsPerMfma = (kGroups + kMfmas / 2 - 1) / (kMfmas / 2);
 #pragma unroll
@@ -756,9 +761,16 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
                     if (piece < kGroups) read_scale_group(parity ^ 1, row_at, col_at, piece);
                     else read_group(stage_next, 0, piece - kGroups);
                 }
+                if (n == kMfmas / 2) {
+                    // Every regular copy of the item is out: its scale / index copies and the cursor's stage arithmetic go
+                    // under the remaining MFMAs instead of behind the last one, where the matrix pipe would drain
+                    // meanwhile (45 scalar instructions used to sit there).  The counted waits only get stricter by it.
+                    issue_span_copies();
+                    copy_stage = copy_stage + 1 == kStages ? 0 : copy_stage + 1;
+                    asm volatile("" : "+s"(copy_stage));  // computed here, not sunk to the end of the item
+                }
             }
-            issue_span_copies();
-            advance_copy_cursor(false);
+            finish_copy_cursor();
             stage_now = stage_next;
         }
         kt += 2;
