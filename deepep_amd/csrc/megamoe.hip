@@ -774,7 +774,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             stage_now = stage_next;
         }
         kt += 2;
-        if (kt == ktiles) {
+        // (marked unlikely: the register allocator then keeps the loop's values in place and does its shuffling around the
+        // epilogue, once per tile, instead of at the head of the item loop)
+        if (__builtin_expect(kt == ktiles, 0)) {
                     settle_accumulators();
             // tie every accumulator to a statement behind the wait, so that no read of it can be moved above
 #pragma unroll
