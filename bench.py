@@ -24,6 +24,8 @@ Other modes:
 from __future__ import annotations
 
 import argparse
+import contextlib
+import gc
 import json
 import os
 import sys
@@ -81,6 +83,19 @@ class Timer:
             self.cycles_per_us = 2_000_000 / (start.elapsed_time(stop) * 1000.0)
         return self.cycles_per_us
 
+    @staticmethod
+    @contextlib.contextmanager
+    def no_collector():
+        """The timed loops run without Python's cyclic garbage collector: a full collection over the benchmark's heap
+        takes tens of milliseconds and would land in whichever launch happens to trigger it."""
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            yield
+        finally:
+            if was_enabled:
+                gc.enable()
+
     def back_to_back(self, fn, head_start=False):
         """Average microseconds over `iters` launches queued without gaps.  head_start: the GPU is kept busy first by a
         spin kernel (no memory traffic that the timed kernels would have to wait out) for as long as the host needs to
@@ -96,11 +111,12 @@ class Timer:
         torch.cuda.synchronize()
         if head_start and hasattr(torch.cuda, "_sleep"):
             torch.cuda._sleep(int(self.spin_cycles_per_us() * host_us * self.iters * 1.5) + 100_000)
-        start.record()
-        for _ in range(self.iters):
-            fn()
-        stop.record()
-        torch.cuda.synchronize()
+        with self.no_collector():
+            start.record()
+            for _ in range(self.iters):
+                fn()
+            stop.record()
+            torch.cuda.synchronize()
         return start.elapsed_time(stop) * 1000.0 / self.iters
 
     def flushed(self, fn, read_sweep=False):
@@ -113,15 +129,16 @@ class Timer:
         pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(self.iters)]
         for _ in range(self.warmups):
             fn()
-        for start, stop in pairs:
-            if read_sweep:
-                self.flush.view(torch.int64).sum()
-            else:
-                self.flush.zero_()
-            start.record()
-            fn()
-            stop.record()
-        torch.cuda.synchronize()
+        with self.no_collector():
+            for start, stop in pairs:
+                if read_sweep:
+                    self.flush.view(torch.int64).sum()
+                else:
+                    self.flush.zero_()
+                start.record()
+                fn()
+                stop.record()
+            torch.cuda.synchronize()
         times = sorted(a.elapsed_time(b) * 1000.0 for a, b in pairs)
         pick = lambda q: times[min(len(times) - 1, int(q * len(times)))]
         return dict(mean=sum(times) / len(times), min=times[0], p50=pick(0.5), p95=pick(0.95))
@@ -289,6 +306,14 @@ def megamoe_bench(torch, ops, timer, with_cpu):
         "workload": "8192 tokens x top-8, all 32 experts local (65 536 rows), one weight set (705 MB); whole forward",
         "rows": rows, "us_forward": us, "flushed_us": cold, "gflop": flops / 1e9, "tflops_forward": flops / us / 1e6,
         "frac_of_fp8_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS,
+    }
+    us, cold, rows, flops = megamoe_shape(torch, ops, timer, 512, 256, 32, 8, weight_sets=1)
+    weight_bytes = 32 * (2 * inter * hidden + hidden * inter) // 2
+    result["decode_share"] = {
+        "workload": "512 tokens x top-8, 32 of 256 experts local (about 16 rows per expert): the GEMMs are bound by streaming "
+        "their 705 MB of FP4 weights (64-row tiles, non-temporal weight copies); whole forward",
+        "rows": rows, "us_forward": us, "flushed_us": cold, "weight_bytes": weight_bytes,
+        "weights_GBps_forward": weight_bytes / us / 1e3, "frac_of_8TBps": weight_bytes / us / 1e3 / HBM_PEAK_GBS,
     }
     if with_cpu:
         result["cpu_baseline"] = megamoe_cpu_baseline(hidden, inter)
@@ -471,11 +496,12 @@ def main():
     for _ in range(args.warmup):
         rows, _, _ = step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        rows, _, _ = step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with Timer.no_collector():
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            rows, _, _ = step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
 
     nbytes = algorithmic_bytes(tokens, hidden, topk, rows)
