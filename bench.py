@@ -525,6 +525,13 @@ def main():
         "combine": timer.kernel(lambda: ops.combine(grows, r2row, out=out_buf), nbytes["combine"], read_sweep=True),
         "combine_weighted": timer.kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), nbytes["combine"] + rows * 4, read_sweep=True),
     }
+    # the stand-alone quantiser on the batch's tokens and the dequantiser on its dispatched rows (checking-side kernels of
+    # the reference: per_token_cast_to_fp8 / per_token_cast_back)
+    recv_q, recv_s, _ = ops.dispatch_copy(q_pre, s_pre, None, r2row, r2route, rows)
+    scale_bytes = (hidden // 128) * 4
+    kernels["cast_to_fp8"] = timer.kernel(lambda: ops.cast_to_fp8(xd), tokens * (3 * hidden + scale_bytes), head_start=True)
+    kernels["cast_back"] = timer.kernel(lambda: ops.cast_back(recv_q, recv_s), rows * (3 * hidden + scale_bytes))
+    del recv_q, recv_s
 
     dominant = kernels["combine"]
     result = {
