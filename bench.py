@@ -315,6 +315,11 @@ def megamoe_bench(torch, ops, timer, with_cpu):
         "rows": rows, "us_forward": us, "flushed_us": cold, "weight_bytes": weight_bytes,
         "weights_GBps_forward": weight_bytes / us / 1e3, "frac_of_8TBps": weight_bytes / us / 1e3 / HBM_PEAK_GBS,
     }
+    # the MX activation quantiser the public API runs when it is given BF16 rows (per-32 e8m0 scales)
+    xb = torch.randn(64 * 256, hidden, device="cuda").bfloat16()
+    result["mx_quant"] = timer.kernel(lambda: ops.mx_quant(xb), xb.numel() * 3 + xb.numel() // 32)
+    result["mx_quant"]["workload"] = "BF16 [16384,7168] -> e4m3 codes + e8m0 scale per 32"
+    del xb
     if with_cpu:
         result["cpu_baseline"] = megamoe_cpu_baseline(hidden, inter)
     return result
