@@ -32,6 +32,8 @@ constexpr int kWaves = 4;             // wavefronts (= chunks) per workgroup
 constexpr int kThreads = kWaves * kWave;
 constexpr int kHistInts = 16384;      // chunks * padded experts never exceeds this
 constexpr int kBlockHistInts = kHistInts / kWaves + DPEP_MAX_LOCAL_EXPERTS;  // workgroups * experts, rounded up
+constexpr int kLargeHistInts = 65536;  // the two-launch form of large inputs, where the workspace has the room
+constexpr int kLargeBlockHistInts = kLargeHistInts / kWaves + DPEP_MAX_LOCAL_EXPERTS;
 constexpr int kMinChunk = 256;        // routes per wavefront, lower bound (multiple of 64)
 constexpr int kPrefetch = 8;          // 64-route steps whose ids are fetched at once
 constexpr int kKeep = 16;             // 64-route steps of a chunk that the one-launch kernel holds in registers
@@ -513,9 +515,9 @@ int padded_experts(int num_local)
 }
 
 // Chunk length: as many chunks as the histogram budget allows (16..256), at least kMinChunk routes each.
-int chunk_routes(int n_routes, int padded_local)
+int chunk_routes(int n_routes, int padded_local, int hist_ints = kHistInts)
 {
-    int max_chunks = kHistInts / padded_local;
+    int max_chunks = hist_ints / padded_local;
     max_chunks = max_chunks > 256 ? 256 : (max_chunks < 16 ? 16 : max_chunks);
     int chunk = (n_routes + max_chunks - 1) / max_chunks;
     chunk = (chunk + kWave - 1) / kWave * kWave;
@@ -585,17 +587,25 @@ int launch_layout(void* ws, const IdxT* idx, int num_tokens, int num_topk, int n
     }
     w->layout_launches = w->layout_launches == 0xffffffffu ? 1u : w->layout_launches + 1u;  // never 0
     const int padded = padded_experts(num_local);
-    const int chunk = chunk_routes(n_routes, padded);
+    int chunk = chunk_routes(n_routes, padded);
+    const bool one_launch = n_routes > 0 && chunk <= kKeep * kWave && w->layout_one_launch;
+    // Inputs that take two launches anyway get shorter chunks (more waves at work), with the larger histograms the
+    // workspace has room for: 131 072 routes over 256 local experts 16 -> 64 workgroups.
+    int hist_ints = kHistInts;
+    if (!one_launch) {
+        hist_ints = kLargeHistInts;
+        chunk = chunk_routes(n_routes, padded, kLargeHistInts);
+    }
     const int num_chunks = (n_routes + chunk - 1) / chunk;
     int* wave_hist = static_cast<int*>(w->base);
-    int* block_hist = wave_hist + kHistInts;
+    int* block_hist = wave_hist + hist_ints;
     const int blocks = (num_chunks + kWaves - 1) / kWaves;
     if (report_to_host) {
         w->sequence = w->sequence == 0xffffffffu ? 1u : w->sequence + 1u;  // never 0: that is "nothing launched"
         w->mailbox_local = num_local;
     }
     uint32_t* mailbox = report_to_host ? w->mailbox_device : nullptr;
-    if (blocks > 0 && chunk <= kKeep * kWave && w->layout_one_launch) {
+    if (one_launch) {
         char* sync = static_cast<char*>(w->sync);
         hipLaunchKernelGGL(layout_fused_kernel<IdxT>, dim3(blocks + 1), dim3(kThreads), 0, stream, idx, n_routes, num_experts,
                            expert_begin, num_local, padded, chunk, num_chunks, counts, psum, offsets, num_rows, route_to_row,
@@ -665,7 +675,7 @@ extern "C" {
 size_t dpep_layout_workspace_bytes(int num_tokens, int num_topk, int num_local_experts)
 {
     if (num_tokens < 0 || num_topk < 1 || num_local_experts < 1) return 0;
-    return static_cast<size_t>(dpep::kHistInts + dpep::kBlockHistInts) * sizeof(int);
+    return static_cast<size_t>(dpep::kLargeHistInts + dpep::kLargeBlockHistInts) * sizeof(int);
 }
 
 int dpep_layout(void* ws, const int64_t* topk_idx, int num_tokens, int num_topk, int num_experts, int expert_begin,
