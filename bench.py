@@ -149,7 +149,8 @@ class Timer:
         warm = self.back_to_back(fn, head_start)
         cold = self.flushed(fn)
         if read_sweep:
-            extra = dict(extra or {}, after_read_sweep_us=self.flushed(fn, read_sweep=True))
+            swept = self.flushed(fn, read_sweep=True)
+            extra = dict(extra or {}, after_read_sweep_us=swept, frac_after_read_sweep=nbytes / swept["mean"] / 1e3 / HBM_PEAK_GBS)
         entry = dict(
             bytes=nbytes,
             us=cold["mean"],
@@ -453,6 +454,8 @@ def main():
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="also launch a plain copy of known size (identity dispatch of [32768,7168] BF16: 469.76 MB "
                         "read + 469.76 MB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled")
+    parser.add_argument("--dispatch-stores", choices=("through", "streaming", "cached"),
+                        help="store policy of the dispatch kernels (default: the library's, write-through)")
     parser.add_argument("--ingest-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"))
     parser.add_argument("--protocol", metavar="PRESET", help="run the reference's generic benchmark workload PRESET "
                         "(smoke, decode, prefill) and print one `measured` record per operation")
@@ -481,6 +484,8 @@ def main():
             print(json.dumps(record))
         return
 
+    if args.dispatch_stores:
+        ops.dispatch_store_policy(args.dispatch_stores)
     x, idx, w, cfg = cases.make_inputs("C3", seed=0)
     tokens, hidden, topk, experts = cfg["tokens"], cfg["hidden"], cfg["topk"], cfg["experts"]
     rows_expected = tokens * topk
@@ -564,7 +569,8 @@ def main():
             "kernel_timing": f"{args.kernel_warmup} warm-ups + {args.kernel_iters} launches per kernel and protocol; "
             "`us` / `GBps` / `frac_of_8TBps` are the cache-flushed mean (256 MiB fill before every launch), "
             "`back_to_back_us` / `frac_back_to_back` the same launches queued without gaps, `after_read_sweep_us` the "
-            "launches after a read-only pass over 256 MiB (caches evicted, no dirty lines left to write back)",
+            "launches after a read-only pass over 256 MiB (caches evicted, no dirty lines left to write back: "
+            "`frac_after_read_sweep`)",
         },
         "roofline": {
             "kernel": "combine_kernel<0, false>",
@@ -582,7 +588,14 @@ def main():
         "kernels": kernels,
         "dispatch_plus_combine_us": kernels["dispatch_fp8_quant"]["us"] + kernels["combine"]["us"],
         "dispatch_plus_combine_frac_of_8TBps": moved / (kernels["dispatch_fp8_quant"]["us"] + kernels["combine"]["us"]) / 1e3 / HBM_PEAK_GBS,
+        "dispatch_stores": ops.dispatch_store_policy(),
     }
+    # the same sum under the two other protocols; the fill figure above also pays for writing back the fill's own dirty
+    # lines, which leave the caches while the timed kernel runs
+    for key, pick in (("after_read_sweep", lambda k: k["after_read_sweep_us"]["mean"]), ("back_to_back", lambda k: k["back_to_back_us"])):
+        both = pick(kernels["dispatch_fp8_quant"]) + pick(kernels["combine"])
+        result[f"dispatch_plus_combine_{key}_us"] = both
+        result[f"dispatch_plus_combine_{key}_frac_of_8TBps"] = moved / both / 1e3 / HBM_PEAK_GBS
     if args.calibrate_copy:
         ident = torch.arange(rows, dtype=torch.int32, device=dev)
         for _ in range(5):

@@ -28,6 +28,7 @@ SIGNATURES = {
     "dpep_layout": (_I, (_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P)),
     "dpep_layout_static": (_I, (_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P)),
     "dpep_layout_wait": (_I, (_P, _P, _I, ctypes.POINTER(ctypes.c_int32), ctypes.c_longlong)),
+    "dpep_dispatch_store_policy": (_I, (_I,)),
     "dpep_dispatch_copy": (_I, (_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_dispatch_quant_fp8": (_I, (_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_layout_dispatch_small": (_I, (_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P)),
@@ -42,6 +43,8 @@ SIGNATURES = {
     "dpep_megamoe_padded_dim": (_I, (_I,)),
     "dpep_megamoe_prepared_shape": (_I, (_I, _I, _I, ctypes.POINTER(_I), ctypes.POINTER(_I), ctypes.POINTER(_I))),
     "dpep_megamoe_prepare_weights": (_I, (_P, _P, _I, _I, _I, _I, _P, _P, _P)),
+    "dpep_megamoe_fill_report": (_I, (_P, _I, _I, _I, _I, _I, _I, ctypes.POINTER(ctypes.c_int32),
+                                      ctypes.POINTER(ctypes.c_int64), _P)),
     "dpep_megamoe_forward": (_I, (_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
                                   _P, _P, _P)),
 }

@@ -51,7 +51,6 @@ struct Workspace {
     int layout_one_launch;
     uint32_t layout_launches;  // number of the most recent layout launch (never 0)
     uint32_t timeout_seen;     // number of the last timed-out launch the host has been told about
-    uint32_t gemm_launches;    // number of the most recent MegaMoE forward (never 0)
     int gemm_zero_fill;        // 1 (default): idle workgroups of the first GEMM zero rows of unserved tokens; 0: the reduce does
     int megamoe_served_only;   // 1: rows of y whose token no local expert serves are left untouched; 0 (default): zeroed
     int gemm_tile_rows;  // 0: the grouped GEMM chooses its tile height; 64 / 128 / 192: forced (tests)
@@ -59,8 +58,8 @@ struct Workspace {
 // Device memory the kernels synchronise through, behind the caller's bytes, zero when the workspace is created:
 // at offset 0 the one-launch layout's epoch (64 bits: the highest tag any launch has used; a launch tags what it
 // publishes with epoch + 1 and raises the epoch when it ends, so a replayed HIP graph gets a fresh tag too); at
-// kSyncFillStop the word through which the MegaMoE fillers are told to stop (it holds the number of the launch that wrote
-// it last and needs no clearing); at kSyncReporterTag the tag the one-launch layout's reporter workgroup has settled on
+// kSyncFillStop the word through which the MegaMoE fillers are told to stop (a counter that only grows: a filler stops when
+// it differs from what the filler found at its start, so it needs no clearing and no value from the host); at kSyncReporterTag the tag the one-launch layout's reporter workgroup has settled on
 // (64 bits; it publishes no histogram, so this is how the others know that it has read the epoch); from kSyncTagged on the
 // tagged per-workgroup histograms of the one-launch layout.
 constexpr size_t kSyncFillStop = 64;
@@ -69,8 +68,8 @@ constexpr size_t kSyncTagged = 256;
 constexpr size_t kSyncTaggedWords = 4096 + DPEP_MAX_LOCAL_EXPERTS;  // (workgroups + 1) * experts never exceeds this
 constexpr size_t kSyncBytes = kSyncTagged + kSyncTaggedWords * 8;
 // The host mailbox (pinned memory, 32-bit words): word 0 = number of rows and word 1 = sequence number of the layout
-// that reported last (one 8-byte store); word kMailboxTimeout = launch number of a layout kernel whose barrier wait
-// ran out; from word kMailboxCounts on, 16-byte aligned, the per-expert counts.
+// that reported last (one 8-byte store); word kMailboxTimeout = launch number of a layout kernel whose wait for the
+// other workgroups' histograms ran out; from word kMailboxCounts on, 16-byte aligned, the per-expert counts.
 constexpr int kMailboxTimeout = 2;
 constexpr int kMailboxCounts = 4;
 constexpr int kMailboxWords = kMailboxCounts + (DPEP_MAX_LOCAL_EXPERTS + 3) / 4 * 4;

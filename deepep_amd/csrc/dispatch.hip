@@ -1,9 +1,12 @@
 // Expand-permute payload dispatch: out[row(t,s)] = x[t] for every route that owns a row, optionally
 // fused with the per-128-element FP8 e4m3fn block quantiser.  HBM-bound: 16-byte coalesced loads,
-// non-temporal 16-byte stores, each input row read once and written to its K destinations.
+// 16-byte stores, each input row read once and written to its K destinations.  How the token-major kernels store
+// is a process-wide policy (dpep_dispatch_store_policy): write-through by default, streaming or cached on request.
 //
 // Observable contract: tests/elastic/test_dispatch.py:1391-1416 (payload, scales and weights arrive
 // bit-exactly in row order), tests/clos/common.py:276-279; quantiser deep_ep/utils/math.py:45-61.
+#include <type_traits>
+
 #include "common.h"
 
 #pragma clang fp contract(off)
@@ -16,7 +19,35 @@ constexpr int kTargetBlocks = 8192;  // rows are split into column parts until a
 constexpr int kMaxScaleCols = 1024;  // hidden <= 131072 for the fused quantiser
 constexpr int kRowMajorRatio = 1;  // row-major kernels when rows <= ratio * tokens
 
+// Store policy of the token-major kernels' payload rows.  Write-through (device-scope `sc1`): the rows pass through the
+// memory-side cache on their way to HBM, which takes the kernel's time the same way whatever the caches held before
+// the launch (clean lines of other tensors, the input just produced, or the kernel's own previous output).  Streaming
+// (non-temporal): the rows go to HBM past the caches at the streaming-write rate; the input stays cached from one call to
+// the next, so a loop that dispatches the same buffer again and again is faster this way and a call whose input is
+// cold is slower.  Cached: plain stores.
+int g_store_policy = DPEP_STORE_THROUGH;
+
+template <int kPolicy>
+__device__ __forceinline__ void store16_as(void* p, u32x4 v)
+{
+    if (kPolicy == DPEP_STORE_THROUGH) store16_through(p, v);
+    else if (kPolicy == DPEP_STORE_STREAMING) store16_nt(p, v);
+    else *reinterpret_cast<u32x4*>(p) = v;
+}
+
+// Calls launch(std::integral_constant<int, policy>) for the current policy.
+template <typename Launch>
+void with_store_policy(Launch&& launch)
+{
+    switch (__atomic_load_n(&g_store_policy, __ATOMIC_RELAXED)) {
+    case DPEP_STORE_STREAMING: launch(std::integral_constant<int, DPEP_STORE_STREAMING>{}); break;
+    case DPEP_STORE_CACHED: launch(std::integral_constant<int, DPEP_STORE_CACHED>{}); break;
+    default: launch(std::integral_constant<int, DPEP_STORE_THROUGH>{}); break;
+    }
+}
+
 // ---- token-major copy: one workgroup per (token, column part); read once, write K times -----------
+template <int kPolicy>
 __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
     const u32x4* __restrict__ x, const float* __restrict__ scales, const float* __restrict__ weights,
     const int* __restrict__ route_to_row, int num_topk, int vec_per_row, int vec_per_part, int parts, int scale_cols,
@@ -31,7 +62,7 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
     // The token's first values are asked for before its routes are known (see the quantising kernel below).
     const int v_first = v_begin + threadIdx.x;
     u32x4 first = {0u, 0u, 0u, 0u};
-    if (v_first < v_end) first = load16(src + v_first);  // plain loads with streaming stores measured fastest here
+    if (v_first < v_end) first = load16(src + v_first);
     if (threadIdx.x == 0) any_valid = 0;
     __syncthreads();
     if (threadIdx.x < num_topk) {
@@ -45,7 +76,7 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
         const u32x4 value = v == v_first ? first : load16(src + v);
         for (int s = 0; s < num_topk; ++s) {
             const int row = rows[s];
-            if (row >= 0) store16_nt(out + static_cast<size_t>(row) * vec_per_row + v, value);
+            if (row >= 0) store16_as<kPolicy>(out + static_cast<size_t>(row) * vec_per_row + v, value);
         }
     }
     if (part == 0) {
@@ -64,19 +95,21 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_token_kernel(
 }
 
 // ---- row-major copy: one workgroup per (output row, column part); for sparse receive shares -------
+template <int kPolicy>
 __global__ __launch_bounds__(kMaxThreads) void dispatch_copy_row_kernel(
     const u32x4* __restrict__ x, const float* __restrict__ scales, const float* __restrict__ weights,
-    const int* __restrict__ row_to_route, int num_topk, int vec_per_row, int vec_per_part, int parts, int scale_cols,
-    u32x4* __restrict__ out, float* __restrict__ out_scales, float* __restrict__ out_weights)
+    const int* __restrict__ row_to_route, int num_tokens, int num_topk, int vec_per_row, int vec_per_part, int parts,
+    int scale_cols, u32x4* __restrict__ out, float* __restrict__ out_scales, float* __restrict__ out_weights)
 {
     const int row = blockIdx.x / parts, part = blockIdx.x % parts;
-    const int route = row_to_route[row];
+    // (clamped: a map left incomplete by a layout launch that reported a time-out must not become a wild address)
+    const int route = min(max(row_to_route[row], 0), num_tokens * num_topk - 1);
     const int token = route / num_topk;
     const int v_begin = part * vec_per_part;
     const int v_end = min(v_begin + vec_per_part, vec_per_row);
     const u32x4* src = x + static_cast<size_t>(token) * vec_per_row;
     u32x4* dst = out + static_cast<size_t>(row) * vec_per_row;
-    for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x) store16_nt(dst + v, load16(src + v));
+    for (int v = v_begin + threadIdx.x; v < v_end; v += blockDim.x) store16_as<kPolicy>(dst + v, load16(src + v));
     if (part == 0) {
         if (scales != nullptr)
             for (int c = threadIdx.x; c < scale_cols; c += blockDim.x)
@@ -136,6 +169,7 @@ __device__ __forceinline__ Quant16 quantize16(u32x4 lo, u32x4 hi)
 }
 
 // token-major: one workgroup per (token, column part); units = 16-element groups per row (H/16).
+template <int kPolicy>
 __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
     const u32x4* __restrict__ x, const float* __restrict__ weights, const int* __restrict__ route_to_row, int num_topk,
     int units_per_row, int units_per_part, int parts, u32x4* __restrict__ out, float* __restrict__ out_scales,
@@ -189,14 +223,14 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
 #pragma unroll
         for (int j = 0; j < kEarly; ++j) {
             const int u = u_first + j * static_cast<int>(blockDim.x);
-            if (u < u_end) store16_nt(out + static_cast<size_t>(row) * units_per_row + u, codes[j]);
+            if (u < u_end) store16_as<kPolicy>(out + static_cast<size_t>(row) * units_per_row + u, codes[j]);
         }
     }
     for (int u = u_first + kEarly * static_cast<int>(blockDim.x); u < u_end; u += blockDim.x) {  // rows wider than that
         const Quant16 q = quantize16(load16(src + 2 * u), load16(src + 2 * u + 1));
         for (int s = 0; s < num_topk; ++s) {
             const int row = rows[s];
-            if (row >= 0) store16_nt(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
+            if (row >= 0) store16_as<kPolicy>(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
         }
         if ((u & 7) == 0) part_scales[(u - u_begin) >> 3] = q.scale;
     }
@@ -215,13 +249,14 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_token_kernel(
 
 // row-major: one workgroup per (output row, column part); row_to_route == nullptr means identity
 // (row == token), which is the stand-alone quantiser.
+template <int kPolicy>
 __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_row_kernel(
-    const u32x4* __restrict__ x, const float* __restrict__ weights, const int* __restrict__ row_to_route, int num_topk,
-    int units_per_row, int units_per_part, int parts, u32x4* __restrict__ out, float* __restrict__ out_scales,
+    const u32x4* __restrict__ x, const float* __restrict__ weights, const int* __restrict__ row_to_route, int num_tokens,
+    int num_topk, int units_per_row, int units_per_part, int parts, u32x4* __restrict__ out, float* __restrict__ out_scales,
     float* __restrict__ out_weights)
 {
     const int row = blockIdx.x / parts, part = blockIdx.x % parts;
-    const int route = row_to_route != nullptr ? row_to_route[row] : row;
+    const int route = row_to_route != nullptr ? min(max(row_to_route[row], 0), num_tokens * num_topk - 1) : row;
     const int token = row_to_route != nullptr ? route / num_topk : row;
     const int u_begin = part * units_per_part;
     const int u_end = min(u_begin + units_per_part, units_per_row);
@@ -229,7 +264,7 @@ __global__ __launch_bounds__(kMaxThreads) void dispatch_quant_row_kernel(
     const u32x4* src = x + static_cast<size_t>(token) * units_per_row * 2;
     for (int u = u_begin + threadIdx.x; u < u_end; u += blockDim.x) {
         const Quant16 q = quantize16(load16(src + 2 * u), load16(src + 2 * u + 1));
-        store16_nt(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
+        store16_as<kPolicy>(out + static_cast<size_t>(row) * units_per_row + u, q.codes);
         if ((u & 7) == 0) out_scales[static_cast<size_t>(row) * scale_cols + (u >> 3)] = q.scale;
     }
     if (part == 0 && weights != nullptr && threadIdx.x == 0) out_weights[row] = weights[route];
@@ -498,6 +533,17 @@ int check_common(const char* what, int num_tokens, int num_topk, int num_rows, c
 
 extern "C" {
 
+int dpep_dispatch_store_policy(int policy)
+{
+    using namespace dpep;
+    const int before = __atomic_load_n(&g_store_policy, __ATOMIC_RELAXED);
+    if (policy == DPEP_STORE_QUERY) return before;
+    DPEP_REQUIRE(policy == DPEP_STORE_THROUGH || policy == DPEP_STORE_STREAMING || policy == DPEP_STORE_CACHED,
+                 "dispatch_store_policy: %d is not DPEP_STORE_THROUGH, _STREAMING, _CACHED or _QUERY", policy);
+    __atomic_store_n(&g_store_policy, policy, __ATOMIC_RELAXED);
+    return before;
+}
+
 int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_weights, const int32_t* route_to_row,
                        const int32_t* row_to_route, int num_tokens, int num_topk, int num_rows, int row_bytes,
                        int scale_cols, void* out, float* out_scales, float* out_weights, void* stream)
@@ -516,15 +562,20 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
     // the token-major grid does not depend on R, so a launch that does not know R yet takes it
     if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(kRowMajorRatio) * num_tokens) {
         const Split sp = choose_split(num_tokens, vec, 1);
-        hipLaunchKernelGGL(dispatch_copy_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
-                           static_cast<const u32x4*>(x), scales, topk_weights, route_to_row, num_topk, vec, sp.per_part,
-                           sp.parts, scale_cols, static_cast<u32x4*>(out), out_scales, out_weights);
+        with_store_policy([&](auto policy) {
+            hipLaunchKernelGGL(dispatch_copy_token_kernel<decltype(policy)::value>, dim3(num_tokens * sp.parts),
+                               dim3(sp.threads), 0, s, static_cast<const u32x4*>(x), scales, topk_weights, route_to_row,
+                               num_topk, vec, sp.per_part, sp.parts, scale_cols, static_cast<u32x4*>(out), out_scales,
+                               out_weights);
+        });
         return launch_status("dispatch_copy_token");
     }
     const Split sp = choose_split(num_rows, vec, 1);
-    hipLaunchKernelGGL(dispatch_copy_row_kernel, dim3(num_rows * sp.parts), dim3(sp.threads), 0, s,
-                       static_cast<const u32x4*>(x), scales, topk_weights, row_to_route, num_topk, vec, sp.per_part,
-                       sp.parts, scale_cols, static_cast<u32x4*>(out), out_scales, out_weights);
+    with_store_policy([&](auto policy) {
+        hipLaunchKernelGGL(dispatch_copy_row_kernel<decltype(policy)::value>, dim3(num_rows * sp.parts), dim3(sp.threads), 0,
+                           s, static_cast<const u32x4*>(x), scales, topk_weights, row_to_route, num_tokens, num_topk, vec,
+                           sp.per_part, sp.parts, scale_cols, static_cast<u32x4*>(out), out_scales, out_weights);
+    });
     return launch_status("dispatch_copy_row");
 }
 
@@ -544,15 +595,19 @@ int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int3
     // the token-major grid does not depend on R, so a launch that does not know R yet takes it
     if (num_rows < 0 || static_cast<long long>(num_rows) > static_cast<long long>(kRowMajorRatio) * num_tokens) {
         const Split sp = choose_split(num_tokens, units, 8);
-        hipLaunchKernelGGL(dispatch_quant_token_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0, s,
-                           static_cast<const u32x4*>(x), topk_weights, route_to_row, num_topk, units, sp.per_part,
-                           sp.parts, static_cast<u32x4*>(out), out_scales, out_weights);
+        with_store_policy([&](auto policy) {
+            hipLaunchKernelGGL(dispatch_quant_token_kernel<decltype(policy)::value>, dim3(num_tokens * sp.parts),
+                               dim3(sp.threads), 0, s, static_cast<const u32x4*>(x), topk_weights, route_to_row, num_topk,
+                               units, sp.per_part, sp.parts, static_cast<u32x4*>(out), out_scales, out_weights);
+        });
         return launch_status("dispatch_quant_token");
     }
     const Split sp = choose_split(num_rows, units, 8);
-    hipLaunchKernelGGL(dispatch_quant_row_kernel, dim3(num_rows * sp.parts), dim3(sp.threads), 0, s,
-                       static_cast<const u32x4*>(x), topk_weights, row_to_route, num_topk, units, sp.per_part, sp.parts,
-                       static_cast<u32x4*>(out), out_scales, out_weights);
+    with_store_policy([&](auto policy) {
+        hipLaunchKernelGGL(dispatch_quant_row_kernel<decltype(policy)::value>, dim3(num_rows * sp.parts), dim3(sp.threads),
+                           0, s, static_cast<const u32x4*>(x), topk_weights, row_to_route, num_tokens, num_topk, units,
+                           sp.per_part, sp.parts, static_cast<u32x4*>(out), out_scales, out_weights);
+    });
     return launch_status("dispatch_quant_row");
 }
 
@@ -626,9 +681,12 @@ int dpep_cast_to_fp8(const void* x, int num_tokens, int hidden, void* out, float
         return launch_status("cast_to_fp8");
     }
     const Split sp = choose_split(num_tokens, units, 8);
-    hipLaunchKernelGGL(dispatch_quant_row_kernel, dim3(num_tokens * sp.parts), dim3(sp.threads), 0,
-                       static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), nullptr, nullptr, 1, units,
-                       sp.per_part, sp.parts, static_cast<u32x4*>(out), out_scales, nullptr);
+    with_store_policy([&](auto policy) {
+        hipLaunchKernelGGL(dispatch_quant_row_kernel<decltype(policy)::value>, dim3(num_tokens * sp.parts),
+                           dim3(sp.threads), 0, static_cast<hipStream_t>(stream), static_cast<const u32x4*>(x), nullptr,
+                           nullptr, num_tokens, 1, units, sp.per_part, sp.parts, static_cast<u32x4*>(out), out_scales,
+                           nullptr);
+    });
     return launch_status("cast_to_fp8");
 }
 

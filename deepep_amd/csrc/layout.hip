@@ -336,8 +336,10 @@ __device__ __forceinline__ bool expert_bases(LayoutLds& lds, const int* __restri
     __syncthreads();
     const bool valid = !kTagged || lds.timed_out == 0;
     if (!valid) {
-        // A histogram is missing: every count is reported as zero, and the host is told (this store is acknowledged
-        // before the reporter publishes the mailbox's sequence word below, so the host never sees one without the other).
+        // A histogram is missing: every count is reported as zero, and the host is told.  (The reporter's own store is
+        // acknowledged before it publishes the mailbox's sequence word below, so the host never sees a reporter's
+        // time-out later than its report; another workgroup's time-out may reach the host after the report, and is
+        // then found by the next call on the workspace.)
         if (tid == 0) __hip_atomic_store(source->timeouts, source->launch_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         for (int e = tid; e < num_local; e += kThreads) {
             lds.totals[e] = 0;
@@ -471,7 +473,12 @@ __global__ __launch_bounds__(kThreads) void layout_fused_kernel(
     // (the reporter owns no chunk and publishes nothing: row gridDim.x - 1 is only ever waited for by a test that wants
     // the wait to run out)
     if (!reporter) publish_tagged(lds, num_local, tagged, tag);
-    const TaggedSource source = {tagged, tag, rows, limit_ticks, timeouts, launch_id};
+    // The reporter gives up first (the others wait twice as long): a launch that the reporter passes as valid is then
+    // one in which every histogram arrived within the reporter's bound, so another workgroup can only have run out of
+    // time if its own wait began more than a whole bound before the reporter's.  What remains of that window is closed
+    // on the consumers' side: such a workgroup marks its routes as having no row, and the kernels that read
+    // row_to_route clamp what they find there.
+    const TaggedSource source = {tagged, tag, rows, reporter ? limit_ticks : 2 * limit_ticks, timeouts, launch_id};
     const bool in_time = expert_bases<true>(lds, nullptr, nullptr, num_local, padded_local, num_chunks, gridDim.x - 1, counts,
                                             psum, offsets, num_rows, mailbox, sequence, &source);
     // (asked for here, needed only at the very end: the load travels while the routes are assigned)

@@ -11,6 +11,8 @@
 //   B: lane l holds column l%32; 4 VGPRs = 32 nibbles k in [32g, 32g+32), low nibble first
 //   scales: lane l supplies the e8m0 byte of (row or column l%32, 32-wide k block l/32)
 //   D: acc[j] is row (j/4)*8 + (l/32)*4 + j%4, column l%32
+#include <atomic>
+
 #include "common.h"
 #include "gemm_schedule.h"
 
@@ -54,34 +56,56 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
     return static_cast<uint32_t>(packed);
 }
 
-// One lane owns 8 consecutive BF16 values; 4 adjacent lanes own one 32-element block.
-__global__ __launch_bounds__(256) void mx_quant_kernel(const u32x4* __restrict__ x, long long num_units,
-                                                       int units_per_row, u32x2* __restrict__ codes,
-                                                       uint8_t* __restrict__ scales)
+// One lane owns 16 consecutive BF16 values (32 bytes in, one 16-byte vector of codes out, consecutive lanes writing
+// consecutive vectors); two adjacent lanes own one 32-element block.  The workgroup's 128 scale bytes are staged in LDS
+// and leave as eight 16-byte stores instead of one byte-wide store per block, which turned every scale row into
+// read-modify-write traffic.  The tensors are treated as flat arrays: hidden is a multiple of 32, so blocks never
+// straddle rows.  kVectorScales: the scale pointer is 16-byte aligned.
+constexpr int kMxThreads = 256;
+
+template <bool kVectorScales>
+__global__ __launch_bounds__(kMxThreads) void mx_quant_kernel(const u32x4* __restrict__ x, long long num_units,
+                                                              u32x4* __restrict__ codes, uint8_t* __restrict__ scales)
 {
-    const long long u = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    __shared__ __attribute__((aligned(16))) uint8_t staged[kMxThreads / 2];
+    const long long u = static_cast<long long>(blockIdx.x) * kMxThreads + threadIdx.x;
     const bool live = u < num_units;
-    u32x4 raw = {0, 0, 0, 0};
-    if (live) raw = x[u];
-    float v[8];
+    u32x4 raw[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+    if (live) {
+        raw[0] = load16(x + 2 * u);
+        raw[1] = load16(x + 2 * u + 1);
+    }
+    float v[16];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        v[2 * i] = bf16_to_f32(raw[i] & 0xffffu);
-        v[2 * i + 1] = bf16_to_f32(raw[i] >> 16);
+    for (int i = 0; i < 8; ++i) {
+        v[2 * i] = bf16_to_f32(raw[i >> 2][i & 3] & 0xffffu);
+        v[2 * i + 1] = bf16_to_f32(raw[i >> 2][i & 3] >> 16);
     }
     float amax = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
     amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
     const int byte = mx_scale_byte(amax);
-    if (!live) return;
-    u32x2 out;
-    out[0] = pack4_e4m3(mx_scaled(v[0], byte), mx_scaled(v[1], byte), mx_scaled(v[2], byte), mx_scaled(v[3], byte));
-    out[1] = pack4_e4m3(mx_scaled(v[4], byte), mx_scaled(v[5], byte), mx_scaled(v[6], byte), mx_scaled(v[7], byte));
-    codes[u] = out;
-    if ((u & 3) == 0) scales[u >> 2] = static_cast<uint8_t>(byte);
-    (void)units_per_row;
+    if (live) {
+        u32x4 out;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            out[i] = pack4_e4m3(mx_scaled(v[4 * i], byte), mx_scaled(v[4 * i + 1], byte), mx_scaled(v[4 * i + 2], byte),
+                                mx_scaled(v[4 * i + 3], byte));
+        store16_through(codes + u, out);
+    }
+    if ((threadIdx.x & 1) == 0) staged[threadIdx.x >> 1] = static_cast<uint8_t>(byte);
+    __syncthreads();
+    // blocks (= scale bytes) of this workgroup: [first, first + 128) clipped to the end
+    const long long first = static_cast<long long>(blockIdx.x) * (kMxThreads / 2);
+    const long long num_blocks = num_units >> 1;
+    const int present = static_cast<int>(min(static_cast<long long>(kMxThreads / 2), num_blocks - first));
+    if (kVectorScales && present == kMxThreads / 2) {
+        if (threadIdx.x < kMxThreads / 32)
+            store16_through(scales + first + threadIdx.x * 16, *reinterpret_cast<const u32x4*>(staged + threadIdx.x * 16));
+    } else if (static_cast<int>(threadIdx.x) < present) {
+        scales[first + threadIdx.x] = staged[threadIdx.x];
+    }
 }
 
 // =====================================================================================================
@@ -228,6 +252,7 @@ struct GemmParams {
     const uint8_t* a_scales;   // [*, K/32] e8m0
     const int* row_to_route;   // first GEMM: source row = row_to_route[r] / topk
     int topk;
+    int a_rows;                // rows of a_codes (the gather clamps to them)
     const int* offsets;        // [L+1] exclusive row prefix per expert
     int num_local;
     const uint8_t* w;          // prepared fragments, expert stride N*K/2
@@ -244,8 +269,11 @@ struct GemmParams {
     // without a tile stream zeros into the output rows of the tokens that no local expert serves (most tokens of a
     // rank's share), which the weighted reduce would otherwise have to write after the GEMMs: the stores cost the
     // matrix pipes nothing.  Every wave of such a workgroup is a filler f and takes tokens f, f + fillers, ...
-    // until a workgroup with a tile reaches its epilogue and writes the launch's number into *fill_stop (a number,
-    // not a flag, so that nothing has to clear it and a word left over from an earlier launch stops nobody);
+    // until a workgroup with a tile reaches its epilogue and raises *fill_stop.  The word is a counter that only ever
+    // grows (device memory of the workspace): a filler remembers the value it found when it started and stops when
+    // the word differs, so nothing has to clear it, no value comes from the host, and every replay of a captured
+    // launch stops its own fillers.  (Launches on a workspace run one after the other, so a filler's first read sees
+    // every increment of the launches before it and none of its own launch: the first increment is a whole tile away.)
     // fill_state[0] = number of fillers, fill_state[1 + f] = tokens filler f got through.  All of it is null / zero in
     // launches that do not fill.
     u32x4* fill_out;                // [fill_tokens, fill_vec] or nullptr
@@ -253,7 +281,6 @@ struct GemmParams {
     int fill_tokens, fill_vec, fill_topk;
     int* fill_state;
     int* fill_stop;
-    int launch_id;                  // never 0
     int forced_rt;                  // 1..3: tile height 64 * forced_rt whatever the cost model says (tests); 0: the model decides
 };
 
@@ -417,8 +444,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
         const int filler = (first - total_tiles) * kGemmWaves + wave;
         const u32x4 zero = {0u, 0u, 0u, 0u};
         int done = 0;
+        const int stop_at_start = __hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         for (int token = filler; token < p.fill_tokens; token += fillers, ++done) {
-            if (__hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.launch_id) break;
+            if (__hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != stop_at_start) break;
             const bool mine = lane < p.fill_topk && p.fill_route_to_row[static_cast<size_t>(token) * p.fill_topk + lane] >= 0;
             if (__ballot(mine) != 0ull) continue;  // some local expert serves the token: the reduce writes its row
             u32x4* row = p.fill_out + static_cast<size_t>(token) * p.fill_vec;
@@ -465,13 +493,14 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 #pragma unroll
         for (int i = 0; i < 2 * RT; ++i) {
             const int r = min(i * 32 + wave * 8 + (lane >> 3), info.valid - 1);
-            const int src = kGather ? index[r] / p.topk : info.row0 + r;
+            // (clamped: a map left incomplete by a layout launch that ran out of time must not become a wild address)
+            const int src = kGather ? min(max(index[r] / p.topk, 0), p.a_rows - 1) : info.row0 + r;
             a_off[i] = static_cast<uint32_t>(src) * static_cast<uint32_t>(p.k) + a_chunk;
         }
         {
             // thread t serves row t % kBM (surplus waves repeat rows, which keeps every wave's copy count equal)
             const int r = min(tid % kBM, info.valid - 1);
-            const int src = kGather ? index[r] / p.topk : info.row0 + r;
+            const int src = kGather ? min(max(index[r] / p.topk, 0), p.a_rows - 1) : info.row0 + r;
             sa_src = p.a_scales + static_cast<size_t>(src) * scale_bytes;
         }
         const bool shared = info.expert >= p.num_routed;
@@ -631,7 +660,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
             // The last row tile of the epilogue is about what a filler needs to finish the row it is on: tell them to
             // stop (the first workgroup to get here does; the others are at most a few microseconds behind).
             if (i == RT - 1 && fillers != 0 && tid == 0)
-                __hip_atomic_store(p.fill_stop, p.launch_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(p.fill_stop, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int tile_rows = min(32, info.valid - wm * 32 * RT - 32 * i);  // may be <= 0
             const size_t out_row0 = static_cast<size_t>(info.row0) + wm * 32 * RT + 32 * i;
 #pragma unroll
@@ -855,11 +884,17 @@ template <int RT, bool kGateUp>
 int launch_gemm_rt(const GemmParams& p, hipStream_t stream, const char* what)
 {
     constexpr int kLds = GemmCfg<RT, kGateUp>::kLdsBytes;
-    static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
-    if (!configured) {
+    // Raising the dynamic LDS limit is a setting per function and per device (each device holds its own copy of the
+    // code object).  One flag per device; two threads that both find it clear both make the (idempotent) call.
+    constexpr int kMaxDevices = 64;
+    static std::atomic<bool> configured[kMaxDevices];
+    int device = 0;
+    DPEP_HIP(hipGetDevice(&device));
+    const bool tracked = device >= 0 && device < kMaxDevices;
+    if (!tracked || !configured[device].load(std::memory_order_acquire)) {
         DPEP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<RT, kGateUp>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-        configured = true;
+        if (tracked) configured[device].store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((grouped_gemm_kernel<RT, kGateUp>), dim3(gemm_grid()), dim3(kGemmThreads), kLds, stream, p);
     return launch_status(what);
@@ -1012,12 +1047,17 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
     DPEP_REQUIRE(rows >= 0, "mx_quant: bad row count %d", rows);
     DPEP_REQUIRE(hidden > 0 && hidden % 32 == 0, "mx_quant: hidden=%d must be a positive multiple of 32", hidden);
     if (rows == 0) return DPEP_OK;
-    DPEP_REQUIRE(x && codes && scales && aligned16(x) && (reinterpret_cast<uintptr_t>(codes) & 7u) == 0,
-                 "mx_quant: NULL or misaligned buffer");
-    const long long units = static_cast<long long>(rows) * (hidden / 8);
-    const unsigned blocks = static_cast<unsigned>((units + 255) / 256);
-    hipLaunchKernelGGL(mx_quant_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const u32x4*>(x), units, hidden / 8, static_cast<u32x2*>(codes), scales);
+    DPEP_REQUIRE(x && codes && scales && aligned16(x) && aligned16(codes), "mx_quant: NULL or misaligned buffer");
+    const long long units = static_cast<long long>(rows) * (hidden / 16);
+    DPEP_REQUIRE((units + kMxThreads - 1) / kMxThreads < (1ll << 31), "mx_quant: %d x %d values are more than one launch takes",
+                 rows, hidden);
+    const unsigned blocks = static_cast<unsigned>((units + kMxThreads - 1) / kMxThreads);
+    if (aligned16(scales))
+        hipLaunchKernelGGL(mx_quant_kernel<true>, dim3(blocks), dim3(kMxThreads), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const u32x4*>(x), units, static_cast<u32x4*>(codes), scales);
+    else
+        hipLaunchKernelGGL(mx_quant_kernel<false>, dim3(blocks), dim3(kMxThreads), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const u32x4*>(x), units, static_cast<u32x4*>(codes), scales);
     return launch_status("mx_quant");
 }
 
@@ -1108,6 +1148,28 @@ size_t dpep_megamoe_workspace_bytes(int num_tokens, int num_topk, int hidden, in
     return mega_layout(num_tokens, num_topk, hidden, intermediate, num_local, num_shared).total;
 }
 
+int dpep_megamoe_fill_report(void* ws, int num_tokens, int num_topk, int hidden, int intermediate, int num_local,
+                             int num_shared, int32_t* fillers_host, int64_t* tokens_filled_host, void* stream)
+{
+    using namespace dpep;
+    Workspace* w = as_workspace(ws);
+    DPEP_REQUIRE(w != nullptr && fillers_host != nullptr && tokens_filled_host != nullptr,
+                 "megamoe_fill_report: not a live workspace, or NULL output");
+    DPEP_REQUIRE(num_tokens >= 1 && num_topk >= 1 && hidden >= 1 && intermediate >= 1 && num_local >= 1 && num_shared >= 0,
+                 "megamoe_fill_report: bad sizes");
+    const MegaLayout l = mega_layout(num_tokens, num_topk, hidden, intermediate, num_local, num_shared);
+    DPEP_REQUIRE(l.total <= w->bytes, "megamoe_fill_report: these are not the sizes of a forward on this workspace");
+    static thread_local int32_t state[1 + 4096];
+    DPEP_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    DPEP_HIP(hipMemcpy(state, static_cast<uint8_t*>(w->base) + l.fill_state, sizeof(state), hipMemcpyDeviceToHost));
+    const int fillers = state[0] < 0 ? 0 : state[0] > 4096 ? 4096 : state[0];
+    int64_t filled = 0;
+    for (int f = 0; f < fillers; ++f) filled += state[1 + f];
+    *fillers_host = fillers;
+    *tokens_filled_host = filled;
+    return DPEP_OK;
+}
+
 int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales, const int32_t* topk_idx,
                          const float* topk_weights, const uint8_t* w1, const uint8_t* s1, const uint8_t* w2,
                          const uint8_t* s2, const uint8_t* shared_w1, const uint8_t* shared_s1,
@@ -1176,6 +1238,7 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     }
     g1.row_to_route = row_to_route;
     g1.topk = num_topk;
+    g1.a_rows = num_tokens;
     g1.offsets = offsets;
     g1.num_local = num_local + num_shared;
     g1.num_routed = num_local;
@@ -1196,8 +1259,6 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     // zero those rows of y meanwhile, and the weighted reduce skips what they got through.
     int* fill_state = reinterpret_cast<int*>(base + l.fill_state);
     int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->sync) + kSyncFillStop);
-    w->gemm_launches = w->gemm_launches >= 0x7fffffffu ? 1u : w->gemm_launches + 1u;  // never 0
-    g1.launch_id = static_cast<int>(w->gemm_launches);
     g1.forced_rt = w->gemm_tile_rows / 64;
     // (served-only: rows of y whose token no local expert serves are nobody's business, neither the fillers' nor the
     // reduce's; with shared experts every token is served)

@@ -74,7 +74,6 @@ int dpep_workspace_create(size_t bytes, void** ws)
     w->exchange_extra_rows = 0;
     w->layout_one_launch = 1;
     w->gemm_tile_rows = 0;
-    w->gemm_launches = 0;
     w->gemm_zero_fill = 1;
     w->megamoe_served_only = 0;
     w->layout_launches = 0;

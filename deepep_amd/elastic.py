@@ -472,42 +472,22 @@ class ElasticBuffer:
         if handle is None:
             # Path selection as in the reference (elastic.py:710-746): small batches on EP16+ with weights and
             # default options prefer the low-latency path, decided from host metadata only.
-            first = x[0] if isinstance(x, tuple) and len(x) == 2 else x
-            if isinstance(first, torch.Tensor) and first.ndim == 2:
-                capacity = (
-                    (self.num_max_tokens_per_rank or -(-first.shape[0] // runtime.world_size))
-                    if num_max_tokens_per_rank is None
-                    else num_max_tokens_per_rank
-                )
-                within_bound = type(capacity) is int and (
-                    not self.num_max_tokens_per_rank or capacity <= self.num_max_tokens_per_rank
-                )
-                ll_options = (
-                    within_bound
-                    and type(do_handle_copy) is bool
-                    and (do_cpu_sync is None or type(do_cpu_sync) is bool)
-                    and (do_expand is None or do_expand is True)
-                    and (expert_alignment is None or type(expert_alignment) is int and expert_alignment == 1)
-                    and type(num_sms) is int
-                    and num_sms == 0
-                    and type(num_qps) is int
-                    and num_qps == 0
-                    and cumulative_local_expert_recv_stats is None
-                    and previous_event is None
-                    and previous_event_before_epilogue is None
-                    and async_with_compute_stream is False
-                    and allocate_on_comm_stream is False
-                    and do_zero_padding is False
-                    and use_tma_aligned_col_major_sf is False
-                )
-                plan = self._low_latency_plan(x, topk_idx, topk_weights, num_experts, capacity) if ll_options else None
-                if plan is not None:
-                    if runtime.capacity != LOW_LATENCY_WORKSPACE_BYTES:
-                        raise ValueError(
-                            "LL dispatch requires Buffer(num_bytes=8589934592), exactly 8 GiB; "
-                            f"got {runtime.capacity} bytes for EP{runtime.world_size}"
-                        )
-                    return self._dispatch_low_latency(x, topk_idx, topk_weights, num_experts, capacity, do_handle_copy, plan)
+            options = dict(
+                do_handle_copy=do_handle_copy, do_cpu_sync=do_cpu_sync, do_expand=do_expand, expert_alignment=expert_alignment,
+                num_sms=num_sms, num_qps=num_qps, cumulative_local_expert_recv_stats=cumulative_local_expert_recv_stats,
+                previous_event=previous_event, previous_event_before_epilogue=previous_event_before_epilogue,
+                async_with_compute_stream=async_with_compute_stream, allocate_on_comm_stream=allocate_on_comm_stream,
+                do_zero_padding=do_zero_padding, use_tma_aligned_col_major_sf=use_tma_aligned_col_major_sf,
+            )
+            chosen = self._choose_low_latency(x, topk_idx, topk_weights, num_experts, num_max_tokens_per_rank, options)
+            if chosen is not None:
+                capacity, plan = chosen
+                if runtime.capacity != LOW_LATENCY_WORKSPACE_BYTES:
+                    raise ValueError(
+                        "LL dispatch requires Buffer(num_bytes=8589934592), exactly 8 GiB; "
+                        f"got {runtime.capacity} bytes for EP{runtime.world_size}"
+                    )
+                return self._dispatch_low_latency(x, topk_idx, topk_weights, num_experts, capacity, do_handle_copy, plan)
         with runtime.notify_lock:
             if runtime.notify_failed:
                 raise RuntimeError("A previous communication launch failed; restart the distributed job")
@@ -642,6 +622,47 @@ class ElasticBuffer:
             except Exception:
                 runtime.notify_failed = True
                 raise
+
+    # What each option of a fresh dispatch must be for the call to be eligible for the low-latency path
+    # (deep_ep/backends/mesh_clos/elastic.py:710-746 decides the same from host metadata alone): a type the value must
+    # have exactly (None: not checked), and the values accepted.
+    _LOW_LATENCY_OPTIONS = {
+        "do_handle_copy": (bool, (True, False)),
+        "do_cpu_sync": (None, (None, True, False)),
+        "do_expand": (None, (None, True)),
+        "expert_alignment": (None, (None, 1)),
+        "num_sms": (int, (0,)),
+        "num_qps": (int, (0,)),
+        "cumulative_local_expert_recv_stats": (None, (None,)),
+        "previous_event": (None, (None,)),
+        "previous_event_before_epilogue": (None, (None,)),
+        "async_with_compute_stream": (None, (False,)),
+        "allocate_on_comm_stream": (None, (False,)),
+        "do_zero_padding": (None, (False,)),
+        "use_tma_aligned_col_major_sf": (None, (False,)),
+    }
+
+    def _choose_low_latency(self, x, topk_idx, topk_weights, num_experts, num_max_tokens_per_rank, options):
+        """(capacity, plan) when a fresh dispatch takes the low-latency path, else None."""
+        payload = x[0] if isinstance(x, tuple) and len(x) == 2 else x
+        if not isinstance(payload, torch.Tensor) or payload.ndim != 2:
+            return None
+        declared = self.num_max_tokens_per_rank
+        if num_max_tokens_per_rank is not None:
+            capacity = num_max_tokens_per_rank
+        else:
+            capacity = declared or -(-payload.shape[0] // self._live_runtime().world_size)
+        if type(capacity) is not int or (declared and capacity > declared):
+            return None
+        for name, (exact_type, accepted) in self._LOW_LATENCY_OPTIONS.items():
+            value = options[name]
+            # identity or exact-type equality: 0 == False and 1 == True must not pass for each other
+            if exact_type is not None and type(value) is not exact_type:
+                return None
+            if not any(value is good or (type(value) is type(good) and value == good) for good in accepted):
+                return None
+        plan = self._low_latency_plan(x, topk_idx, topk_weights, num_experts, capacity)
+        return None if plan is None else (capacity, plan)
 
     def _low_latency_plan(self, x, topk_idx, topk_weights, num_experts, capacity):
         """Host-metadata check that selects the low-latency path (elastic.py:401-450); never reads routes.

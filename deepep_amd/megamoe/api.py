@@ -371,26 +371,22 @@ def fp8_fp4_mega_moe(y, l1_weights, l2_weights, sym_buffer, shared_l1_weights=No
     Inputs are the buffer's own x / x_sf / topk_idx / topk_weights (first y.shape[0] rows); ``x=`` is an
     optional BF16 [BS,H] override that is MX-quantised internally.  Route weights are applied after GMM2.
     """
-    if recipe != (1, 1, 32) or activation != "swiglu" or activation_clamp is not None or fast_math is not True:
+    fixed = {"recipe": (recipe, (1, 1, 32)), "activation": (activation, "swiglu"), "activation_clamp": (activation_clamp, None)}
+    if fast_math is not True or any(given != only for given, only in fixed.values()):
         raise NotImplementedError("Supports recipe=(1,1,32), SwiGLU, no clamp, default math only")
     if not isinstance(sym_buffer, SymmBuffer):
         raise TypeError("sym_buffer must be this installation's MegaMoE SymmBuffer")
     sym_buffer._ensure_alive()
-    if y.ndim != 2 or y.dtype != torch.bfloat16:
+    if not (y.ndim == 2 and y.dtype == torch.bfloat16):
         raise ValueError("y must be BF16 [BS,H]")
-    bs = y.shape[0]
-    if x is not None and (x.dtype != torch.bfloat16 or tuple(x.shape) != (bs, sym_buffer.hidden)):
+    batch = y.shape[0]
+    if x is None:
+        # the buffer's own staging tensors, as many rows as y has
+        activations = (sym_buffer.x[:batch], sym_buffer.x_sf[:batch])
+    elif x.dtype == torch.bfloat16 and tuple(x.shape) == (batch, sym_buffer.hidden):
+        activations = x
+    else:
         raise ValueError("x override must be BF16 [BS,H]; omit x for buffered FP8 input")
-    _run(
-        (sym_buffer.x[:bs], sym_buffer.x_sf[:bs]) if x is None else x,
-        sym_buffer.topk_idx[:bs],
-        sym_buffer.topk_weights[:bs],
-        l1_weights,
-        l2_weights,
-        sym_buffer,
-        shared_l1_weights=shared_l1_weights,
-        shared_l2_weights=shared_l2_weights,
-        out=y,
-        timer=timer,
-        cumulative_stats=cumulative_local_expert_recv_stats,
-    )
+    shared = dict(shared_l1_weights=shared_l1_weights, shared_l2_weights=shared_l2_weights)
+    _run(activations, sym_buffer.topk_idx[:batch], sym_buffer.topk_weights[:batch], l1_weights, l2_weights, sym_buffer,
+         out=y, timer=timer, cumulative_stats=cumulative_local_expert_recv_stats, **shared)

@@ -99,6 +99,19 @@ class Workspace:
                 _lib.check(self._lib.dpep_workspace_destroy(handle), "workspace_destroy")
 
 
+STORE_POLICIES = {"through": 0, "streaming": 1, "cached": 2}
+
+
+def dispatch_store_policy(policy: Optional[str] = None) -> str:
+    """Set (or, with no argument, read) how the dispatch kernels store their payload rows: ``"through"`` (default),
+    ``"streaming"`` or ``"cached"``.  Process-wide.  Returns the policy that was in force before the call."""
+    if policy is not None and policy not in STORE_POLICIES:
+        raise ValueError(f"dispatch_store_policy: {policy!r} is not one of {sorted(STORE_POLICIES)}")
+    code = _lib.load().dpep_dispatch_store_policy(3 if policy is None else STORE_POLICIES[policy])
+    _lib.check(min(code, 0), "dispatch_store_policy")
+    return {v: k for k, v in STORE_POLICIES.items()}[code]
+
+
 def layout_workspace_bytes(num_tokens: int, num_topk: int, num_local: int) -> int:
     return int(_lib.load().dpep_layout_workspace_bytes(num_tokens, num_topk, num_local))
 
@@ -438,6 +451,16 @@ def megamoe_prepare_weights(w_packed, w_scales, gate_up: bool):
         )
     _lib.check(status, "megamoe_prepare_weights")
     return out_w, out_s
+
+
+def megamoe_fill_report(ws, num_tokens, num_topk, hidden, intermediate, num_local, num_shared: int = 0):
+    """(filler waves, tokens they looked at) of the most recent forward on ``ws``; waits for the current stream."""
+    fillers, filled = ctypes.c_int32(0), ctypes.c_int64(0)
+    device = ws.device
+    status = _lib.load().dpep_megamoe_fill_report(ws.handle, num_tokens, num_topk, hidden, intermediate, num_local, num_shared,
+                                                  ctypes.byref(fillers), ctypes.byref(filled), _stream(device))
+    _lib.check(status, "megamoe_fill_report")
+    return fillers.value, filled.value
 
 
 def megamoe_forward(ws, x_codes, x_scales, topk_idx, topk_weights, w1, s1, w2, s2, num_experts, expert_begin,

@@ -12,11 +12,16 @@ from . import ops
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Quantise each group of 128 values to E4M3 with FP32 scales, on the GPU (HIP kernel).
 
-    Bit-identical to the reference's torch expression on CPU.  ``x`` must be a contiguous BF16 [T, H] GPU tensor with
-    H a multiple of 16; a last block shorter than 128 is quantised as if padded with zeros, as in the reference."""
+    Bit-identical to the reference's torch expression on CPU.  ``x`` is a BF16 [T, H] GPU tensor of any width: a last
+    block shorter than 128 is quantised as if padded with zeros, as in the reference (the kernel takes widths that
+    are multiples of 16; other widths are padded to the next one here and the codes cut back to H)."""
     if x.dim() != 2:
         raise AssertionError("x must be a 2D tensor")
-    return ops.cast_to_fp8(x)
+    hidden = x.shape[1]
+    if hidden % 16 == 0 or hidden == 0:
+        return ops.cast_to_fp8(x)
+    codes, scales = ops.cast_to_fp8(torch.nn.functional.pad(x, (0, 16 - hidden % 16)))
+    return codes[:, :hidden].contiguous(), scales
 
 
 def per_token_cast_back(x_fp8: torch.Tensor, x_scales: torch.Tensor) -> torch.Tensor:

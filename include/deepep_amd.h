@@ -111,6 +111,20 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
                        int num_topk, int num_rows, int row_bytes, int scale_cols, void* out,
                        float* out_scales, float* out_weights, void* stream);
 
+/* How dpep_dispatch_copy, dpep_dispatch_quant_fp8 and dpep_cast_to_fp8 store their payload rows; process-wide, no
+ * counterpart in the reference (its rows leave through the transport).  Returns the policy in force before the call
+ * (DPEP_STORE_QUERY changes nothing), or DPEP_EINVAL.
+ *   DPEP_STORE_THROUGH    (default) write-through stores: the same kernel time whether the caches held the input, other
+ *                         tensors' clean lines or the previous call's output when the launch started
+ *   DPEP_STORE_STREAMING  non-temporal stores past the caches: fastest when one buffer is dispatched again and again
+ *                         (the input then stays cached between calls), slowest when the input is cold
+ *   DPEP_STORE_CACHED     plain stores */
+#define DPEP_STORE_THROUGH 0
+#define DPEP_STORE_STREAMING 1
+#define DPEP_STORE_CACHED 2
+#define DPEP_STORE_QUERY 3
+int dpep_dispatch_store_policy(int policy);
+
 /* Fused per-128-element FP8 e4m3fn quantisation + expand-permute: the reference's caller-side
  * per_token_cast_to_fp8 (deep_ep/utils/math.py:45-61) followed by the FP8 dispatch above, in one pass.
  *   x             bf16 [T,H], H % 128 == 0
@@ -214,6 +228,13 @@ int dpep_megamoe_prepared_shape(int n, int k, int gate_up, int* padded_n, int* p
  * SwiGLU is lane-local (the counterpart of _interleave_gate_up_128, api.py:285-293). */
 int dpep_megamoe_prepare_weights(const uint8_t* w_packed, const uint8_t* w_scales, int num_local, int n,
                                  int k, int gate_up, uint8_t* out_packed, uint8_t* out_scales, void* stream);
+
+/* Diagnosis, no counterpart in the reference: what the idle workgroups of the most recent dpep_megamoe_forward's first
+ * GEMM did (see "gemm_zero_fill").  Waits for `stream`, then reports the number of filler waves of that launch (0: the
+ * launch had a tile for every workgroup, or zero fill is off) and the tokens they looked at before they were told to
+ * stop.  The sizes are those of the forward call. */
+int dpep_megamoe_fill_report(void* ws, int num_tokens, int num_topk, int hidden, int intermediate, int num_local,
+                             int num_shared, int32_t* fillers_host, int64_t* tokens_filled_host, void* stream);
 
 /* Fused W4A8 MoE forward for one rank's local experts (Plan::forward, experiments/megamoe/csrc/forward.cpp:340-478
  * -> mega_moe_kernel_do, kernel_launch.hpp:8-13):

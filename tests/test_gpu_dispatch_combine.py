@@ -231,6 +231,19 @@ def test_cast_to_fp8_short_last_block(ops, tokens, hidden):
     np.testing.assert_array_equal(f32_bits(s), f32_bits(s_ref))
 
 
+@pytest.mark.parametrize("tokens,hidden", [(7, 200), (3, 5), (2, 129), (4, 7168 + 33)])
+def test_per_token_cast_to_fp8_any_width(tokens, hidden):
+    """The public helper takes any width, like the reference's (deep_ep/utils/math.py:44-61 zero-pads to 128)."""
+    from deepep_amd.utils import per_token_cast_to_fp8
+
+    x = (torch.randn(tokens, hidden, generator=torch.Generator().manual_seed(hidden)) * 2).bfloat16()
+    q_ref, s_ref = oquant.cast_to_fp8_torch(torch.nn.functional.pad(x, (0, (-hidden) % 128)))
+    q, s = per_token_cast_to_fp8(x.cuda())
+    assert tuple(q.shape) == (tokens, hidden) and q.is_contiguous() and tuple(s.shape) == (tokens, (hidden + 127) // 128)
+    np.testing.assert_array_equal(fp8_bits(q), fp8_bits(q_ref)[:, :hidden])
+    np.testing.assert_array_equal(f32_bits(s), f32_bits(s_ref))
+
+
 def _finite_codes(shape, seed):
     codes = np.random.default_rng(seed).integers(0, 256, shape, dtype=np.uint8)
     codes[(codes & 0x7F) == 0x7F] = 0x7E  # 0x7F / 0xFF are NaN in e4m3fn; checked apart
@@ -394,6 +407,55 @@ def test_full_size_prefill_properties(ops, ws):
     rows_bf16, _, _ = ops.dispatch_copy(xi, None, None, got["route_to_row"], got["row_to_route"], rows)
     back, _ = ops.combine(rows_bf16, got["route_to_row"])
     assert torch.equal(back.float(), xi.float() * 8)
+
+
+def test_full_size_rank_share_properties(ops, ws):
+    """The EP64 rank share at full size (64 x 256 = 16384 candidate tokens, 6 of 384 experts local, top-8, H=7168; the
+    reference runs its payload checks at the configured size, tests/elastic/test_dispatch.py:1670-1908): the sparse-share
+    kernels (row-major fused FP8 dispatch, served-only combine) against size-independent properties.  Rows of the
+    fused dispatch equal the stand-alone quantiser's rows of their tokens; BF16 rows equal their tokens; the weighted
+    combine of integer-valued rows is exact and can be stated per token; the served-only combine gives served tokens
+    the full combine's rows and leaves the others untouched."""
+    x, idx, w, cfg = cases.make_inputs("C4")
+    tokens, hidden, topk = cfg["tokens"], cfg["hidden"], cfg["topk"]
+    assert tokens == 16384 and hidden == 7168
+    got, want, rows = _check_layout(ops, ws, idx.numpy(), cfg["experts"], cfg["expert_begin"], cfg["num_local"])
+    assert 1500 < rows < 2600 and rows <= tokens  # sparse share: the row-major kernels run
+    xd, wd = x.cuda(), w.cuda()
+    route = got["row_to_route"][:rows].long()
+    token_of_row = route // topk
+    q, s = ops.cast_to_fp8(xd)
+    out, out_s, out_w = ops.dispatch_quant_fp8(xd, wd, got["route_to_row"], got["row_to_route"], rows)
+    assert torch.equal(out.view(torch.uint8), q.view(torch.uint8)[token_of_row])
+    assert torch.equal(out_s.view(torch.int32), s.view(torch.int32)[token_of_row])
+    assert torch.equal(out_w.view(torch.int32), wd.view(-1).view(torch.int32)[route])
+    # the pre-quantised copy and the BF16 copy move the same rows
+    cq, cs, _ = ops.dispatch_copy(q, s, None, got["route_to_row"], got["row_to_route"], rows)
+    assert torch.equal(cq.view(torch.uint8), out.view(torch.uint8)) and torch.equal(cs.view(torch.int32), out_s.view(torch.int32))
+    xi = torch.randint(-8, 9, x.shape, generator=torch.Generator().manual_seed(2)).bfloat16().cuda()
+    rows_bf16, _, _ = ops.dispatch_copy(xi, None, None, got["route_to_row"], got["row_to_route"], rows)
+    assert torch.equal(rows_bf16.view(torch.int16), xi.view(torch.int16)[token_of_row])
+    # weights k / 4 and |x| <= 8: every product and partial sum is exact, so the combine is x * (sum of the weights of
+    # the token's local slots) whatever the order
+    slot_w = ((torch.arange(rows) % 4 + 1).float() / 4).cuda()
+    local = got["route_to_row"] >= 0
+    weight_sum = torch.zeros(tokens, device="cuda")
+    weight_sum.index_add_(0, token_of_row, slot_w)
+    full, _ = ops.combine(rows_bf16, got["route_to_row"], slot_w)
+    assert torch.equal(full.float(), xi.float() * weight_sum[:, None])
+    served = local.any(dim=1)
+    assert 0 < int(served.sum()) < tokens
+    sentinel = torch.full((tokens, hidden), 7.0, dtype=torch.bfloat16, device="cuda")
+    part, _ = ops.combine(rows_bf16, got["route_to_row"], slot_w, out=sentinel.clone(), served_only=True)
+    assert torch.equal(part[served].view(torch.int16), full[served].view(torch.int16))
+    assert torch.equal(part[~served], sentinel[~served]) and not full[~served].any()
+    # N(0,1) rows: no closed form, but the two combines must still agree on the served tokens, unweighted too
+    y = torch.randn(rows, hidden, generator=torch.Generator().manual_seed(3)).bfloat16().cuda()
+    for row_w in (None, out_w):
+        full, _ = ops.combine(y, got["route_to_row"], row_w)
+        part, _ = ops.combine(y, got["route_to_row"], row_w, out=sentinel.clone(), served_only=True)
+        assert torch.equal(part[served].view(torch.int16), full[served].view(torch.int16))
+        assert torch.equal(part[~served], sentinel[~served])
 
 
 def test_argument_errors(ops, ws):

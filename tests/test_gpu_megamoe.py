@@ -31,6 +31,31 @@ def test_mx_quant_bit_exact(ops, scale):
     np.testing.assert_array_equal(fp8_bits(codes), ref_codes)
 
 
+@pytest.mark.parametrize("rows,hidden", [(1, 32), (3, 96), (5, 4096), (129, 160), (64, 7168), (2, 8192 + 32)])
+@pytest.mark.parametrize("scale_offset", [0, 1, 4])
+def test_mx_quant_ragged_sizes_and_unaligned_scales(ops, rows, hidden, scale_offset):
+    """Sizes that end inside a workgroup's 4096 values, and scale pointers off the 16-byte grid (the kernel then
+    stores byte by byte), called through the C-ABI with caller-owned buffers."""
+    import ctypes
+
+    from deepep_amd import _lib
+
+    gen = torch.Generator().manual_seed(rows * 131 + hidden)
+    x = (torch.randn(rows, hidden, generator=gen) * 3.0).bfloat16().cuda()
+    codes = torch.zeros(rows * hidden, dtype=torch.uint8, device="cuda")
+    store = torch.full((rows * (hidden // 32) + 32,), 0xEE, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    status = _lib.load().dpep_mx_quant(ctypes.c_void_p(x.data_ptr()), rows, hidden, ctypes.c_void_p(codes.data_ptr()),
+                                       ctypes.c_void_p(store.data_ptr() + scale_offset), ctypes.c_void_p(stream))
+    _lib.check(status, "mx_quant")
+    ref_codes, ref_scales = mm.mx_quantize(x.float().cpu().numpy())
+    got = store.cpu().numpy()
+    n = rows * (hidden // 32)
+    np.testing.assert_array_equal(got[scale_offset:scale_offset + n].reshape(rows, -1), ref_scales)
+    assert (got[:scale_offset] == 0xEE).all() and (got[scale_offset + n:] == 0xEE).all()  # nothing written outside
+    np.testing.assert_array_equal(codes.cpu().numpy().reshape(rows, hidden), ref_codes)
+
+
 def test_mx_quant_reference_anchors(ops):
     # experiments/megamoe/tests/test_reference.py:37-45
     x = torch.full((2, 64), 0.5)
@@ -360,6 +385,70 @@ def test_megamoe_forward_in_hip_graph(ops):
                 torch.cuda.synchronize()
                 graph.replay()
                 torch.cuda.synchronize()
+                assert torch.equal(counts, want_counts)
+                assert torch.equal(y.view(torch.int16), want_y.view(torch.int16)), f"replay {turn} differs from eager"
+    finally:
+        torch.cuda.synchronize()
+        ws.destroy()
+
+
+def test_megamoe_forward_in_hip_graph_keeps_its_fillers(ops):
+    """A rank's share (most tokens unserved, fewer tiles than workgroups) captured once and replayed: on every replay the
+    idle workgroups of the first GEMM must again zero rows of unserved tokens (their stop signal is a device-side
+    counter, not a value fixed at capture), and every replay must equal the eager forward bit for bit."""
+    tokens, hidden, inter, experts, begin, local, topk = 1536, 512, 512, 64, 8, 2, 4
+    dev = "cuda"
+    problems = [_make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=s) for s in (21, 22, 23)]
+    _, _, l1, l2, _, _ = problems[0]
+    w1, s1 = ops.megamoe_prepare_weights(torch.from_numpy(l1[0]).to(dev), torch.from_numpy(l1[1]).reshape(local, 2 * inter, -1).to(dev), True)
+    w2, s2 = ops.megamoe_prepare_weights(torch.from_numpy(l2[0]).to(dev), torch.from_numpy(l2[1]).reshape(local, hidden, -1).to(dev), False)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local))
+    x_codes = torch.empty((tokens, hidden), dtype=torch.uint8, device=dev)
+    x_scales = torch.empty((tokens, hidden // 32), dtype=torch.uint8, device=dev)
+    idx = torch.empty((tokens, topk), dtype=torch.int32, device=dev)
+    weights = torch.empty((tokens, topk), dtype=torch.float32, device=dev)
+    y = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+
+    def load(problem):
+        codes, scales, _, _, ids, wts = problem
+        x_codes.copy_(torch.from_numpy(codes)); x_scales.copy_(torch.from_numpy(scales))
+        idx.copy_(torch.from_numpy(ids)); weights.copy_(torch.from_numpy(wts))
+
+    def forward():
+        ops.megamoe_forward(ws, x_codes.view(torch.float8_e4m3fn), x_scales, idx, weights, w1, s1, w2, s2, experts, begin, local, y, counts)
+
+    def report():
+        return ops.megamoe_fill_report(ws, tokens, topk, hidden, inter, local)
+
+    try:
+        eager = []
+        for problem in problems:
+            load(problem)
+            y.fill_(float("nan"))
+            forward()
+            torch.cuda.synchronize()
+            fillers, filled = report()
+            assert fillers > 0 and filled > 0, (fillers, filled)
+            eager.append((y.clone(), counts.clone()))
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            forward()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            forward()
+        for turn in range(2):
+            for problem, (want_y, want_counts) in zip(problems, eager):
+                load(problem)
+                y.fill_(float("nan"))
+                torch.cuda.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                fillers, filled = report()
+                assert fillers > 0 and filled > 0, f"replay {turn}: {fillers} fillers looked at {filled} tokens"
                 assert torch.equal(counts, want_counts)
                 assert torch.equal(y.view(torch.int16), want_y.view(torch.int16)), f"replay {turn} differs from eager"
     finally:
