@@ -455,7 +455,7 @@ def main():
                         help="also launch a plain copy of known size (identity dispatch of [32768,7168] BF16: 469.76 MB "
                         "read + 469.76 MB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled")
     parser.add_argument("--dispatch-stores", choices=("through", "streaming", "cached"),
-                        help="store policy of the dispatch kernels (default: the library's, write-through)")
+                        help="store policy of the dispatch kernels (default: the library's, streaming)")
     parser.add_argument("--ingest-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"))
     parser.add_argument("--protocol", metavar="PRESET", help="run the reference's generic benchmark workload PRESET "
                         "(smoke, decode, prefill) and print one `measured` record per operation")

@@ -1,7 +1,7 @@
 // Expand-permute payload dispatch: out[row(t,s)] = x[t] for every route that owns a row, optionally
 // fused with the per-128-element FP8 e4m3fn block quantiser.  HBM-bound: 16-byte coalesced loads,
 // 16-byte stores, each input row read once and written to its K destinations.  How the token-major kernels store
-// is a process-wide policy (dpep_dispatch_store_policy): write-through by default, streaming or cached on request.
+// is a process-wide policy (dpep_dispatch_store_policy): streaming by default, write-through or cached on request.
 //
 // Observable contract: tests/elastic/test_dispatch.py:1391-1416 (payload, scales and weights arrive
 // bit-exactly in row order), tests/clos/common.py:276-279; quantiser deep_ep/utils/math.py:45-61.
@@ -19,13 +19,15 @@ constexpr int kTargetBlocks = 8192;  // rows are split into column parts until a
 constexpr int kMaxScaleCols = 1024;  // hidden <= 131072 for the fused quantiser
 constexpr int kRowMajorRatio = 1;  // row-major kernels when rows <= ratio * tokens
 
-// Store policy of the token-major kernels' payload rows.  Write-through (device-scope `sc1`): the rows pass through the
-// memory-side cache on their way to HBM, which takes the kernel's time the same way whatever the caches held before
-// the launch (clean lines of other tensors, the input just produced, or the kernel's own previous output).  Streaming
-// (non-temporal): the rows go to HBM past the caches at the streaming-write rate; the input stays cached from one call to
-// the next, so a loop that dispatches the same buffer again and again is faster this way and a call whose input is
-// cold is slower.  Cached: plain stores.
-int g_store_policy = DPEP_STORE_THROUGH;
+// Store policy of the payload rows.  Streaming (non-temporal, the default): the rows go to HBM past the caches at the
+// streaming-write rate, and the kernel's time is the time of its traffic.  Write-through (device-scope `sc1`) and cached
+// stores let the 256 MiB memory-side cache take the rows first: the kernel itself ends sooner when that cache holds clean
+// lines at launch, but the rows still have to reach HBM, and whatever runs next pays for it (measured at T=4096, H=7168,
+// top-8: the fused FP8 dispatch after a read-only sweep of 256 MiB takes 59.6 us streaming and 49.5 us write-through; with
+// the sweep that follows charged to it, 60.9 against 85.9 us; inside a dispatch + combine loop 49.6 against 69.8 us, and the
+// combine behind it 88.3 against 101.6 us).  A caller whose next kernel reads the rows while they are still in the
+// memory-side cache may still prefer write-through, hence the knob.
+int g_store_policy = DPEP_STORE_STREAMING;
 
 template <int kPolicy>
 __device__ __forceinline__ void store16_as(void* p, u32x4 v)
@@ -40,9 +42,9 @@ template <typename Launch>
 void with_store_policy(Launch&& launch)
 {
     switch (__atomic_load_n(&g_store_policy, __ATOMIC_RELAXED)) {
-    case DPEP_STORE_STREAMING: launch(std::integral_constant<int, DPEP_STORE_STREAMING>{}); break;
+    case DPEP_STORE_THROUGH: launch(std::integral_constant<int, DPEP_STORE_THROUGH>{}); break;
     case DPEP_STORE_CACHED: launch(std::integral_constant<int, DPEP_STORE_CACHED>{}); break;
-    default: launch(std::integral_constant<int, DPEP_STORE_THROUGH>{}); break;
+    default: launch(std::integral_constant<int, DPEP_STORE_STREAMING>{}); break;
     }
 }
 

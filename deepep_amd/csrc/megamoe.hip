@@ -60,7 +60,9 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 // consecutive vectors); two adjacent lanes own one 32-element block.  The workgroup's 128 scale bytes are staged in LDS
 // and leave as eight 16-byte stores instead of one byte-wide store per block, which turned every scale row into
 // read-modify-write traffic.  The tensors are treated as flat arrays: hidden is a multiple of 32, so blocks never
-// straddle rows.  kVectorScales: the scale pointer is 16-byte aligned.
+// straddle rows.  Input and codes stream past the caches (the input is read once; with cached loads the kernel's time
+// depended on what the caches held before: 48 us back to back, 89 us behind a 256 MiB fill, against 58-63 us this way
+// under every protocol).  kVectorScales: the scale pointer is 16-byte aligned.
 constexpr int kMxThreads = 256;
 
 template <bool kVectorScales>
@@ -72,8 +74,8 @@ __global__ __launch_bounds__(kMxThreads) void mx_quant_kernel(const u32x4* __res
     const bool live = u < num_units;
     u32x4 raw[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
     if (live) {
-        raw[0] = load16(x + 2 * u);
-        raw[1] = load16(x + 2 * u + 1);
+        raw[0] = load16_nt(x + 2 * u);
+        raw[1] = load16_nt(x + 2 * u + 1);
     }
     float v[16];
 #pragma unroll
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(kMxThreads) void mx_quant_kernel(const u32x4* __res
         for (int i = 0; i < 4; ++i)
             out[i] = pack4_e4m3(mx_scaled(v[4 * i], byte), mx_scaled(v[4 * i + 1], byte), mx_scaled(v[4 * i + 2], byte),
                                 mx_scaled(v[4 * i + 3], byte));
-        store16_through(codes + u, out);
+        store16_nt(codes + u, out);
     }
     if ((threadIdx.x & 1) == 0) staged[threadIdx.x >> 1] = static_cast<uint8_t>(byte);
     __syncthreads();

@@ -103,8 +103,8 @@ STORE_POLICIES = {"through": 0, "streaming": 1, "cached": 2}
 
 
 def dispatch_store_policy(policy: Optional[str] = None) -> str:
-    """Set (or, with no argument, read) how the dispatch kernels store their payload rows: ``"through"`` (default),
-    ``"streaming"`` or ``"cached"``.  Process-wide.  Returns the policy that was in force before the call."""
+    """Set (or, with no argument, read) how the dispatch kernels store their payload rows: ``"streaming"`` (default),
+    ``"through"`` or ``"cached"``.  Process-wide.  Returns the policy that was in force before the call."""
     if policy is not None and policy not in STORE_POLICIES:
         raise ValueError(f"dispatch_store_policy: {policy!r} is not one of {sorted(STORE_POLICIES)}")
     code = _lib.load().dpep_dispatch_store_policy(3 if policy is None else STORE_POLICIES[policy])

@@ -114,10 +114,11 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
 /* How dpep_dispatch_copy, dpep_dispatch_quant_fp8 and dpep_cast_to_fp8 store their payload rows; process-wide, no
  * counterpart in the reference (its rows leave through the transport).  Returns the policy in force before the call
  * (DPEP_STORE_QUERY changes nothing), or DPEP_EINVAL.
- *   DPEP_STORE_THROUGH    (default) write-through stores: the same kernel time whether the caches held the input, other
- *                         tensors' clean lines or the previous call's output when the launch started
- *   DPEP_STORE_STREAMING  non-temporal stores past the caches: fastest when one buffer is dispatched again and again
- *                         (the input then stays cached between calls), slowest when the input is cold
+ *   DPEP_STORE_STREAMING  (default) non-temporal stores: the rows go to HBM past the caches, the kernel's time is the
+ *                         time of its traffic and nothing is left for the next kernel to write back
+ *   DPEP_STORE_THROUGH    write-through stores: the memory-side cache takes the rows first, so the kernel itself ends
+ *                         sooner when that cache is clean and the kernel that follows pays for the write-back, unless it
+ *                         is the reader of those rows and finds them there
  *   DPEP_STORE_CACHED     plain stores */
 #define DPEP_STORE_THROUGH 0
 #define DPEP_STORE_STREAMING 1
