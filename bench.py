@@ -143,14 +143,47 @@ class Timer:
         pick = lambda q: times[min(len(times) - 1, int(q * len(times)))]
         return dict(mean=sum(times) / len(times), min=times[0], p50=pick(0.5), p95=pick(0.95))
 
-    def kernel(self, fn, nbytes, head_start=False, extra=None, read_sweep=False):
+    def drained(self, fn):
+        """Mean microseconds of [launch, read-only sweep of 256 MiB] after such a sweep, minus a sweep that follows a
+        sweep: the launch with whatever it leaves in the caches for later (dirty lines of write-through or cached
+        stores, which the next kernel would have to write back) charged to it."""
+        torch = self.torch
+        if self.flush is None:
+            self.flush = torch.zeros(FLUSH_BYTES, dtype=torch.uint8, device="cuda")
+        sweep = lambda: self.flush.view(torch.int64).sum()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(3):
+            sweep()
+        start.record()
+        for _ in range(self.iters):
+            sweep()
+        stop.record()
+        torch.cuda.synchronize()
+        alone = start.elapsed_time(stop) * 1000.0 / self.iters
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(self.iters)]
+        with self.no_collector():
+            for begin, end in pairs:
+                sweep()
+                begin.record()
+                fn()
+                sweep()
+                end.record()
+            torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) * 1000.0 for a, b in pairs) / len(pairs) - alone
+
+    def kernel(self, fn, nbytes, head_start=False, extra=None, read_sweep=False, drain=False):
         """One `kernels` entry: flushed statistics, the back-to-back figure, and GB/s of both against 8 TB/s.
-        read_sweep: also the statistics after a read-only flush (`after_read_sweep_us`)."""
+        read_sweep: also the statistics after a read-only flush (`after_read_sweep_us`); drain: and with the sweep that
+        follows charged to the launch (`after_read_sweep_with_drain_us`)."""
         warm = self.back_to_back(fn, head_start)
         cold = self.flushed(fn)
         if read_sweep:
             swept = self.flushed(fn, read_sweep=True)
             extra = dict(extra or {}, after_read_sweep_us=swept, frac_after_read_sweep=nbytes / swept["mean"] / 1e3 / HBM_PEAK_GBS)
+        if drain:
+            with_drain = self.drained(fn)
+            extra = dict(extra or {}, after_read_sweep_with_drain_us=with_drain,
+                         frac_after_read_sweep_with_drain=nbytes / with_drain / 1e3 / HBM_PEAK_GBS)
         entry = dict(
             bytes=nbytes,
             us=cold["mean"],
@@ -529,12 +562,19 @@ def main():
     copy_dispatch_bytes = tokens * (hidden + (hidden // 128) * 4) + tokens * topk * 4 + rows * (hidden + (hidden // 128) * 4 + 4)
     kernels = {
         "layout": timer.kernel(lambda: ops.layout(ws, idxd, experts), nbytes["layout"], head_start=True, read_sweep=True),
-        "dispatch_fp8_quant": timer.kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), nbytes["dispatch"], read_sweep=True),
+        "dispatch_fp8_quant": timer.kernel(lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), nbytes["dispatch"], read_sweep=True, drain=True),
         "dispatch_fp8_copy": timer.kernel(lambda: ops.dispatch_copy(q_pre, s_pre, wd, r2row, r2route, rows), copy_dispatch_bytes, read_sweep=True),
         "dispatch_bf16": timer.kernel(lambda: ops.dispatch_copy(xd, None, wd, r2row, r2route, rows), bf16_dispatch_bytes, read_sweep=True),
         "combine": timer.kernel(lambda: ops.combine(grows, r2row, out=out_buf), nbytes["combine"], read_sweep=True),
         "combine_weighted": timer.kernel(lambda: ops.combine(grows, r2row, recv_w, out=out_buf), nbytes["combine"] + rows * 4, read_sweep=True),
     }
+    # The same fused dispatch under the write-through store policy: it ends sooner behind a read sweep because the
+    # memory-side cache takes its rows, and leaves their write-back to whatever runs next (`..._with_drain_us`).
+    before = ops.dispatch_store_policy("through")
+    kernels["dispatch_fp8_quant_write_through"] = timer.kernel(
+        lambda: ops.dispatch_quant_fp8(xd, wd, r2row, r2route, rows), nbytes["dispatch"], read_sweep=True, drain=True,
+        extra={"note": "not the default: dpep_dispatch_store_policy(DPEP_STORE_THROUGH)"})
+    ops.dispatch_store_policy(before)
     # the stand-alone quantiser on the batch's tokens and the dequantiser on its dispatched rows (checking-side kernels of
     # the reference: per_token_cast_to_fp8 / per_token_cast_back)
     recv_q, recv_s, _ = ops.dispatch_copy(q_pre, s_pre, None, r2row, r2route, rows)

@@ -54,6 +54,7 @@ struct Workspace {
     int gemm_zero_fill;        // 1 (default): idle workgroups of the first GEMM zero rows of unserved tokens; 0: the reduce does
     int megamoe_served_only;   // 1: rows of y whose token no local expert serves are left untouched; 0 (default): zeroed
     int gemm_tile_rows;  // 0: the grouped GEMM chooses its tile height; 64 / 128 / 192: forced (tests)
+    int gemm_column_waves;  // which grouped GEMM kernel runs: 1 = waves split the columns, weights straight to registers; 0 = 2 x 2 waves, weights through LDS
 };
 // Device memory the kernels synchronise through, behind the caller's bytes, zero when the workspace is created:
 // at offset 0 the one-launch layout's epoch (64 bits: the highest tag any launch has used; a launch tags what it

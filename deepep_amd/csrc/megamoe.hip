@@ -12,6 +12,8 @@
 //   scales: lane l supplies the e8m0 byte of (row or column l%32, 32-wide k block l/32)
 //   D: acc[j] is row (j/4)*8 + (l/32)*4 + j%4, column l%32
 #include <atomic>
+#include <type_traits>
+#include <utility>
 
 #include "common.h"
 #include "gemm_schedule.h"
@@ -31,6 +33,19 @@ namespace {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose counter is a compile-time constant in
+// the body (register arrays and instruction immediates are indexed by it).
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_each(F&& f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    static_for_each(f, std::make_integer_sequence<int, N>{});
+}
 
 // =====================================================================================================
 // MXFP8 activation quantiser (block 32 along the row)
@@ -284,6 +299,7 @@ struct GemmParams {
     int* fill_state;
     int* fill_stop;
     int forced_rt;                  // 1..3: tile height 64 * forced_rt whatever the cost model says (tests); 0: the model decides
+    int column_waves;               // 1: the kernel whose waves split the tile's columns and load their weights straight into registers
 };
 
 // gate / (1 + exp(-gate)) * up with the hardware exponential and reciprocal (about 1 ulp each; the
@@ -328,6 +344,11 @@ __device__ __forceinline__ void copy16_weights_to_lds(const void* uniform_base, 
                      "s"(uniform_base)
                      : "memory");
 }
+__device__ __forceinline__ void copy4_to_lds(const void* uniform_base, uint32_t lane_offset, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(base), "v"(lane_offset), "s"(uniform_base) : "memory");
+}
 __device__ __forceinline__ void copy4_to_lds(const void* src, uint32_t lds_base)
 {
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
@@ -343,6 +364,16 @@ __device__ __forceinline__ void copy16_to_lds_unless(const void* src, uint32_t l
         "s_mov_b32 m0, %0\n\ts_cmp_lg_u32 %2, 0\n\ts_cbranch_scc1 .Lskip_copy_%=\n\t"
         "global_load_lds_dwordx4 %1, off\n.Lskip_copy_%=:" ::"s"(base),
         "v"(src), "s"(flag)
+        : "memory", "scc");
+}
+__device__ __forceinline__ void copy4_to_lds_unless(const void* uniform_base, uint32_t lane_offset, uint32_t lds_base, int skip)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    const int flag = __builtin_amdgcn_readfirstlane(skip);
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_cmp_lg_u32 %3, 0\n\ts_cbranch_scc1 .Lskip_copy_%=\n\t"
+        "global_load_lds_dword %1, %2\n.Lskip_copy_%=:" ::"s"(base),
+        "v"(lane_offset), "s"(uniform_base), "s"(flag)
         : "memory", "scc");
 }
 __device__ __forceinline__ void copy4_to_lds_unless(const void* src, uint32_t lds_base, int skip)
@@ -844,6 +875,543 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     wait_copies_then_barrier<0>();
 }
 
+// =====================================================================================================
+// Grouped GEMM, column-wave form: the weights go straight from memory to registers
+// =====================================================================================================
+// The prepared weight layout already is the per-lane B operand of the scaled MFMA, so a wave that owns whole
+// 32-column tiles can load its weight fragments with plain 16-byte loads and never share them.  Here the four waves
+// split the tile's 256 columns (64 each: two column tiles; for the first GEMM one gate / up pair) and every wave covers
+// ALL the tile's rows (2 * RT row tiles of 32): the same RT * 4 accumulator tiles per wave as the 2 x 2 form, but the
+// weights need no LDS write, no LDS read and no barrier, and the LDS ring holds activations only (8 KiB * RT per
+// stage), which buys a fourth stage at 192 rows.  The ring has exactly as many stages as the item loop is unrolled
+// (4): an item's stage, its weight registers and the selection of its scale bytes are all compile-time constants,
+// the LDS target of a copy is one scalar add away from a per-wave base, and a tile ends only behind the fourth body
+// (k is a multiple of 512 here).  Everything of item i + 4 is requested in the body of item i, so the one counted wait
+// per item lets two whole items of copies and loads stay in flight.
+// The weight fragments of the four items in flight live in the 64 accumulation registers behind the accumulators (a[192:255]
+// at 192 rows), which the loads and the
+// MFMAs name themselves: the compiler never sees them as values.  It could not be trusted with them: a register that
+// an asynchronous load has been told to fill counts as defined right behind the load, and a register allocator that moves
+// such a value (it parked weight fragments in spare registers when they were ordinary operands) copies what the register
+// held BEFORE the load landed.  Every weight load declares all 64 clobbered, so nothing the compiler keeps alive in
+// the loop can sit there (the accumulators end up below); that it also puts no short-lived value
+// there is checked on the generated code by tests/test_gemm_registers.py.  Column scales travel through LDS like the row
+// scales (each wave copies and reads only the 1 KiB of its own two column tiles).
+template <int RT>
+struct ColCfg {
+    static constexpr int kBM = 64 * RT;
+    static constexpr int kRowTiles = 2 * RT;           // 32-row MFMA tiles per workgroup tile, all of them on every wave
+    static constexpr int kColTiles = 2;                // 32-column MFMA tiles per wave
+    static constexpr int kStages = 4;                  // LDS stages = items the requests run ahead = unroll of the item loop
+    static constexpr int kStageBytes = kBM * kBK;      // activations only
+    static constexpr int kRowScaleSlot = kBM * 16;
+    static constexpr int kOffRowScales = kStages * kStageBytes;
+    static constexpr int kColScaleSlot = 4096;
+    static constexpr int kOffColScales = kOffRowScales + 2 * kRowScaleSlot;
+    static constexpr int kStagingWave = 32 * kStagingRowStride;
+    static constexpr int kOffStaging = kOffColScales + 2 * kColScaleSlot;
+    static constexpr int kLdsBytes = kOffStaging + kGemmWaves * kStagingWave;
+    static constexpr int kRequests = kRowTiles + 2 * kColTiles;  // per thread and item: activation copies + weight loads
+    // 64-row tiles leave room (200 registers per lane, 53 KiB of LDS) for two workgroups on a CU: launches of that height are
+    // bound by streaming their weights, and a second workgroup doubles the requests in flight
+    static constexpr int kWorkgroupsPerCu = RT == 1 ? 2 : 1;
+    static constexpr int kWeightRegs = 64 * RT;  // first of the 64 accumulation registers that hold weight fragments: right behind the accumulators
+    // In flight at an item's wait such that the NEXT item's operands have arrived: the requests of the two items after it.
+    static constexpr int kWait = 2 * kRequests;
+};
+
+// Asynchronous 16-byte copy global -> LDS whose LDS address is a per-wave base (SGPR) plus a compile-time constant.
+template <int kLdsConst>
+__device__ __forceinline__ void copy16_to_lds_at(const void* uniform_base, uint32_t lane_offset, uint32_t wave_lds_base)
+{
+    asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" ::"s"(wave_lds_base), "n"(kLdsConst),
+                 "v"(lane_offset), "s"(uniform_base)
+                 : "memory", "scc");
+}
+// The 64 registers of the weight fragments, as clobber lists: they follow the accumulators (64 * RT registers), so that a
+// kernel with few accumulators also needs few registers in all.
+#define DPEP_WEIGHT_REGS_64 \
+    "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79",    \
+        "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94",       \
+        "a95", "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108",     \
+        "a109", "a110", "a111", "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121",        \
+        "a122", "a123", "a124", "a125", "a126", "a127"
+#define DPEP_WEIGHT_REGS_128 \
+    "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141",    \
+        "a142", "a143", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154",        \
+        "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167",        \
+        "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180",        \
+        "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191"
+#define DPEP_WEIGHT_REGS_192 \
+    "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205",    \
+        "a206", "a207", "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218",        \
+        "a219", "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231",        \
+        "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244",        \
+        "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
+// Asynchronous 16-byte load into a[kReg : kReg + 3].  Nothing is an output as far as the compiler knows.  kFirst: the
+// first of the kernel's 64 weight registers (all of them are declared clobbered, whichever four are loaded).
+#define DPEP_WEIGHT_LOAD(hint, clobbers)                                                                                \
+    asm volatile("global_load_dwordx4 a[%3:%4], %0, %1 offset:%2 " hint ::"v"(lane_offset), "s"(uniform_base), "n"(kImm), \
+                 "n"(kReg), "n"(kReg + 3)                                                                               \
+                 : "memory", clobbers)
+template <int kFirst, int kReg, int kImm, bool kStreamed>
+__device__ __forceinline__ void load16_to_weight_regs(const void* uniform_base, uint32_t lane_offset)
+{
+    static_assert(kFirst == 64 || kFirst == 128 || kFirst == 192, "weight registers start at a64, a128 or a192");
+    static_assert(kReg >= kFirst && kReg + 3 < kFirst + 64, "not one of the kernel's weight registers");
+    if constexpr (kFirst == 64) {
+        if (kStreamed) DPEP_WEIGHT_LOAD("nt", DPEP_WEIGHT_REGS_64);
+        else DPEP_WEIGHT_LOAD("sc1", DPEP_WEIGHT_REGS_64);
+    } else if constexpr (kFirst == 128) {
+        if (kStreamed) DPEP_WEIGHT_LOAD("nt", DPEP_WEIGHT_REGS_128);
+        else DPEP_WEIGHT_LOAD("sc1", DPEP_WEIGHT_REGS_128);
+    } else {
+        if (kStreamed) DPEP_WEIGHT_LOAD("nt", DPEP_WEIGHT_REGS_192);
+        else DPEP_WEIGHT_LOAD("sc1", DPEP_WEIGHT_REGS_192);
+    }
+}
+// Scaled MFMA, B operand a[kReg : kReg + 3], the scale bytes chosen at compile time: byte kByteA of scale_a, byte kByteB
+// of scale_b.
+template <int kReg, int kByteA, int kByteB>
+__device__ __forceinline__ void mfma_fp8_fp4_regs(v16f& acc, const v8i& a, int scale_a, int scale_b)
+{
+    asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, a[%8:%9], %0, %2, %3 op_sel:[%4,%5,0] op_sel_hi:[%6,%7,0] blgp:4"
+                 : "+a"(acc)
+                 : "v"(a), "v"(scale_a), "v"(scale_b), "n"(kByteA & 1), "n"(kByteB & 1), "n"(kByteA >> 1), "n"(kByteB >> 1), "n"(kReg),
+                   "n"(kReg + 3));
+}
+
+// The lane's number, worked out on the spot (two instructions) instead of kept in a register: the code that runs once
+// per tile or span (tile switches, scale requests, the epilogue) takes its lane-dependent addresses from this, so that the
+// item loop does not have to carry them.
+__device__ __forceinline__ int lane_now()
+{
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+
+template <int RT, bool kGateUp>
+__global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void grouped_gemm_colwave_kernel(GemmParams p)
+{
+    constexpr bool kGather = kGateUp;
+    using Cfg = ColCfg<RT>;
+    constexpr int kBM = Cfg::kBM, kStages = Cfg::kStages, kStageBytes = Cfg::kStageBytes, kRowTiles = Cfg::kRowTiles;
+    constexpr int kCols = Cfg::kColTiles;
+    constexpr bool kStreamed = RT == 1;  // few rows per expert: every weight byte is read once or twice
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    __shared__ int tile_base[kMaxMoeExperts + 1];
+    __shared__ int row_offsets[kMaxMoeExperts + 1];
+    __shared__ int tile_index[2][kGemmThreads];  // row_to_route of a tile's rows; slots alternate per tile
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 5, lr = lane & 31;
+    const int n_tiles = p.n / kBN;
+    const int ktiles = p.k / kBK;  // a multiple of 4
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+    const uint32_t lds_index = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&tile_index[0][0]));
+    const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+
+    if (tid <= p.num_local) row_offsets[tid] = p.offsets[tid];
+    __syncthreads();
+    if (tid == 0) {
+        int total = 0;
+        for (int e = 0; e < p.num_local; ++e) {
+            tile_base[e] = total;
+            const int rows = row_offsets[e + 1] - row_offsets[e];
+            total += (rows + kBM - 1) / kBM * n_tiles;
+        }
+        tile_base[p.num_local] = total;
+    }
+    __syncthreads();
+    const int total_tiles = tile_base[p.num_local];
+
+    // Tiles to workgroups, and what the workgroups without a tile do: as in grouped_gemm_kernel.
+    const bool one_round = total_tiles < static_cast<int>(gridDim.x);
+    const int fillers = one_round && p.fill_out != nullptr ? (static_cast<int>(gridDim.x) - total_tiles) * kGemmWaves : 0;
+    const bool spread = one_round && fillers == 0 && (gridDim.x & 7) == 0;
+    const int per_xcd = spread ? (total_tiles + 7) / 8 : (gridDim.x + 7) / 8;
+    const int first = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    const int stride = one_round ? total_tiles + 1 : per_xcd * 8;
+    const bool has_tile = first < total_tiles && (!spread || static_cast<int>(blockIdx.x >> 3) < per_xcd);
+    if (blockIdx.x == 0 && tid == 0 && p.fill_state != nullptr) p.fill_state[0] = fillers;
+    if (!has_tile) {
+        if (fillers == 0) return;
+        const int filler = (first - total_tiles) * kGemmWaves + wave;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        int done = 0;
+        const int stop_at_start = __hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int token = filler; token < p.fill_tokens; token += fillers, ++done) {
+            if (__hip_atomic_load(p.fill_stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != stop_at_start) break;
+            const bool mine = lane < p.fill_topk && p.fill_route_to_row[static_cast<size_t>(token) * p.fill_topk + lane] >= 0;
+            if (__ballot(mine) != 0ull) continue;
+            u32x4* row = p.fill_out + static_cast<size_t>(token) * p.fill_vec;
+            for (int v = lane; v < p.fill_vec; v += 64) store16_nt(row + v, zero);
+        }
+        if (lane == 0) p.fill_state[1 + filler] = done;
+        return;
+    }
+    const int my_tiles = one_round ? 1 : (total_tiles - first + stride - 1) / stride;
+
+    auto decode = [&](int tile) {
+        int e = 0;
+        while (tile >= tile_base[e + 1]) ++e;
+        const int row_begin = row_offsets[e], rows = row_offsets[e + 1] - row_begin;
+        const int m_tiles = (rows + kBM - 1) / kBM;
+        const int local = tile - tile_base[e];
+        // Inside an expert the tiles are numbered panel by panel: kPanel column tiles wide (the last panel may be
+        // narrower), all row tiles high, row by row.  The 32 consecutive tiles an XCD works on at a time are then a block of
+        // about 4 row tiles x 8 column tiles, whose activation rows and weight columns that XCD's L2 fetches once, instead
+        // of every row tile of a few column tiles (which made each of the eight XCDs fetch all the rows of a large expert).
+        constexpr int kPanel = 8;
+        const int panel = local / (m_tiles * kPanel), in_panel = local - panel * (m_tiles * kPanel);
+        const int width = min(kPanel, n_tiles - panel * kPanel);
+        TileInfo info;
+        info.expert = e;
+        info.nt = panel * kPanel + in_panel % width;
+        const int m0 = (in_panel / width) * kBM;
+        info.row0 = row_begin + m0;
+        info.valid = min(kBM, rows - m0);
+        return info;
+    };
+
+    // ---- request cursor: what is asked for next (activation copies, weight loads, scales, gather indices) ----------
+    // activation copy c of wave w fills LDS rows c*32 + w*8 + lane/8; chunk (lane%8) ^ ((row>>1)&7) of the 128-byte row
+    const int a_chunk = ((lane & 7) ^ ((wave * 4 + (lane >> 4)) & 7)) * 16;
+    uint32_t a_off[kRowTiles];
+    uint32_t sa_off = 0;  // this thread's row of scale bytes, from p.a_scales
+    const uint32_t b_lane = static_cast<uint32_t>(wave * 4096 + lane * 16);  // this wave's four fragments of an item are contiguous
+    const uint8_t* b_base = p.w;
+    const uint8_t* sb_base = p.ws;  // column scales of the tile under the cursor (thread t copies bytes 16 t .. 16 t + 15 of a span)
+    int index_row0 = 0, index_valid = 1;  // rows whose gather indices are fetched next
+    int copy_tile = first, copy_kt = 0, copy_span = -1, copy_ordinal = 0;
+    const int scale_bytes = p.k / 32;  // per row
+    const int spans = ktiles / 4;
+    TileInfo next_info = decode(first);
+
+    auto point_at_tile = [&](const TileInfo& info) {
+        const int* index = tile_index[copy_ordinal & 1];
+        // (the lane's row numbers are worked out afresh at every tile switch: kept in registers across the item loop
+        // they cost the loop a register each, or a place on the stack)
+        const int lane_here = lane_now(), tid_here = wave * 64 + lane_here;
+#pragma unroll
+        for (int i = 0; i < kRowTiles; ++i) {
+            const int r = min(i * 32 + wave * 8 + (lane_here >> 3), info.valid - 1);  // rows past the tile's end repeat its last row
+            const int src = kGather ? min(max(index[r] / p.topk, 0), p.a_rows - 1) : info.row0 + r;
+            a_off[i] = static_cast<uint32_t>(src) * static_cast<uint32_t>(p.k) + a_chunk;
+        }
+        {
+            const int r = min(tid_here % kBM, info.valid - 1);
+            const int src = kGather ? min(max(index[r] / p.topk, 0), p.a_rows - 1) : info.row0 + r;
+            sa_off = static_cast<uint32_t>(src) * static_cast<uint32_t>(scale_bytes);
+        }
+        const bool shared = info.expert >= p.num_routed;
+        const size_t weight_index = shared ? info.expert - p.num_routed : info.expert;
+        b_base = (shared ? p.w_shared : p.w) + weight_index * p.n * (p.k / 2) + static_cast<size_t>(info.nt) * ktiles * 16384;
+        sb_base = (shared ? p.ws_shared : p.ws) + (weight_index * n_tiles + info.nt) * spans * Cfg::kColScaleSlot;
+    };
+    auto aim_index_prefetch = [&](const TileInfo& info) {
+        index_row0 = info.row0;
+        index_valid = info.valid;
+    };
+    auto index_offset = [&]() {  // this thread's entry of row_to_route, in bytes
+        return static_cast<uint32_t>(index_row0 + min(wave * 64 + lane_now(), index_valid - 1)) * 4u;
+    };
+
+    // Column scales of the current span and of the next one: [column tile] x 8 bytes = k tiles 0..3 x k steps 0..1.
+    u32x2 bscale_now[kCols], bscale_next[kCols];
+
+    // The requests of the item under the cursor, which goes to ring position kPos; issued in pieces between MFMAs.
+    auto request_activations = [&](auto pos, auto piece) {
+        constexpr int kPos = decltype(pos)::value, kPiece = decltype(piece)::value;
+        copy16_to_lds_at<kPos * kStageBytes + kPiece * 4096>(p.a_codes + static_cast<size_t>(copy_kt) * kBK, a_off[kPiece], wave_lds);
+    };
+    auto request_weights = [&](auto pos, auto step) {
+        constexpr int kPos = decltype(pos)::value, kStep = decltype(step)::value;
+        const uint8_t* item = b_base + static_cast<size_t>(copy_kt) * 16384;
+        // fragment (column tile c, k step) of the wave's four: 2048 c + 1024 step bytes in; registers 16 pos + 8 step + 4 c
+        constexpr int kReg = Cfg::kWeightRegs + 16 * kPos + 8 * kStep;
+        load16_to_weight_regs<Cfg::kWeightRegs, kReg, kStep * 1024, kStreamed>(item, b_lane);
+        load16_to_weight_regs<Cfg::kWeightRegs, kReg + 4, 2048 + kStep * 1024, kStreamed>(item, b_lane);
+    };
+    // A span's first item (ring position 0) also asks for the span's scales, into the LDS slots of the span's parity: 16
+    // bytes of row scales per row and the span's 4 KiB of column scales.  A tile's first item asks for the gather indices of
+    // the workgroup's next tile.
+    auto request_span = [&]() {
+        ++copy_span;
+        const int window = min(copy_kt * 4, scale_bytes - 16);
+        copy16_to_lds(p.a_scales + window, sa_off, lds0 + Cfg::kOffRowScales + (copy_span & 1) * Cfg::kRowScaleSlot + ((wave * 64) % kBM) * 16);
+        copy16_to_lds(sb_base + static_cast<size_t>(copy_kt >> 2) * Cfg::kColScaleSlot, static_cast<uint32_t>(wave * 1024 + lane_now() * 16),
+                      lds0 + Cfg::kOffColScales + (copy_span & 1) * Cfg::kColScaleSlot + wave * 1024);
+        if (kGather)
+            copy4_to_lds_unless(p.row_to_route, index_offset(), lds_index + ((copy_ordinal + 1) & 1) * (kGemmThreads * 4) + wave * 256, copy_kt);
+    };
+    // (k tiles come in fours, so a tile can only end behind ring position 3)
+    auto advance_cursor = [&](bool in_prologue, bool last_of_four) {
+        ++copy_kt;
+        if (last_of_four && copy_kt == ktiles) {
+            if (copy_tile + stride < total_tiles) {
+                // (a tile has at least four items, so only a switch inside the prologue can come before a counted wait
+                // has covered the fetch of the next tile's indices)
+                if (kGather && switch_needs_drain(in_prologue, ktiles, kStages)) wait_copies_then_barrier<0>();
+                copy_tile += stride;
+                copy_kt = 0;
+                ++copy_ordinal;
+                point_at_tile(next_info);
+                if (copy_tile + stride < total_tiles) next_info = decode(copy_tile + stride);
+                aim_index_prefetch(next_info);
+            } else {
+                copy_kt = ktiles - 4;  // past the last tile: keep asking for its last span (never used)
+            }
+        }
+    };
+
+    if (kGather) {
+        aim_index_prefetch(next_info);
+        copy4_to_lds(p.row_to_route, index_offset(), lds_index + wave * 256);
+        wait_copies_then_barrier<0>();
+    }
+    point_at_tile(next_info);
+    if (first + stride < total_tiles) next_info = decode(first + stride);
+    aim_index_prefetch(next_info);
+
+    // ---- fragment addresses inside a stage ---------------------------------------------------------
+    int a_addr[2][2];  // [k step][lo/hi 16 bytes] of row tile 0; row tile i lies i * 4096 bytes further (same swizzle)
+    {
+        const int sw = (lr >> 1) & 7;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            a_addr[kb][0] = lr * kBK + (((kb * 4 + g) ^ sw) << 4);
+            a_addr[kb][1] = lr * kBK + (((kb * 4 + 2 + g) ^ sw) << 4);
+        }
+    }
+    // LDS address of this lane's row-scale entry in the slot of the span being read; row tile i lies i * 512 bytes further,
+    // k tile q of the span 4 q bytes (one register and instruction offsets, not a register per row tile)
+    int row_scale_at = Cfg::kOffRowScales + lr * 16;
+
+    v8i afrag[2][kRowTiles];   // [k step][row tile]
+    int ascale[2][kRowTiles];  // [item parity][row tile]: the row-scale word of the k tile, moved so that this lane half's
+                               // first k block is byte 0 (its second is byte 2)
+    auto read_fragment = [&](int stage, int kb, int i) {
+        const uint8_t* at = lds + stage * kStageBytes + i * 4096;
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(at + a_addr[kb][0]);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(at + a_addr[kb][1]);
+        afrag[kb][i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    };
+    int col_scale_slot = 0;  // byte offset of the LDS slot whose span's column scales are read next
+    auto read_row_scale = [&](int parity, int pos, int i) {
+        ascale[parity][i] = static_cast<int>(*reinterpret_cast<const uint32_t*>(lds + row_scale_at + (i * 512 + pos * 4)));
+    };
+    auto read_col_scales = [&]() {
+        const int sb_addr = Cfg::kOffColScales + wave * 1024 + lane_now() * 8;  // this wave's column tile c: + c * 512
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) bscale_next[c] = *reinterpret_cast<const u32x2*>(lds + sb_addr + c * 512 + col_scale_slot);
+    };
+
+    v16f acc[kRowTiles][kCols];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < kRowTiles; ++i)
+#pragma unroll
+            for (int c = 0; c < kCols; ++c)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) acc[i][c][j] = 0.0f;
+    };
+
+    // ---- epilogue of one tile (per-wave staging region, no workgroup synchronisation) ----------------
+    uint8_t* region = lds + Cfg::kOffStaging + wave * Cfg::kStagingWave;
+    auto epilogue = [&](const TileInfo& info) {
+        constexpr int kPasses = kGateUp ? 1 : kCols;
+        const int lane = lane_now(), g = lane >> 5, lr = lane & 31;  // (the epilogue's own copies: see lane_now)
+#pragma unroll
+        for (int i = 0; i < kRowTiles; ++i) {
+            if (i == kRowTiles - 1 && fillers != 0 && wave == 0 && lane == 0)
+                __hip_atomic_fetch_add(p.fill_stop, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int tile_rows = min(32, info.valid - 32 * i);  // may be <= 0
+            const size_t out_row0 = static_cast<size_t>(info.row0) + 32 * i;
+            // (a row tile's accumulators leave their registers here, not earlier: read all at once at the head of the
+            // epilogue, the twelve tiles would need 192 more registers than the loop's own state leaves free)
+#pragma unroll
+            for (int c = 0; c < kCols; ++c) asm volatile("" : "+a"(acc[i][c]));
+#pragma unroll
+            for (int pass = 0; pass < kPasses; ++pass) {
+#pragma unroll
+                for (int j = 0; j < 16; j += 2) {
+                    float value[2];
+#pragma unroll
+                    for (int d = 0; d < 2; ++d) {
+                        if (kGateUp) {
+                            const uint32_t rounded = pack_bf16x2(acc[i][0][j + d], acc[i][1][j + d]);
+                            value[d] = silu_mul(__uint_as_float(rounded << 16), __uint_as_float(rounded & 0xffff0000u));
+                        } else {
+                            value[d] = acc[i][pass][j + d];
+                        }
+                    }
+                    const uint32_t pair = pack_bf16x2(value[0], value[1]);
+                    const int r = (j >> 2) * 8 + g * 4 + (j & 3);
+                    uint8_t* cell = region + r * kStagingRowStride + lr * 2;
+                    *reinterpret_cast<uint16_t*>(cell) = static_cast<uint16_t>(pair);
+                    *reinterpret_cast<uint16_t*>(cell + kStagingRowStride) = static_cast<uint16_t>(pair >> 16);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                if (kGateUp) {
+                    const int act_width = p.n / 2;
+                    const int act_col = (info.nt * (kBN / 64) + wave) * 32;
+                    const int r = lane >> 1, half = lane & 1;
+                    float v[16];
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const u32x4 raw = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + half * 32 + q * 16);
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            v[q * 8 + 2 * t] = bf16_to_f32(raw[t] & 0xffffu);
+                            v[q * 8 + 2 * t + 1] = bf16_to_f32(raw[t] >> 16);
+                        }
+                    }
+                    float amax = 0.0f;
+#pragma unroll
+                    for (int t = 0; t < 16; ++t) amax = fmaxf(amax, fabsf(v[t]));
+                    amax = fmaxf(amax, __shfl_xor(amax, 1));
+                    const int byte = mx_scale_byte(amax);
+                    u32x4 codes;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        codes[t] = pack4_e4m3(mx_scaled(v[4 * t], byte), mx_scaled(v[4 * t + 1], byte),
+                                              mx_scaled(v[4 * t + 2], byte), mx_scaled(v[4 * t + 3], byte));
+                    if (r < tile_rows) {
+                        *reinterpret_cast<u32x4*>(p.act_codes + (out_row0 + r) * act_width + act_col + half * 16) = codes;
+                        if (half == 0)
+                            p.act_scales[(out_row0 + r) * (act_width / 32) + (act_col >> 5)] = static_cast<uint8_t>(byte);
+                    }
+                } else {
+                    const int col = info.nt * kBN + (wave * kCols + pass) * 32 + (lane & 3) * 8;
+#pragma unroll
+                    for (int it = 0; it < 2; ++it) {
+                        const int r = it * 16 + (lane >> 2);
+                        if (r < tile_rows && col < p.out_cols) {
+                            const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
+                            *reinterpret_cast<u32x4*>(p.out + (out_row0 + r) * p.out_cols + col) = chunk;
+                        }
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    };
+
+    // ---- prologue: everything of items 0..3, then item 0's first fragments -------------------------------
+    auto request_item = [&](auto pos) {
+        if (decltype(pos)::value == 0) request_span();
+        static_for<kRowTiles>([&](auto piece) { request_activations(pos, piece); });
+        request_weights(pos, std::integral_constant<int, 0>{});
+        request_weights(pos, std::integral_constant<int, 1>{});
+        advance_cursor(true, decltype(pos)::value == 3);
+    };
+    request_item(std::integral_constant<int, 0>{});
+    request_item(std::integral_constant<int, 1>{});
+    request_item(std::integral_constant<int, 2>{});
+    request_item(std::integral_constant<int, 3>{});
+    wait_copies_then_barrier<3 * Cfg::kRequests>();  // item 0 and its span have arrived
+    int read_span = 0;
+    read_col_scales();
+#pragma unroll
+    for (int i = 0; i < kRowTiles; ++i) {
+        read_row_scale(0, 0, i);
+        read_fragment(0, 0, i);
+    }
+    clear_acc();
+    asm volatile("s_nop 3");
+    int tile = first, kt = 0;
+    TileInfo info = decode(first);
+    const long long total_items = static_cast<long long>(my_tiles) * ktiles;
+    constexpr int kMfmas = kRowTiles * kCols;  // per k step; MFMA n works on row tile n % kRowTiles, column tile n / kRowTiles
+
+    // One item at ring position kPos.  First k step: its MFMAs, with the LDS reads of the second k step's fragments dealt
+    // out between them; then the wait + barrier, after which the item's own stage may be refilled.  Second k step: its
+    // MFMAs, with the activation copies of the item four ahead, and the reads of the next item's row scales and first
+    // fragments, dealt out between them.  Behind the last MFMA of a k step its weight registers are free: the weight loads
+    // of the item four ahead follow.
+    auto item_body = [&](auto pos) {
+        constexpr int kPos = decltype(pos)::value;
+        constexpr int kParity = kPos & 1, kNextPos = (kPos + 1) & 3;
+        if (kPos == 0) {
+            // the span's column scales were read from LDS under the previous item's last MFMAs
+#pragma unroll
+            for (int c = 0; c < kCols; ++c) bscale_now[c] = bscale_next[c];
+        }
+        const int scale_b0 = static_cast<int>(bscale_now[0][kPos >> 1]), scale_b1 = static_cast<int>(bscale_now[1][kPos >> 1]);
+        int shifted[kRowTiles];
+#pragma unroll
+        for (int i = 0; i < kRowTiles; ++i) shifted[i] = ascale[kParity][i] >> (8 * g);
+        // MFMA number n of a k step works on row tile n / kCols, column tile n % kCols: a row tile's fragment is done with
+        // after two MFMAs, and the fragment that replaces it (same row tile, next k step) is asked for right then, so
+        // that little more than one k step of fragments is ever held in registers.
+        auto mfma = [&](auto step, auto number) {
+            constexpr int kStep = decltype(step)::value, kN = decltype(number)::value;
+            constexpr int kI = kN / kCols, kC = kN % kCols;
+            mfma_fp8_fp4_regs<Cfg::kWeightRegs + 16 * kPos + 8 * kStep + 4 * kC, 2 * kStep, 2 * (kPos & 1) + kStep>(
+                acc[kI][kC], afrag[kStep][kI], shifted[kI], kC == 0 ? scale_b0 : scale_b1);
+        };
+        static_for<kMfmas>([&](auto n) {
+            constexpr int kN = decltype(n)::value;
+            mfma(std::integral_constant<int, 0>{}, n);
+            if constexpr (kN % kCols == 0) read_fragment(kPos, 1, kN / kCols);
+        });
+        // The next item's operands have arrived once each thread has at most the requests of the two items after it in
+        // flight; past the barrier every wave has also read the last fragment of this item's stage, which is refilled next.
+        wait_copies_then_barrier<Cfg::kWait>();
+        if (kPos == 0) request_span();
+        request_weights(pos, std::integral_constant<int, 0>{});
+        if (kPos == 3) {
+            // the next item opens a span: its scales sit in the other LDS slots
+            ++read_span;
+            row_scale_at += (read_span & 1) ? Cfg::kRowScaleSlot : -Cfg::kRowScaleSlot;
+            asm volatile("" : "+v"(row_scale_at));  // (kept as one value: see its declaration)
+            col_scale_slot = (read_span & 1) * Cfg::kColScaleSlot;
+            read_col_scales();
+        }
+        static_for<kMfmas>([&](auto n) {
+            constexpr int kN = decltype(n)::value;
+            mfma(std::integral_constant<int, 1>{}, n);
+            // one activation copy behind every second MFMA, the next item's row scale and first fragment of the row tile
+            // just finished behind the others
+            if constexpr (kN % kCols == 0) request_activations(pos, std::integral_constant<int, kN / kCols>{});
+            if constexpr (kN % kCols == kCols - 1) {
+                read_row_scale(kParity ^ 1, kNextPos, kN / kCols);
+                read_fragment(kNextPos, 0, kN / kCols);
+            }
+        });
+        request_weights(pos, std::integral_constant<int, 1>{});
+        advance_cursor(false, kPos == 3);
+    };
+
+    for (long long item = 0; item < total_items; item += 4) {
+        item_body(std::integral_constant<int, 0>{});
+        item_body(std::integral_constant<int, 1>{});
+        item_body(std::integral_constant<int, 2>{});
+        item_body(std::integral_constant<int, 3>{});
+        kt += 4;
+        if (__builtin_expect(kt == ktiles, 0)) {
+            settle_accumulators();
+#pragma unroll
+            for (int i = 0; i < kRowTiles; ++i)
+#pragma unroll
+                for (int c = 0; c < kCols; ++c) asm volatile("" : "+a"(acc[i][c]));
+            epilogue(info);
+            clear_acc();
+            asm volatile("s_nop 3");
+            kt = 0;
+            tile += stride;
+            if (tile < total_tiles) info = decode(tile);
+        }
+    }
+    // Nothing may still be in flight into this workgroup's LDS or registers when it retires.
+    wait_copies_then_barrier<0>();
+}
+
 // Shared experts take every token: their rows follow the routed ones, expert-major, token order.
 // offsets[num_routed + 1 + s] = R + (s + 1) * B and row_to_route[R + s * B + t] = t * topk (so that the gather's
 // route / topk is t), with R read from the device.
@@ -882,22 +1450,41 @@ int gemm_grid()
     return cus / 8 * 8;  // one resident workgroup per CU (the LDS ring takes most of the 160 KiB)
 }
 
-template <int RT, bool kGateUp>
-int launch_gemm_rt(const GemmParams& p, hipStream_t stream, const char* what)
+// Raising the dynamic LDS limit is a setting per function and per device (each device holds its own copy of the code
+// object).  One flag per device; two threads that both find it clear both make the (idempotent) call.
+template <typename Kernel>
+int allow_lds(Kernel kernel, int bytes, std::atomic<bool>* configured, int max_devices)
 {
-    constexpr int kLds = GemmCfg<RT, kGateUp>::kLdsBytes;
-    // Raising the dynamic LDS limit is a setting per function and per device (each device holds its own copy of the
-    // code object).  One flag per device; two threads that both find it clear both make the (idempotent) call.
-    constexpr int kMaxDevices = 64;
-    static std::atomic<bool> configured[kMaxDevices];
     int device = 0;
     DPEP_HIP(hipGetDevice(&device));
-    const bool tracked = device >= 0 && device < kMaxDevices;
+    const bool tracked = device >= 0 && device < max_devices;
     if (!tracked || !configured[device].load(std::memory_order_acquire)) {
-        DPEP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<RT, kGateUp>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+        DPEP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
         if (tracked) configured[device].store(true, std::memory_order_release);
     }
+    return DPEP_OK;
+}
+
+template <int RT, bool kGateUp>
+int launch_gemm_rt(const GemmParams& p, double expected_tiles, hipStream_t stream, const char* what)
+{
+    constexpr int kMaxDevices = 64;
+    if (p.column_waves && p.k % 512 == 0) {
+        constexpr int kLds = ColCfg<RT>::kLdsBytes;
+        static std::atomic<bool> configured[kMaxDevices];
+        if (int rc = allow_lds(&grouped_gemm_colwave_kernel<RT, kGateUp>, kLds, configured, kMaxDevices)) return rc;
+        // Two workgroups on a CU each run at about half speed: worth it where that does not add rounds (512 tiles on
+        // 256 CUs: one round of 512 instead of two of 256, with twice the requests in flight; 700 tiles: two slow rounds
+        // would replace three fast ones).
+        const int cus = gemm_grid();
+        int per_cu = 1;
+        if (ColCfg<RT>::kWorkgroupsPerCu == 2 && 2.0 * ceil(expected_tiles / (2.0 * cus)) <= ceil(expected_tiles / cus)) per_cu = 2;
+        hipLaunchKernelGGL((grouped_gemm_colwave_kernel<RT, kGateUp>), dim3(cus * per_cu), dim3(kGemmThreads), kLds, stream, p);
+        return launch_status(what);
+    }
+    constexpr int kLds = GemmCfg<RT, kGateUp>::kLdsBytes;
+    static std::atomic<bool> configured[kMaxDevices];
+    if (int rc = allow_lds(&grouped_gemm_kernel<RT, kGateUp>, kLds, configured, kMaxDevices)) return rc;
     hipLaunchKernelGGL((grouped_gemm_kernel<RT, kGateUp>), dim3(gemm_grid()), dim3(kGemmThreads), kLds, stream, p);
     return launch_status(what);
 }
@@ -916,12 +1503,13 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
     const double mean = expected_rows_per_expert > 1 ? expected_rows_per_expert : 1;
     const double sigma = sqrt(mean);
     int best = 2;
-    double best_cost = 1e30;
+    double best_cost = 1e30, tiles_of[4] = {0.0, 0.0, 0.0, 0.0};
     for (int rt = 1; rt <= 3; ++rt) {
         const int bm = 64 * rt;
         double m_tiles = 1.0;  // E[ceil(X / bm)] = sum over j >= 0 of P(X > j * bm)
         for (int j = 1; j * bm < mean + 6.0 * sigma; ++j) m_tiles += 0.5 * erfc((j * bm - mean) / (sigma * 1.4142135623730951));
         const double tiles = p.num_local * m_tiles * n_tiles;
+        tiles_of[rt] = tiles;
         const double rounds = ceil(tiles / cus - 0.02);  // a stray tile in one launch out of fifty does not count
         // Microseconds, fitted to kernel traces on an MI355X over shares from 32 to 2048 rows per expert, 4 to 32
         // experts and two problem sizes (it reproduced the measured order of the three heights in 14 of 16 small cases,
@@ -938,9 +1526,9 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
         }
     }
     if (p.forced_rt >= 1 && p.forced_rt <= 3) best = p.forced_rt;
-    if (best == 1) return launch_gemm_rt<1, kGateUp>(p, stream, what);
-    if (best == 2) return launch_gemm_rt<2, kGateUp>(p, stream, what);
-    return launch_gemm_rt<3, kGateUp>(p, stream, what);
+    if (best == 1) return launch_gemm_rt<1, kGateUp>(p, tiles_of[1], stream, what);
+    if (best == 2) return launch_gemm_rt<2, kGateUp>(p, tiles_of[2], stream, what);
+    return launch_gemm_rt<3, kGateUp>(p, tiles_of[3], stream, what);
 }
 
 }  // namespace
@@ -1262,6 +1850,7 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     int* fill_state = reinterpret_cast<int*>(base + l.fill_state);
     int* fill_stop = reinterpret_cast<int*>(static_cast<char*>(w->sync) + kSyncFillStop);
     g1.forced_rt = w->gemm_tile_rows / 64;
+    g1.column_waves = w->gemm_column_waves;
     // (served-only: rows of y whose token no local expert serves are nobody's business, neither the fillers' nor the
     // reduce's; with shared experts every token is served)
     const bool served_only = num_shared == 0 && w->megamoe_served_only;
@@ -1293,6 +1882,7 @@ int dpep_megamoe_forward(void* ws, const void* x_codes, const uint8_t* x_scales,
     g2.out = reinterpret_cast<uint16_t*>(base + l.out2);
     g2.out_cols = hidden;
     g2.forced_rt = g1.forced_rt;
+    g2.column_waves = g1.column_waves;
     if (int rc = launch_gemm2(g2, per_expert, s)) return rc;
     return combine_routes(base + l.out2, topk_weights, route_to_row, num_tokens, num_topk,
                           static_cast<int>(expected_rows),

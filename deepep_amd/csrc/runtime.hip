@@ -74,6 +74,7 @@ int dpep_workspace_create(size_t bytes, void** ws)
     w->exchange_extra_rows = 0;
     w->layout_one_launch = 1;
     w->gemm_tile_rows = 0;
+    w->gemm_column_waves = 1;
     w->gemm_zero_fill = 1;
     w->megamoe_served_only = 0;
     w->layout_launches = 0;
@@ -145,6 +146,8 @@ int dpep_workspace_tune(void* ws, const char* key, long long value)
         w->gemm_zero_fill = value != 0;
     } else if (strcmp(key, "megamoe_served_only") == 0) {
         w->megamoe_served_only = value != 0;
+    } else if (strcmp(key, "gemm_column_waves") == 0) {
+        w->gemm_column_waves = value != 0;
     } else if (strcmp(key, "gemm_tile_rows") == 0) {
         DPEP_REQUIRE(value == 0 || value == 64 || value == 128 || value == 192,
                      "workspace_tune: gemm_tile_rows is 0 (automatic), 64, 128 or 192");
