@@ -39,6 +39,7 @@ SIGNATURES = {
     "dpep_combine_served": (_I, (_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)),
     "dpep_mx_quant": (_I, (_P, _I, _I, _P, _P, _P)),
     "dpep_megamoe_schedule_check": (_I, (_I, _I, _I, _I, _I)),
+    "dpep_megamoe_schedule_check_column_waves": (_I, (_I, _I, _I, _I, _I)),
     "dpep_megamoe_workspace_bytes": (_Z, (_I, _I, _I, _I, _I, _I)),
     "dpep_megamoe_padded_dim": (_I, (_I,)),
     "dpep_megamoe_prepared_shape": (_I, (_I, _I, _I, ctypes.POINTER(_I), ctypes.POINTER(_I), ctypes.POINTER(_I))),

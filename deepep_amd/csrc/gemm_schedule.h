@@ -24,6 +24,18 @@ struct GemmRing {
     static constexpr int kWaitPlain = (kAhead - 2) * kCopies;
 };
 
+// The column-wave kernel (weights straight to registers): per tile height the ring of four stages that is also the unroll of
+// its item loop, the asynchronous requests per thread and item (activation copies + four weight loads; a span's first item
+// adds two scale copies, a tile's first item the fetch of the next tile's gather indices), and what may still be in flight at
+// an item's wait such that the NEXT item's operands have arrived: the requests of the two items after it.
+template <int RT>
+struct ColumnRing {
+    static constexpr int kStages = 4;
+    static constexpr int kRequests = 2 * RT + 4;
+    static constexpr int kWait = 2 * kRequests;
+    static constexpr int kPrologueWait = (kStages - 1) * kRequests;  // behind the prologue's four items: item 0 has arrived
+};
+
 // When the copy cursor may trust the next tile's gather indices.  They are fetched (asynchronously, into LDS)
 // together with the first item of the current tile, and read when the cursor moves on to that next tile, right after
 // it has issued the current tile's last item.  Waits only happen in the main loop, one per consumed item, and the

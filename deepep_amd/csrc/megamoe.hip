@@ -898,26 +898,22 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
 // there is checked on the generated code by tests/test_gemm_registers.py.  Column scales travel through LDS like the row
 // scales (each wave copies and reads only the 1 KiB of its own two column tiles).
 template <int RT>
-struct ColCfg {
+struct ColCfg : ColumnRing<RT> {
+    using ColumnRing<RT>::kStages;                     // LDS stages = items the requests run ahead = unroll of the item loop
     static constexpr int kBM = 64 * RT;
     static constexpr int kRowTiles = 2 * RT;           // 32-row MFMA tiles per workgroup tile, all of them on every wave
     static constexpr int kColTiles = 2;                // 32-column MFMA tiles per wave
-    static constexpr int kStages = 4;                  // LDS stages = items the requests run ahead = unroll of the item loop
     static constexpr int kStageBytes = kBM * kBK;      // activations only
     static constexpr int kRowScaleSlot = kBM * 16;
     static constexpr int kOffRowScales = kStages * kStageBytes;
     static constexpr int kColScaleSlot = 4096;
     static constexpr int kOffColScales = kOffRowScales + 2 * kRowScaleSlot;
-    static constexpr int kStagingWave = 32 * kStagingRowStride;
-    static constexpr int kOffStaging = kOffColScales + 2 * kColScaleSlot;
-    static constexpr int kLdsBytes = kOffStaging + kGemmWaves * kStagingWave;
-    static constexpr int kRequests = kRowTiles + 2 * kColTiles;  // per thread and item: activation copies + weight loads
+    static constexpr int kLdsBytes = kOffColScales + 2 * kColScaleSlot;
+    static_assert(ColumnRing<RT>::kRequests == kRowTiles + 2 * kColTiles, "per thread and item: activation copies + weight loads");
     // 64-row tiles leave room (200 registers per lane, 53 KiB of LDS) for two workgroups on a CU: launches of that height are
     // bound by streaming their weights, and a second workgroup doubles the requests in flight
     static constexpr int kWorkgroupsPerCu = RT == 1 ? 2 : 1;
     static constexpr int kWeightRegs = 64 * RT;  // first of the 64 accumulation registers that hold weight fragments: right behind the accumulators
-    // In flight at an item's wait such that the NEXT item's operands have arrived: the requests of the two items after it.
-    static constexpr int kWait = 2 * kRequests;
 };
 
 // Asynchronous 16-byte copy global -> LDS whose LDS address is a per-wave base (SGPR) plus a compile-time constant.
@@ -942,17 +938,21 @@ __device__ __forceinline__ void copy16_to_lds_at(const void* uniform_base, uint3
         "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167",        \
         "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180",        \
         "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191"
-#define DPEP_WEIGHT_REGS_192 \
-    "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205",    \
-        "a206", "a207", "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218",        \
-        "a219", "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231",        \
-        "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244",        \
-        "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
-// Asynchronous 16-byte load into a[kReg : kReg + 3].  Nothing is an output as far as the compiler knows.  kFirst: the
-// first of the kernel's 64 weight registers (all of them are declared clobbered, whichever four are loaded).
-#define DPEP_WEIGHT_LOAD(hint, clobbers)                                                                                \
-    asm volatile("global_load_dwordx4 a[%3:%4], %0, %1 offset:%2 " hint ::"v"(lane_offset), "s"(uniform_base), "n"(kImm), \
-                 "n"(kReg), "n"(kReg + 3)                                                                               \
+#define DPEP_WEIGHT_REGS_V192 \
+    "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205",    \
+        "v206", "v207", "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218",        \
+        "v219", "v220", "v221", "v222", "v223", "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231",        \
+        "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244",        \
+        "v245", "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255"
+// Asynchronous 16-byte load into the weight registers kReg .. kReg + 3.  Nothing is an output as far as the compiler knows.
+// kFirst: the first of the kernel's 64 weight registers (all of them are declared clobbered, whichever four are loaded).
+// At 64 and 128 rows they are accumulation registers right behind the accumulators (a64.. / a128..); at 192 rows, where the
+// accumulators fill 192 of the 256 accumulation registers, they are the ordinary registers v192..v255 (the kernel's own
+// values need fewer than 150, and with every accumulation register taken the register allocator started to put
+// loop-carried values on the stack).
+#define DPEP_WEIGHT_LOAD(file, hint, clobbers)                                                                                  \
+    asm volatile("global_load_dwordx4 " file "[%3:%4], %0, %1 offset:%2 " hint ::"v"(lane_offset), "s"(uniform_base), "n"(kImm), \
+                 "n"(kReg), "n"(kReg + 3)                                                                                       \
                  : "memory", clobbers)
 template <int kFirst, int kReg, int kImm, bool kStreamed>
 __device__ __forceinline__ void load16_to_weight_regs(const void* uniform_base, uint32_t lane_offset)
@@ -960,25 +960,35 @@ __device__ __forceinline__ void load16_to_weight_regs(const void* uniform_base, 
     static_assert(kFirst == 64 || kFirst == 128 || kFirst == 192, "weight registers start at a64, a128 or a192");
     static_assert(kReg >= kFirst && kReg + 3 < kFirst + 64, "not one of the kernel's weight registers");
     if constexpr (kFirst == 64) {
-        if (kStreamed) DPEP_WEIGHT_LOAD("nt", DPEP_WEIGHT_REGS_64);
-        else DPEP_WEIGHT_LOAD("sc1", DPEP_WEIGHT_REGS_64);
+        if (kStreamed) DPEP_WEIGHT_LOAD("a", "nt", DPEP_WEIGHT_REGS_64);
+        else DPEP_WEIGHT_LOAD("a", "sc1", DPEP_WEIGHT_REGS_64);
     } else if constexpr (kFirst == 128) {
-        if (kStreamed) DPEP_WEIGHT_LOAD("nt", DPEP_WEIGHT_REGS_128);
-        else DPEP_WEIGHT_LOAD("sc1", DPEP_WEIGHT_REGS_128);
+        if (kStreamed) DPEP_WEIGHT_LOAD("a", "nt", DPEP_WEIGHT_REGS_128);
+        else DPEP_WEIGHT_LOAD("a", "sc1", DPEP_WEIGHT_REGS_128);
     } else {
-        if (kStreamed) DPEP_WEIGHT_LOAD("nt", DPEP_WEIGHT_REGS_192);
-        else DPEP_WEIGHT_LOAD("sc1", DPEP_WEIGHT_REGS_192);
+        if (kStreamed) DPEP_WEIGHT_LOAD("v", "nt", DPEP_WEIGHT_REGS_V192);
+        else DPEP_WEIGHT_LOAD("v", "sc1", DPEP_WEIGHT_REGS_V192);
     }
 }
-// Scaled MFMA, B operand a[kReg : kReg + 3], the scale bytes chosen at compile time: byte kByteA of scale_a, byte kByteB
-// of scale_b.
-template <int kReg, int kByteA, int kByteB>
-__device__ __forceinline__ void mfma_fp8_fp4_regs(v16f& acc, const v8i& a, int scale_a, int scale_b)
+// Scaled MFMA with the operands the other way round: the weights (FP4, a[kReg : kReg + 3]) are the instruction's A
+// operand and the activations (FP8) its B operand, so the result comes out transposed: lane l holds activation row
+// l % 32, and acc[j] is weight column (j/4)*8 + (l/32)*4 + j%4 of the tile: four consecutive columns per group of
+// four registers.  A lane's results are then pieces of ONE output row, which the epilogue can store from registers (the
+// other way round a lane holds sixteen rows of one column, and the tile has to be transposed through LDS).  The scale bytes
+// are chosen at compile time: byte kByteW of scale_w, byte kByteX of scale_x.
+template <int kReg, int kByteW, int kByteX>
+__device__ __forceinline__ void mfma_fp4_fp8_regs(v16f& acc, const v8i& x, int scale_w, int scale_x)
 {
-    asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, a[%8:%9], %0, %2, %3 op_sel:[%4,%5,0] op_sel_hi:[%6,%7,0] blgp:4"
-                 : "+a"(acc)
-                 : "v"(a), "v"(scale_a), "v"(scale_b), "n"(kByteA & 1), "n"(kByteB & 1), "n"(kByteA >> 1), "n"(kByteB >> 1), "n"(kReg),
-                   "n"(kReg + 3));
+    if constexpr (kReg >= 192)  // (192-row kernels keep their weights in v192..v255, the others behind their accumulators)
+        asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, v[%8:%9], %1, %0, %2, %3 op_sel:[%4,%5,0] op_sel_hi:[%6,%7,0] cbsz:4"
+                     : "+a"(acc)
+                     : "v"(x), "v"(scale_w), "v"(scale_x), "n"(kByteW & 1), "n"(kByteX & 1), "n"(kByteW >> 1), "n"(kByteX >> 1),
+                       "n"(kReg), "n"(kReg + 3));
+    else
+        asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, a[%8:%9], %1, %0, %2, %3 op_sel:[%4,%5,0] op_sel_hi:[%6,%7,0] cbsz:4"
+                     : "+a"(acc)
+                     : "v"(x), "v"(scale_w), "v"(scale_x), "n"(kByteW & 1), "n"(kByteX & 1), "n"(kByteW >> 1), "n"(kByteX >> 1),
+                       "n"(kReg), "n"(kReg + 3));
 }
 
 // The lane's number, worked out on the spot (two instructions) instead of kept in a register: the code that runs once
@@ -1003,6 +1013,11 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
     __shared__ int tile_base[kMaxMoeExperts + 1];
     __shared__ int row_offsets[kMaxMoeExperts + 1];
     __shared__ int tile_index[2][kGemmThreads];  // row_to_route of a tile's rows; slots alternate per tile
+    // Where each thread's copies of the tile under the cursor start: [0 .. kRowTiles-1] byte offsets of its activation rows
+    // from a_codes, [kRowTiles] of its row of scale bytes from a_scales.  Written at tile switches, read back right before
+    // each copy: kept in registers instead, they are values that live across the whole item loop, and the register
+    // allocator has put such values on the stack (every reload from there waits for all the copies in flight).
+    __shared__ uint32_t copy_offsets[ColCfg<RT>::kRowTiles + 1][kGemmThreads];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1078,9 +1093,8 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
 
     // ---- request cursor: what is asked for next (activation copies, weight loads, scales, gather indices) ----------
     // activation copy c of wave w fills LDS rows c*32 + w*8 + lane/8; chunk (lane%8) ^ ((row>>1)&7) of the 128-byte row
-    const int a_chunk = ((lane & 7) ^ ((wave * 4 + (lane >> 4)) & 7)) * 16;
-    uint32_t a_off[kRowTiles];
-    uint32_t sa_off = 0;  // this thread's row of scale bytes, from p.a_scales
+    auto a_chunk_of = [&](int l) { return ((l & 7) ^ ((wave * 4 + (l >> 4)) & 7)) * 16; };
+    const uint32_t* my_offsets = &copy_offsets[0][tid];  // entry i: + i * kGemmThreads
     const uint32_t b_lane = static_cast<uint32_t>(wave * 4096 + lane * 16);  // this wave's four fragments of an item are contiguous
     const uint8_t* b_base = p.w;
     const uint8_t* sb_base = p.ws;  // column scales of the tile under the cursor (thread t copies bytes 16 t .. 16 t + 15 of a span)
@@ -1099,12 +1113,12 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
         for (int i = 0; i < kRowTiles; ++i) {
             const int r = min(i * 32 + wave * 8 + (lane_here >> 3), info.valid - 1);  // rows past the tile's end repeat its last row
             const int src = kGather ? min(max(index[r] / p.topk, 0), p.a_rows - 1) : info.row0 + r;
-            a_off[i] = static_cast<uint32_t>(src) * static_cast<uint32_t>(p.k) + a_chunk;
+            copy_offsets[i][tid_here] = static_cast<uint32_t>(src) * static_cast<uint32_t>(p.k) + a_chunk_of(lane_here);
         }
         {
             const int r = min(tid_here % kBM, info.valid - 1);
             const int src = kGather ? min(max(index[r] / p.topk, 0), p.a_rows - 1) : info.row0 + r;
-            sa_off = static_cast<uint32_t>(src) * static_cast<uint32_t>(scale_bytes);
+            copy_offsets[kRowTiles][tid_here] = static_cast<uint32_t>(src) * static_cast<uint32_t>(scale_bytes);
         }
         const bool shared = info.expert >= p.num_routed;
         const size_t weight_index = shared ? info.expert - p.num_routed : info.expert;
@@ -1125,7 +1139,7 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
     // The requests of the item under the cursor, which goes to ring position kPos; issued in pieces between MFMAs.
     auto request_activations = [&](auto pos, auto piece) {
         constexpr int kPos = decltype(pos)::value, kPiece = decltype(piece)::value;
-        copy16_to_lds_at<kPos * kStageBytes + kPiece * 4096>(p.a_codes + static_cast<size_t>(copy_kt) * kBK, a_off[kPiece], wave_lds);
+        copy16_to_lds_at<kPos * kStageBytes + kPiece * 4096>(p.a_codes + static_cast<size_t>(copy_kt) * kBK, my_offsets[kPiece * kGemmThreads], wave_lds);
     };
     auto request_weights = [&](auto pos, auto step) {
         constexpr int kPos = decltype(pos)::value, kStep = decltype(step)::value;
@@ -1141,7 +1155,7 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
     auto request_span = [&]() {
         ++copy_span;
         const int window = min(copy_kt * 4, scale_bytes - 16);
-        copy16_to_lds(p.a_scales + window, sa_off, lds0 + Cfg::kOffRowScales + (copy_span & 1) * Cfg::kRowScaleSlot + ((wave * 64) % kBM) * 16);
+        copy16_to_lds(p.a_scales + window, my_offsets[kRowTiles * kGemmThreads], lds0 + Cfg::kOffRowScales + (copy_span & 1) * Cfg::kRowScaleSlot + ((wave * 64) % kBM) * 16);
         copy16_to_lds(sb_base + static_cast<size_t>(copy_kt >> 2) * Cfg::kColScaleSlot, static_cast<uint32_t>(wave * 1024 + lane_now() * 16),
                       lds0 + Cfg::kOffColScales + (copy_span & 1) * Cfg::kColScaleSlot + wave * 1024);
         if (kGather)
@@ -1219,85 +1233,80 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
                 for (int j = 0; j < 16; ++j) acc[i][c][j] = 0.0f;
     };
 
-    // ---- epilogue of one tile (per-wave staging region, no workgroup synchronisation) ----------------
-    uint8_t* region = lds + Cfg::kOffStaging + wave * Cfg::kStagingWave;
+    // ---- epilogue of one tile: straight from the accumulators (see mfma_fp4_fp8_regs) ----------------------------------
+    // A lane holds, for its row, columns q*8 + g*4 .. + 3 (q = 0..3) of a column tile, its partner lane (l ^ 32) the four
+    // columns in between.  Two register swaps between the lane halves give the lower lane columns 0..15 and the upper lane
+    // columns 16..31 of the row as consecutive bytes, which leave as 16-byte stores.
+    auto swap_halves = [](uint32_t lower_q, uint32_t upper_q, uint32_t (&out)[2]) {
+        // lanes 0..31 get (their own lower_q, the partner's lower_q), lanes 32..63 (the partner's upper_q, their own upper_q)
+        const auto swapped = __builtin_amdgcn_permlane32_swap(lower_q, upper_q, false, false);
+        out[0] = swapped[0];
+        out[1] = swapped[1];
+    };
     auto epilogue = [&](const TileInfo& info) {
-        constexpr int kPasses = kGateUp ? 1 : kCols;
         const int lane = lane_now(), g = lane >> 5, lr = lane & 31;  // (the epilogue's own copies: see lane_now)
 #pragma unroll
         for (int i = 0; i < kRowTiles; ++i) {
             if (i == kRowTiles - 1 && fillers != 0 && wave == 0 && lane == 0)
                 __hip_atomic_fetch_add(p.fill_stop, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int tile_rows = min(32, info.valid - 32 * i);  // may be <= 0
-            const size_t out_row0 = static_cast<size_t>(info.row0) + 32 * i;
+            const bool row_exists = lr < info.valid - 32 * i;
+            const size_t row = static_cast<size_t>(info.row0) + 32 * i + lr;
             // (a row tile's accumulators leave their registers here, not earlier: read all at once at the head of the
             // epilogue, the twelve tiles would need 192 more registers than the loop's own state leaves free)
 #pragma unroll
             for (int c = 0; c < kCols; ++c) asm volatile("" : "+a"(acc[i][c]));
-#pragma unroll
-            for (int pass = 0; pass < kPasses; ++pass) {
+            if (kGateUp) {
+                // column tile 0 = gate, 1 = up of the same 32 activation columns
+                float v[16];
+                float amax = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 16; j += 2) {
-                    float value[2];
-#pragma unroll
-                    for (int d = 0; d < 2; ++d) {
-                        if (kGateUp) {
-                            const uint32_t rounded = pack_bf16x2(acc[i][0][j + d], acc[i][1][j + d]);
-                            value[d] = silu_mul(__uint_as_float(rounded << 16), __uint_as_float(rounded & 0xffff0000u));
-                        } else {
-                            value[d] = acc[i][pass][j + d];
-                        }
-                    }
-                    const uint32_t pair = pack_bf16x2(value[0], value[1]);
-                    const int r = (j >> 2) * 8 + g * 4 + (j & 3);
-                    uint8_t* cell = region + r * kStagingRowStride + lr * 2;
-                    *reinterpret_cast<uint16_t*>(cell) = static_cast<uint16_t>(pair);
-                    *reinterpret_cast<uint16_t*>(cell + kStagingRowStride) = static_cast<uint16_t>(pair >> 16);
+                    const uint32_t gate = pack_bf16x2(acc[i][0][j], acc[i][0][j + 1]), up = pack_bf16x2(acc[i][1][j], acc[i][1][j + 1]);
+                    const uint32_t act = pack_bf16x2(silu_mul(__uint_as_float(gate << 16), __uint_as_float(up << 16)),
+                                                     silu_mul(__uint_as_float(gate & 0xffff0000u), __uint_as_float(up & 0xffff0000u)));
+                    v[j] = bf16_to_f32(act & 0xffffu);
+                    v[j + 1] = bf16_to_f32(act >> 16);
+                    amax = fmaxf(amax, fmaxf(fabsf(v[j]), fabsf(v[j + 1])));
                 }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                if (kGateUp) {
-                    const int act_width = p.n / 2;
-                    const int act_col = (info.nt * (kBN / 64) + wave) * 32;
-                    const int r = lane >> 1, half = lane & 1;
-                    float v[16];
+                amax = fmaxf(amax, __shfl_xor(amax, 32));  // the row's other sixteen columns
+                const int byte = mx_scale_byte(amax);
+                uint32_t code[4];
 #pragma unroll
-                    for (int q = 0; q < 2; ++q) {
-                        const u32x4 raw = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + half * 32 + q * 16);
+                for (int q = 0; q < 4; ++q)
+                    code[q] = pack4_e4m3(mx_scaled(v[4 * q], byte), mx_scaled(v[4 * q + 1], byte), mx_scaled(v[4 * q + 2], byte),
+                                         mx_scaled(v[4 * q + 3], byte));
+                uint32_t first[2], second[2];
+                swap_halves(code[0], code[2], first);
+                swap_halves(code[1], code[3], second);
+                const u32x4 codes = {first[0], first[1], second[0], second[1]};
+                const int act_width = p.n / 2;
+                const int act_col = (info.nt * (kBN / 64) + wave) * 32;
+                if (row_exists) {
+                    *reinterpret_cast<u32x4*>(p.act_codes + row * act_width + act_col + g * 16) = codes;
+                    if (g == 0) p.act_scales[row * (act_width / 32) + (act_col >> 5)] = static_cast<uint8_t>(byte);
+                }
+            } else {
 #pragma unroll
-                        for (int t = 0; t < 4; ++t) {
-                            v[q * 8 + 2 * t] = bf16_to_f32(raw[t] & 0xffffu);
-                            v[q * 8 + 2 * t + 1] = bf16_to_f32(raw[t] >> 16);
-                        }
+                for (int c = 0; c < kCols; ++c) {
+                    uint32_t pairs[4][2];  // [q][columns +0,1 | +2,3]
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        pairs[q][0] = pack_bf16x2(acc[i][c][4 * q], acc[i][c][4 * q + 1]);
+                        pairs[q][1] = pack_bf16x2(acc[i][c][4 * q + 2], acc[i][c][4 * q + 3]);
                     }
-                    float amax = 0.0f;
-#pragma unroll
-                    for (int t = 0; t < 16; ++t) amax = fmaxf(amax, fabsf(v[t]));
-                    amax = fmaxf(amax, __shfl_xor(amax, 1));
-                    const int byte = mx_scale_byte(amax);
-                    u32x4 codes;
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        codes[t] = pack4_e4m3(mx_scaled(v[4 * t], byte), mx_scaled(v[4 * t + 1], byte),
-                                              mx_scaled(v[4 * t + 2], byte), mx_scaled(v[4 * t + 3], byte));
-                    if (r < tile_rows) {
-                        *reinterpret_cast<u32x4*>(p.act_codes + (out_row0 + r) * act_width + act_col + half * 16) = codes;
-                        if (half == 0)
-                            p.act_scales[(out_row0 + r) * (act_width / 32) + (act_col >> 5)] = static_cast<uint8_t>(byte);
-                    }
-                } else {
-                    const int col = info.nt * kBN + (wave * kCols + pass) * 32 + (lane & 3) * 8;
-#pragma unroll
-                    for (int it = 0; it < 2; ++it) {
-                        const int r = it * 16 + (lane >> 2);
-                        if (r < tile_rows && col < p.out_cols) {
-                            const u32x4 chunk = *reinterpret_cast<const u32x4*>(region + r * kStagingRowStride + (lane & 3) * 16);
-                            *reinterpret_cast<u32x4*>(p.out + (out_row0 + r) * p.out_cols + col) = chunk;
-                        }
+                    uint32_t s00[2], s01[2], s10[2], s11[2];
+                    swap_halves(pairs[0][0], pairs[2][0], s00);
+                    swap_halves(pairs[0][1], pairs[2][1], s01);
+                    swap_halves(pairs[1][0], pairs[3][0], s10);
+                    swap_halves(pairs[1][1], pairs[3][1], s11);
+                    const u32x4 lower = {s00[0], s01[0], s00[1], s01[1]}, upper = {s10[0], s11[0], s10[1], s11[1]};
+                    const int col = info.nt * kBN + (wave * kCols + c) * 32 + g * 16;
+                    if (row_exists) {
+                        // cached stores: the weighted reduce that follows reads these rows back at once
+                        if (col < p.out_cols) *reinterpret_cast<u32x4*>(p.out + row * p.out_cols + col) = lower;
+                        if (col + 8 < p.out_cols) *reinterpret_cast<u32x4*>(p.out + row * p.out_cols + col + 8) = upper;
                     }
                 }
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
             }
         }
     };
@@ -1314,7 +1323,7 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
     request_item(std::integral_constant<int, 1>{});
     request_item(std::integral_constant<int, 2>{});
     request_item(std::integral_constant<int, 3>{});
-    wait_copies_then_barrier<3 * Cfg::kRequests>();  // item 0 and its span have arrived
+    wait_copies_then_barrier<Cfg::kPrologueWait>();  // item 0 and its span have arrived
     int read_span = 0;
     read_col_scales();
 #pragma unroll
@@ -1346,19 +1355,18 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
         int shifted[kRowTiles];
 #pragma unroll
         for (int i = 0; i < kRowTiles; ++i) shifted[i] = ascale[kParity][i] >> (8 * g);
-        // MFMA number n of a k step works on row tile n / kCols, column tile n % kCols: a row tile's fragment is done with
-        // after two MFMAs, and the fragment that replaces it (same row tile, next k step) is asked for right then, so
-        // that little more than one k step of fragments is ever held in registers.
+        // MFMA number n of a k step works on row tile n / kCols, column tile n % kCols.
         auto mfma = [&](auto step, auto number) {
             constexpr int kStep = decltype(step)::value, kN = decltype(number)::value;
             constexpr int kI = kN / kCols, kC = kN % kCols;
-            mfma_fp8_fp4_regs<Cfg::kWeightRegs + 16 * kPos + 8 * kStep + 4 * kC, 2 * kStep, 2 * (kPos & 1) + kStep>(
-                acc[kI][kC], afrag[kStep][kI], shifted[kI], kC == 0 ? scale_b0 : scale_b1);
+            mfma_fp4_fp8_regs<Cfg::kWeightRegs + 16 * kPos + 8 * kStep + 4 * kC, 2 * (kPos & 1) + kStep, 2 * kStep>(
+                acc[kI][kC], afrag[kStep][kI], kC == 0 ? scale_b0 : scale_b1, shifted[kI]);
         };
         static_for<kMfmas>([&](auto n) {
             constexpr int kN = decltype(n)::value;
             mfma(std::integral_constant<int, 0>{}, n);
-            if constexpr (kN % kCols == 0) read_fragment(kPos, 1, kN / kCols);
+            // (all of them under the first half of the MFMAs: the wait before the barrier then finds them long done)
+            if constexpr (kN < kRowTiles) read_fragment(kPos, 1, kN);
         });
         // The next item's operands have arrived once each thread has at most the requests of the two items after it in
         // flight; past the barrier every wave has also read the last fragment of this item's stage, which is refilled next.
@@ -1517,7 +1525,10 @@ int launch_gemm(const GemmParams& p, int expected_rows_per_expert, hipStream_t s
         // first tile that nothing overlaps (the 192-row kernel's three-stage ring starts slowly), per tile its epilogue
         // and switch, per k tile the main loop; an expert with a single row tile streams its weight tile from HBM with
         // nobody to share it with, which adds about 0.3 us per k tile whatever the height.
-        constexpr double kFirst[3] = {0.0, 0.0, 4.7}, kPerTile[3] = {4.2, 2.9, 3.2}, kPerItem[3] = {0.53, 0.87, 1.22};
+        // (These figures are the column-wave kernel's; how to refit them: force each height with the workspace setting
+        // "gemm_tile_rows" on a many-round launch, take a kernel trace, and solve time = rounds * (per tile + k tiles * per
+        // item) over two k lengths: the two GEMMs of one forward give them.)
+        constexpr double kFirst[3] = {0.0, 0.0, 4.7}, kPerTile[3] = {4.0, 3.0, 3.4}, kPerItem[3] = {0.50, 0.83, 1.15};
         const double per_item = kPerItem[rt - 1] + (m_tiles <= 1.2 ? 0.3 : 0.0);
         const double cost = kFirst[rt - 1] + (rounds < 1.0 ? 1.0 : rounds) * (kPerTile[rt - 1] + (p.k / kBK) * per_item);
         if (cost < best_cost - 1e-9) {
@@ -1614,6 +1625,80 @@ bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, bool drain_
     return ok;
 }
 
+// The same replay for the column-wave kernel: the prologue requests items 0..3 (each: its span's scales and the next tile's
+// gather indices where it opens a span / a tile, its activation copies, its weight loads), then waits; every item's body
+// waits (kWait + slack in flight), then requests the item four ahead in the same order; tiles end behind every ktiles-th
+// item with the epilogue's stores.  slack > 0 replays a kernel whose wait is laxer than the real one.
+template <int RT>
+bool replay_column_waves(int my_tiles, int ktiles, int epilogue_stores, int slack, ScheduleFault* fault)
+{
+    using Ring = ColumnRing<RT>;
+    const long long n_items = static_cast<long long>(my_tiles) * ktiles;
+    if (n_items == 0) return true;
+    static thread_local long long item_last_op[1 << 16];
+    if (n_items >= (1 << 16)) return true;  // not replayed (far beyond any real workgroup's share)
+    long long issued = 0, done = 0;
+    auto wait = [&](long long in_flight) {
+        if (issued - in_flight > done) done = issued - in_flight;
+    };
+    int copy_kt = 0, copy_tile = 0;
+    long long copy_item = 0, index_op = -1;
+    bool ok = true, past_end = false;
+    auto request_item = [&]() {
+        if ((copy_kt & 3) == 0) {
+            issued += 2;                            // row and column scales of the span
+            if (copy_kt == 0) index_op = issued++;  // gather indices of the tile after the cursor's
+        }
+        issued += Ring::kRequests;
+        if (!past_end) item_last_op[copy_item] = issued - 1;
+    };
+    auto advance = [&](bool in_prologue, int item) {
+        ++copy_kt;
+        if (!past_end) ++copy_item;
+        if (copy_kt == ktiles) {
+            if (copy_tile + 1 < my_tiles) {
+                if (switch_needs_drain(in_prologue, ktiles, Ring::kStages)) wait(0);
+                if (index_op >= done && ok) {
+                    ok = false;
+                    *fault = {item, 2};
+                }
+                ++copy_tile;
+                copy_kt = 0;
+            } else {
+                copy_kt = ktiles - 4;  // past the last tile: its last span again (never used)
+                if (!past_end) --copy_item;
+                past_end = true;
+            }
+        }
+    };
+    auto check_item = [&](long long item) {
+        if (item < n_items && item_last_op[item] >= done && ok) {
+            ok = false;
+            *fault = {static_cast<int>(item), 1};
+        }
+    };
+    ++issued;  // the first tile's own indices, fetched synchronously
+    wait(0);
+    for (int j = 0; j < Ring::kStages; ++j) {
+        request_item();
+        advance(true, -1);
+    }
+    wait(Ring::kPrologueWait);
+    check_item(0);
+    int kt = 0;
+    for (long long item = 0; item < n_items; ++item) {
+        wait(Ring::kWait + slack);
+        check_item(item + 1);  // its first fragments leave LDS during this item's second k step, its weights right after
+        request_item();
+        advance(false, static_cast<int>(item));
+        if (++kt == ktiles) {
+            issued += epilogue_stores;
+            kt = 0;
+        }
+    }
+    return ok;
+}
+
 int launch_gemm1(const GemmParams& p, int expected_rows_per_expert, hipStream_t stream)
 {
     if (int rc = check_gemm("gemm1", p.n, p.k, p.num_local)) return rc;
@@ -1665,6 +1750,22 @@ int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktil
     if (!ok)
         return fail(DPEP_EINVAL, "schedule_check: %s read before any wait covers them (item %d)",
                     fault.what == 1 ? "an item's copies are" : "the next tile's gather indices are", fault.item);
+    return DPEP_OK;
+}
+
+int dpep_megamoe_schedule_check_column_waves(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int slack)
+{
+    using namespace dpep;
+    DPEP_REQUIRE(tile_rows == 64 || tile_rows == 128 || tile_rows == 192, "schedule_check: tile_rows is 64, 128 or 192");
+    DPEP_REQUIRE(tiles_per_workgroup >= 0 && ktiles >= 4 && ktiles % 4 == 0 && epilogue_stores >= 0 && slack >= 0,
+                 "schedule_check: bad arguments (the column-wave kernel takes k tiles in fours)");
+    ScheduleFault fault = {0, 0};
+    const bool ok = tile_rows == 64    ? replay_column_waves<1>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault)
+                    : tile_rows == 128 ? replay_column_waves<2>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault)
+                                       : replay_column_waves<3>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault);
+    if (!ok)
+        return fail(DPEP_EINVAL, "schedule_check: %s read before any wait covers them (item %d)",
+                    fault.what == 1 ? "an item's operands are" : "the next tile's gather indices are", fault.item);
     return DPEP_OK;
 }
 

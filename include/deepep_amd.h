@@ -204,6 +204,10 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
  * kernel that trusted every index fetch would do): the check then has to fail for tiles shorter than the copies run ahead,
  * which is how the tests know that it can.  Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
 int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int without_drain);
+/* The same check for the kernel that runs where K is a multiple of 512 (its waves split the tile's columns and load their
+ * weights straight into registers; k tiles come in fours).  slack = operations the replayed wait allows in flight beyond
+ * the kernel's own count: with slack > 0 the check has to fail, which is how the tests know that it can. */
+int dpep_megamoe_schedule_check_column_waves(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int slack);
 
 /* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480).
  * num_shared = number of shared experts (0..8) whose rows (every token, each) are held next to the routed ones. */

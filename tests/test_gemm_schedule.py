@@ -41,3 +41,27 @@ def test_replay_catches_a_schedule_without_the_wait_at_switches(tile_rows, ahead
         assert (status != 0) == must_fail, (tile_rows, ktiles, tiles, lib.dpep_last_error().decode())
         if must_fail:
             assert b"gather indices" in lib.dpep_last_error()
+
+
+@pytest.mark.parametrize("tile_rows", [64, 128, 192])
+def test_column_wave_schedule_holds_everywhere(tile_rows):
+    """The kernel that runs where K is a multiple of 512: every item's activation copies and weight loads, and every
+    tile's gather indices, are covered by a counted wait at every k length (in fours) and number of tiles."""
+    lib = _lib.load()
+    for ktiles, tiles, epilogue in itertools.product((4, 8, 12, 16, 56, 64), (0, 1, 2, 3, 5, 24, 100), (0, 12, 96)):
+        status = lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, epilogue, 0)
+        assert status == 0, (ktiles, tiles, epilogue, lib.dpep_last_error().decode())
+    assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, 3, 6, 0, 0) == -1  # k tiles come in fours
+    assert lib.dpep_megamoe_schedule_check_column_waves(96, 3, 8, 0, 0) == -1
+
+
+@pytest.mark.parametrize("tile_rows,requests", [(64, 6), (128, 8), (192, 10)])
+def test_column_wave_replay_catches_a_wait_that_is_too_lax(tile_rows, requests):
+    """One more item's requests allowed in flight than the kernel allows: the next item's operands are then not
+    guaranteed, and the replay says so.  A few operations of slack are absorbed only where a span's or a tile's extra
+    copies sit between the items (the real count ignores those, which errs on the strict side)."""
+    lib = _lib.load()
+    for ktiles, tiles in itertools.product((4, 8, 16, 56), (1, 2, 24)):
+        assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, 12, requests) == -1, (ktiles, tiles)
+        assert b"operands" in lib.dpep_last_error()
+        assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, 12, 0) == 0
