@@ -1362,16 +1362,29 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
             mfma_fp4_fp8_regs<Cfg::kWeightRegs + 16 * kPos + 8 * kStep + 4 * kC, 2 * (kPos & 1) + kStep, 2 * kStep>(
                 acc[kI][kC], afrag[kStep][kI], kC == 0 ? scale_b0 : scale_b1, shifted[kI]);
         };
+        // First k step.  Behind MFMA kBarrierAt comes the wait + barrier: the second step's fragments were all asked for under
+        // the first kRowTiles MFMAs and have had kBarrierAt - kRowTiles more to arrive.  The activation copies of the item four
+        // ahead (into this item's own stage, free from the barrier on) are dealt out one per kCopyEvery MFMAs over what
+        // is left of the item.
+        constexpr int kBarrierAt = kRowTiles + 1;
+        constexpr int kSlotsLeft = 2 * kMfmas - kBarrierAt - 1, kCopyEvery = kSlotsLeft / kRowTiles;
+        auto copies_behind = [&](auto slot) {  // slot = MFMAs issued since the barrier, 1-based
+            constexpr int kSlot = decltype(slot)::value;
+            if constexpr (kSlot >= 1 && (kSlot - 1) % kCopyEvery == 0 && (kSlot - 1) / kCopyEvery < kRowTiles)
+                request_activations(pos, std::integral_constant<int, (kSlot - 1) / kCopyEvery>{});
+        };
         static_for<kMfmas>([&](auto n) {
             constexpr int kN = decltype(n)::value;
             mfma(std::integral_constant<int, 0>{}, n);
-            // (all of them under the first half of the MFMAs: the wait before the barrier then finds them long done)
             if constexpr (kN < kRowTiles) read_fragment(kPos, 1, kN);
+            if constexpr (kN == kBarrierAt) {
+                // The next item's operands have arrived once each thread has at most the requests of the two items after it
+                // in flight; past the barrier every wave has also read the last fragment of this item's stage.
+                wait_copies_then_barrier<Cfg::kWait>();
+                if (kPos == 0) request_span();
+            }
+            if constexpr (kN > kBarrierAt) copies_behind(std::integral_constant<int, kN - kBarrierAt>{});
         });
-        // The next item's operands have arrived once each thread has at most the requests of the two items after it in
-        // flight; past the barrier every wave has also read the last fragment of this item's stage, which is refilled next.
-        wait_copies_then_barrier<Cfg::kWait>();
-        if (kPos == 0) request_span();
         request_weights(pos, std::integral_constant<int, 0>{});
         if (kPos == 3) {
             // the next item opens a span: its scales sit in the other LDS slots
@@ -1384,9 +1397,8 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
         static_for<kMfmas>([&](auto n) {
             constexpr int kN = decltype(n)::value;
             mfma(std::integral_constant<int, 1>{}, n);
-            // one activation copy behind every second MFMA, the next item's row scale and first fragment of the row tile
-            // just finished behind the others
-            if constexpr (kN % kCols == 0) request_activations(pos, std::integral_constant<int, kN / kCols>{});
+            copies_behind(std::integral_constant<int, kMfmas - 1 - kBarrierAt + kN + 1>{});
+            // the next item's row scale and first fragment of the row tile just finished
             if constexpr (kN % kCols == kCols - 1) {
                 read_row_scale(kParity ^ 1, kNextPos, kN / kCols);
                 read_fragment(kNextPos, 0, kN / kCols);
