@@ -431,11 +431,11 @@ def read_traffic(kernel):
         table = json.load(open(TRAFFIC_FILE))
     except (OSError, ValueError):
         return None
-    found = [entry for name, entry in table.get("kernels", {}).items() if name.rsplit(" @", 1)[0] == kernel]
+    found = [entry for name, entry in table.get("kernels", {}).items() if name.rsplit(" @", 1)[0] == kernel and not name.endswith("]")]
     return max((entry["hbm_bytes"] for entry in found), default=None)
 
 
-def ingest_pmc(fetch_csv, write_csv):
+def ingest_pmc(fetch_csv, write_csv, extra=()):
     """Two rocprofv3 --pmc runs of `bench.py --calibrate-copy --no-extra-shapes` (FETCH_SIZE, then WRITE_SIZE; KiB per
     dispatch) -> profiles/hbm_traffic.json.  Both counters are scaled by what they read for the calibration copy, whose
     traffic is known: [32768,7168] BF16 rows through dispatch_copy_row_kernel = 458 752 KiB read and as much written."""
@@ -455,7 +455,7 @@ def ingest_pmc(fetch_csv, write_csv):
 
     (fetch, calls), (write, _) = averages(fetch_csv, "FETCH_SIZE"), averages(write_csv, "WRITE_SIZE")
     known_kib = 32768 * 7168 * 2 / 1024
-    copy = [name for name in fetch if name.startswith("dispatch_copy_row_kernel @") and name in write]
+    copy = [name for name in fetch if name.startswith("dispatch_copy_row_kernel") and name in write]
     if len(copy) != 1:
         raise SystemExit("the counter files must hold one shape of dispatch_copy_row_kernel: run bench.py with "
                          "--calibrate-copy --no-extra-shapes")
@@ -465,6 +465,15 @@ def ingest_pmc(fetch_csv, write_csv):
         read_bytes, written = fetch[name] * fetch_scale * 1024, write[name] * write_scale * 1024
         kernels[name] = dict(dispatches=calls[name], fetch_kib=fetch[name], write_kib=write[name], hbm_read_bytes=round(read_bytes),
                              hbm_written_bytes=round(written), hbm_bytes=round(read_bytes + written))
+    # Counter passes of a single workload (`bench.py --megamoe-only SHAPE`): scaled by the same factors, keyed
+    # "<kernel> @<grid size> [SHAPE]", so that a kernel that runs in several workloads has an entry for each.
+    for fetch_more, write_more, label in extra:
+        (fetch_x, calls_x), (write_x, _) = averages(fetch_more, "FETCH_SIZE"), averages(write_more, "WRITE_SIZE")
+        for name in sorted(set(fetch_x) & set(write_x)):
+            read_bytes, written = fetch_x[name] * fetch_scale * 1024, write_x[name] * write_scale * 1024
+            kernels[f"{name} [{label}]"] = dict(dispatches=calls_x[name], fetch_kib=fetch_x[name], write_kib=write_x[name],
+                                                hbm_read_bytes=round(read_bytes), hbm_written_bytes=round(written),
+                                                hbm_bytes=round(read_bytes + written))
     table = dict(source="rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs) of `python3 bench.py --steps 5 --warmup 2 "
                  "--kernel-iters 5 --kernel-warmup 2 --no-cpu-baseline --no-extra-shapes --calibrate-copy`; KiB per dispatch, "
                  "averaged over the dispatches of each kernel and grid size (keys: '<kernel> @<grid size>'); most launches "
@@ -489,12 +498,17 @@ def main():
                         "read + 469.76 MB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled")
     parser.add_argument("--dispatch-stores", choices=("through", "streaming", "cached"),
                         help="store policy of the dispatch kernels (default: the library's, streaming)")
+    parser.add_argument("--megamoe-only", choices=("rank_share", "served_only", "large_batch", "decode_share"),
+                        help="run nothing but that W4A8 forward shape (for counter and trace runs of one workload) and print "
+                        "its figures")
     parser.add_argument("--ingest-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"))
+    parser.add_argument("--ingest-extra", nargs=3, action="append", default=[], metavar=("FETCH_CSV", "WRITE_CSV", "LABEL"),
+                        help="with --ingest-pmc: two more counter files, of `bench.py --megamoe-only LABEL`")
     parser.add_argument("--protocol", metavar="PRESET", help="run the reference's generic benchmark workload PRESET "
                         "(smoke, decode, prefill) and print one `measured` record per operation")
     args = parser.parse_args()
     if args.ingest_pmc:
-        ingest_pmc(*args.ingest_pmc)
+        ingest_pmc(*args.ingest_pmc, extra=args.ingest_extra)
         return
     if args.gpus != 1:
         print("bench.py measures one GPU's share; --gpus must be 1 (no multi-GPU path in this build)", file=sys.stderr)
@@ -517,6 +531,15 @@ def main():
             print(json.dumps(record))
         return
 
+    if args.megamoe_only:
+        timer = Timer(torch, args.kernel_iters, args.kernel_warmup)
+        shapes = {"rank_share": (64 * 256, 384, 6, 8, 3, False), "served_only": (64 * 256, 384, 6, 8, 3, True),
+                  "large_batch": (8192, 32, 32, 8, 1, False), "decode_share": (512, 256, 32, 8, 1, False)}
+        tokens, experts, local, topk, sets, served = shapes[args.megamoe_only]
+        us, cold, rows, flops = megamoe_shape(torch, ops, timer, tokens, experts, local, topk, weight_sets=sets, served_only=served)
+        print(json.dumps({"workload": args.megamoe_only, "rows": rows, "us_forward": us, "flushed_us": cold,
+                          "tflops_forward": flops / us / 1e6, "frac_of_fp8_peak": flops / us / 1e6 / MFMA_PEAK_TFLOPS}))
+        return
     if args.dispatch_stores:
         ops.dispatch_store_policy(args.dispatch_stores)
     x, idx, w, cfg = cases.make_inputs("C3", seed=0)
