@@ -88,7 +88,7 @@ def _oracle(x_codes, x_scales, l1, l2, idx, weights, begin):
     return mm.round_bf16(mm.local_reference(xq, idx, weights, d1, d2, begin))
 
 
-def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, tile_rows=0):
+def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, tile_rows=0, column_waves=1):
     tokens, hidden = x_codes.shape
     inter = l2[0].shape[2] * 2
     dev = "cuda"
@@ -96,6 +96,7 @@ def _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, ti
     w2, s2 = ops.megamoe_prepare_weights(torch.from_numpy(l2[0]).to(dev), torch.from_numpy(l2[1]).reshape(local, hidden, -1).to(dev), False)
     ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, idx.shape[1], hidden, inter, local))
     ws.tune("gemm_tile_rows", tile_rows)
+    ws.tune("gemm_column_waves", column_waves)
     y = torch.full((tokens, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
     counts = torch.empty((local,), dtype=torch.int32, device=dev)
     ops.megamoe_forward(
@@ -185,6 +186,26 @@ def test_megamoe_forward_at_every_tile_height(ops, tokens, hidden, inter, expert
     assert np.isfinite(got).all()
     err = mm.relative_frobenius(got, want)
     assert err <= 2e-2, err
+
+
+@pytest.mark.parametrize("tile_rows", [64, 128, 192])
+@pytest.mark.parametrize(
+    "tokens,hidden,inter,experts,begin,local,topk",
+    [
+        (300, 512, 512, 8, 2, 3, 4),     # four k tiles per tile
+        (700, 1024, 512, 2, 0, 2, 1),    # several row tiles per expert
+        (512, 1536, 1024, 16, 0, 16, 4), # several column tiles, three spans in the first GEMM
+    ],
+)
+def test_both_grouped_gemm_kernels_agree_bit_for_bit(ops, tokens, hidden, inter, experts, begin, local, topk, tile_rows):
+    """The kernel whose waves split the tile's columns (weights as the MFMA's first operand, results transposed, epilogue
+    from registers) against the 2 x 2 kernel (weights through LDS, epilogue through an LDS staging area): different
+    code, the same products summed over k in the same order, so the forward's output has to be the same bits."""
+    problem = _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=100 + tile_rows)
+    x_codes, x_scales, l1, l2, idx, weights = problem
+    new, _ = _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, tile_rows=tile_rows, column_waves=1)
+    old, _ = _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, tile_rows=tile_rows, column_waves=0)
+    np.testing.assert_array_equal(new.view(np.uint32), old.view(np.uint32))
 
 
 @pytest.mark.parametrize("tokens,hidden,inter,experts,begin,local,topk,shared", [
