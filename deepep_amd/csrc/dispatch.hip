@@ -554,10 +554,11 @@ int dpep_dispatch_copy(const void* x, const float* scales, const float* topk_wei
     if (int rc = check_common("dispatch_copy", num_tokens, num_topk, num_rows, route_to_row, row_to_route)) return rc;
     DPEP_REQUIRE(row_bytes > 0 && row_bytes % 16 == 0, "dispatch_copy: row_bytes=%d must be a positive multiple of 16",
                  row_bytes);
+    // (a share without rows or a batch without tokens: the outputs are empty buffers, which may well be null pointers)
+    if (num_rows == 0 || num_tokens == 0) return DPEP_OK;
     DPEP_REQUIRE((scales == nullptr) == (out_scales == nullptr), "dispatch_copy: scales and out_scales go together");
     DPEP_REQUIRE(scales == nullptr || scale_cols > 0, "dispatch_copy: scale_cols must be positive with scales");
     DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "dispatch_copy: weights and out_weights go together");
-    if (num_rows == 0 || num_tokens == 0) return DPEP_OK;
     DPEP_REQUIRE(x != nullptr && out != nullptr && aligned16(x) && aligned16(out), "dispatch_copy: x/out must be 16-byte aligned");
     const int vec = row_bytes / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -589,8 +590,8 @@ int dpep_dispatch_quant_fp8(const void* x, const float* topk_weights, const int3
     if (int rc = check_common("dispatch_quant_fp8", num_tokens, num_topk, num_rows, route_to_row, row_to_route)) return rc;
     DPEP_REQUIRE(hidden > 0 && hidden % 128 == 0 && hidden / 128 <= kMaxScaleCols,
                  "dispatch_quant_fp8: hidden=%d must be a positive multiple of 128, at most %d", hidden, 128 * kMaxScaleCols);
+    if (num_rows == 0 || num_tokens == 0) return DPEP_OK;  // (empty outputs may be null pointers)
     DPEP_REQUIRE((topk_weights == nullptr) == (out_weights == nullptr), "dispatch_quant_fp8: weights and out_weights go together");
-    if (num_rows == 0 || num_tokens == 0) return DPEP_OK;
     DPEP_REQUIRE(x && out && out_scales && aligned16(x) && aligned16(out), "dispatch_quant_fp8: x/out must be 16-byte aligned");
     const int units = hidden / 16;
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -734,3 +734,24 @@ def test_combine_served_only_any_topk(ops, topk):
     assert torch.equal(part[served].view(torch.int16), full[served].view(torch.int16))
     assert torch.equal(part[~served], sentinel[~served])
     assert torch.equal(part_back, full_back)
+
+
+def test_share_without_rows_takes_scales_and_weights(ops, ws):
+    """A rank none of whose experts is routed to: the outputs are empty tensors (null pointers at the C boundary), with
+    scales and weights present on the input side; both dispatch entry points return empty outputs instead of rejecting the
+    call."""
+    tokens, topk, hidden = 5, 2, 256
+    idx = torch.zeros((tokens, topk), dtype=torch.int64, device="cuda")  # every route to expert 0
+    lay = ops.layout(ws, idx, 4, 2, 2)  # this rank holds experts 2 and 3
+    _, rows = ops.layout_wait(ws)
+    assert rows == 0
+    x = torch.randn(tokens, hidden, device="cuda").bfloat16()
+    weights = torch.rand(tokens, topk, device="cuda")
+    codes, scales = ops.cast_to_fp8(x)
+    out, out_scales, out_weights = ops.dispatch_copy(codes, scales, weights, lay["route_to_row"], lay["row_to_route"], 0)
+    assert out.shape == (0, hidden) and out_scales.shape == (0, hidden // 128) and out_weights.shape == (0,)
+    out, out_scales, out_weights = ops.dispatch_quant_fp8(x, weights, lay["route_to_row"], lay["row_to_route"], 0)
+    assert out.shape == (0, hidden) and out_scales.shape == (0, hidden // 128) and out_weights.shape == (0,)
+    combined, returned = ops.combine(torch.empty((0, hidden), dtype=torch.bfloat16, device="cuda"), lay["route_to_row"],
+                                     return_values=torch.empty((0,), device="cuda"))
+    assert not combined.any() and not returned.any()
