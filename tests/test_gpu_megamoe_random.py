@@ -55,3 +55,59 @@ def test_forward_at_random_shapes(ops, seed):
         assert per_token.max() <= 6e-2, (per_token.max(), case)
     other, _ = _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, tile_rows=tile_rows, column_waves=0)
     np.testing.assert_array_equal(got.view(np.uint32), other.view(np.uint32), err_msg=str(case))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_forward_with_shared_experts_and_switches_at_random_shapes(ops, seed):
+    """Shared experts (0..2) beside the routed ones, the first GEMM's idle workgroups zeroing or not, and rows of unserved
+    tokens zeroed or left alone, each drawn per seed."""
+    import torch
+
+    tokens, hidden, inter, experts, begin, local, topk, tile_rows = _draw(100 + seed)
+    rng = np.random.default_rng(seed)
+    shared = int(rng.integers(0, 3))
+    zero_fill, served_only = int(rng.integers(0, 2)), int(rng.integers(0, 2)) if shared == 0 else 0
+    case = dict(tokens=tokens, hidden=hidden, inter=inter, experts=experts, begin=begin, local=local, topk=topk, tile_rows=tile_rows,
+                shared=shared, zero_fill=zero_fill, served_only=served_only)
+    print(case, flush=True)
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=seed)
+    sp1, ss1 = mm.quantize_weight_mxfp4((rng.normal(size=(max(shared, 1), 2 * inter, hidden)) * 0.02).astype(np.float32))
+    sp2, ss2 = mm.quantize_weight_mxfp4((rng.normal(size=(max(shared, 1), hidden, inter)) * 0.02).astype(np.float32))
+    dev = "cuda"
+
+    def prepared(packed, scales, count, n, gate_up):
+        return ops.megamoe_prepare_weights(torch.from_numpy(packed).to(dev), torch.from_numpy(scales).reshape(count, n, -1).to(dev), gate_up)
+
+    w1, s1 = prepared(*l1, local, 2 * inter, True)
+    w2, s2 = prepared(*l2, local, hidden, False)
+    extra = None
+    if shared:
+        extra = prepared(sp1[:shared], ss1[:shared], shared, 2 * inter, True) + prepared(sp2[:shared], ss2[:shared], shared, hidden, False)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local, shared))
+    sentinel = 3.0
+    y = torch.full((tokens, hidden), sentinel, dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+    try:
+        ws.tune("gemm_tile_rows", tile_rows)
+        ws.tune("gemm_zero_fill", zero_fill)
+        ws.tune("megamoe_served_only", served_only)
+        ops.megamoe_forward(ws, torch.from_numpy(x_codes).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(x_scales).to(dev),
+                            torch.from_numpy(idx).to(dev), torch.from_numpy(weights).to(dev), w1, s1, w2, s2, experts, begin, local, y,
+                            counts, intermediate=inter, shared=extra)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+    finally:
+        ws.destroy()
+    xq = mm.mx_dequantize(x_codes, x_scales)
+    shared_weights = (mm.unpack_weight(sp1[:shared], ss1[:shared]), mm.unpack_weight(sp2[:shared], ss2[:shared])) if shared else ()
+    want = mm.round_bf16(mm.local_reference(xq, idx, weights, mm.unpack_weight(*l1), mm.unpack_weight(*l2), begin, *shared_weights))
+    np.testing.assert_array_equal(counts.cpu().numpy(), np.bincount(idx.ravel(), minlength=experts)[begin : begin + local], err_msg=str(case))
+    served = ((idx >= begin) & (idx < begin + local)).any(axis=1) | (shared > 0)
+    if served_only:
+        assert (got[~served] == sentinel).all(), case
+    else:
+        assert not got[~served].any(), case
+    assert np.isfinite(got).all(), case
+    if served.any():
+        err = mm.relative_frobenius(got[served], want[served])
+        assert err <= 2e-2, (err, case)
