@@ -128,11 +128,12 @@ struct Quant16 {
     float scale;  // amax / 448
 };
 
-__device__ __forceinline__ float max8(float v)
+// Largest of a value over the 8 lanes that share a 128-element block.
+__device__ __forceinline__ uint32_t max8(uint32_t v)
 {
-    v = fmaxf(v, __shfl_xor(v, 1));
-    v = fmaxf(v, __shfl_xor(v, 2));
-    v = fmaxf(v, __shfl_xor(v, 4));
+    v = max(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 1)));
+    v = max(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 2)));
+    v = max(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 4)));
     return v;
 }
 
@@ -154,18 +155,31 @@ __device__ __forceinline__ Quant16 quantize16(u32x4 lo, u32x4 hi)
         v[8 + 2 * i] = bf16_to_f32(hi[i] & 0xffffu);
         v[8 + 2 * i + 1] = bf16_to_f32(hi[i] >> 16);
     }
-    float amax = 0.0f;
+    // amax as the largest magnitude BIT PATTERN (two BF16 magnitudes per word, v_pk_max_u16): for finite values that is
+    // the largest magnitude, and a NaN, whose pattern lies above infinity's, wins over everything, as it does in the
+    // reference's amax() and clamp() (torch propagates NaN through both, deep_ep/utils/math.py:52-53): a block that
+    // holds a NaN gets a NaN scale and the NaN code 0x7F for every value, whatever the others are.
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    u16x2 both = {0, 0};
 #pragma unroll
-    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
-    amax = fmaxf(max8(amax), 1e-4f);
+    for (int i = 0; i < 4; ++i) {
+        both = __builtin_elementwise_max(both, __builtin_bit_cast(u16x2, lo[i] & 0x7fff7fffu));
+        both = __builtin_elementwise_max(both, __builtin_bit_cast(u16x2, hi[i] & 0x7fff7fffu));
+    }
+    const uint32_t mine = max(static_cast<uint32_t>(both[0]), static_cast<uint32_t>(both[1]));
+    const uint32_t amax_bits = max(max8(mine) << 16, __float_as_uint(1e-4f));
+    const float amax = __uint_as_float(amax_bits);
+    const bool poisoned = amax_bits > 0x7f800000u;
     // The reference writes 448.0 / amax, which torch evaluates as reciprocal(amax) * 448:
     // two correctly rounded fp32 operations, reproduced here.
     const float inv = __fmul_rn(__fdiv_rn(1.0f, amax), 448.0f);
     Quant16 q;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        q.codes[i] = pack4_e4m3(__fmul_rn(v[4 * i], inv), __fmul_rn(v[4 * i + 1], inv), __fmul_rn(v[4 * i + 2], inv),
-                                __fmul_rn(v[4 * i + 3], inv));
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t codes = pack4_e4m3(__fmul_rn(v[4 * i], inv), __fmul_rn(v[4 * i + 1], inv), __fmul_rn(v[4 * i + 2], inv),
+                                          __fmul_rn(v[4 * i + 3], inv));
+        q.codes[i] = poisoned ? 0x7f7f7f7fu : codes;
+    }
     q.scale = __fdiv_rn(amax, 448.0f);
     return q;
 }

@@ -755,3 +755,32 @@ def test_share_without_rows_takes_scales_and_weights(ops, ws):
     combined, returned = ops.combine(torch.empty((0, hidden), dtype=torch.bfloat16, device="cuda"), lay["route_to_row"],
                                      return_values=torch.empty((0,), device="cuda"))
     assert not combined.any() and not returned.any()
+
+
+def test_quantiser_on_infinities_and_nans(ops, ws):
+    """Blocks that hold inf or NaN through the stand-alone quantiser, the fused dispatch (both grids) and the one-launch
+    decode path: codes and scales bit for bit those of the reference expression (a NaN poisons its whole block: NaN scale,
+    code 0x7F throughout; an infinite amax gives an infinite scale)."""
+    import warnings
+
+    from tests.gpu_util import non_finite_blocks
+
+    x = non_finite_blocks()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        want_codes, want_scales = oquant.cast_to_fp8_int(bf16_bits(x))
+    codes, scales = ops.cast_to_fp8(x.cuda())
+    np.testing.assert_array_equal(fp8_bits(codes), want_codes)
+    np.testing.assert_array_equal(f32_bits(scales), want_scales.view(np.uint32))
+    tokens, topk, experts = x.shape[0], 2, 4
+    idx = torch.stack([torch.arange(tokens) % experts, (torch.arange(tokens) + 1) % experts], dim=1).cuda()
+    lay = ops.layout(ws, idx, experts)
+    _, rows = ops.layout_wait(ws)
+    want = olayout.layout(idx.cpu().numpy(), experts)
+    for known in (rows, None):  # row-major grid (R known) and token-major grid (R not known yet)
+        out, out_scales, _ = ops.dispatch_quant_fp8(x.cuda(), None, lay["route_to_row"], lay["row_to_route"], known)
+        np.testing.assert_array_equal(fp8_bits(out[:rows]), olayout.expand_rows(want_codes, want["row_to_route"], topk))
+        np.testing.assert_array_equal(f32_bits(out_scales[:rows]), olayout.expand_rows(want_scales, want["row_to_route"], topk).view(np.uint32))
+    plan, out, out_scales, _ = ops.layout_dispatch_small(ws, idx, x.cuda(), None, None, experts, quantize=True)
+    np.testing.assert_array_equal(fp8_bits(out[:rows]), olayout.expand_rows(want_codes, want["row_to_route"], topk))
+    np.testing.assert_array_equal(f32_bits(out_scales[:rows]), olayout.expand_rows(want_scales, want["row_to_route"], topk).view(np.uint32))

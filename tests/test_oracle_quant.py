@@ -81,3 +81,21 @@ def test_integer_form_matches_torch_on_every_bf16_magnitude():
     q_i, s_i = quant.cast_to_fp8_int(block)
     np.testing.assert_array_equal(q_t.view(torch.uint8).numpy(), q_i)
     np.testing.assert_array_equal(s_t.numpy().view(np.uint32), s_i.view(np.uint32))
+
+
+def test_integer_form_matches_torch_on_non_finite_blocks():
+    """Infinities and NaNs: torch's amax() and clamp() both propagate NaN, so a block that holds one gets a NaN scale and
+    the code 0x7F throughout; an infinite amax gives scale inf, zeros for the finite values and NaN for inf * 0."""
+    import warnings
+
+    from tests.gpu_util import non_finite_blocks
+
+    x = non_finite_blocks()
+    q_t, s_t = quant.cast_to_fp8_torch(x)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        q_i, s_i = quant.cast_to_fp8_int(_bits(x))
+    np.testing.assert_array_equal(q_t.view(torch.uint8).numpy(), q_i)
+    np.testing.assert_array_equal(s_t.numpy().view(np.uint32), s_i.view(np.uint32))
+    assert (q_i[3, :128] == 0x7F).all() and (q_i[10, :128] == 0x7F).all() and (q_i[13, 128:] == 0x7F).all()
+    assert np.isnan(s_i[3, 0]) and not np.isnan(s_i[3, 1]) and np.isinf(s_i[1, 0])
