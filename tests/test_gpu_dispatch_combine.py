@@ -784,3 +784,40 @@ def test_quantiser_on_infinities_and_nans(ops, ws):
     plan, out, out_scales, _ = ops.layout_dispatch_small(ws, idx, x.cuda(), None, None, experts, quantize=True)
     np.testing.assert_array_equal(fp8_bits(out[:rows]), olayout.expand_rows(want_codes, want["row_to_route"], topk))
     np.testing.assert_array_equal(f32_bits(out_scales[:rows]), olayout.expand_rows(want_scales, want["row_to_route"], topk).view(np.uint32))
+
+
+def _same_but_for_nan_encoding(got_bits, want_bits):
+    """Equal bit for bit, except that where both are NaN the sign and payload may differ (x86 and the GPU give the
+    NaN produced by inf - inf, 0 * inf or a NaN operand different signs)."""
+    got_nan, want_nan = (got_bits & 0x7FFF) > 0x7F80, (want_bits & 0x7FFF) > 0x7F80
+    np.testing.assert_array_equal(got_nan, want_nan)
+    np.testing.assert_array_equal(np.where(got_nan, 0, got_bits), np.where(want_nan, 0, want_bits))
+
+
+def test_combine_and_cast_back_on_infinities_and_nans(ops):
+    """Rows that hold +-inf, NaN, -0, the largest finite values and values that vanish in BF16, weights that are inf, 0,
+    NaN, negative or huge: sums that overflow, inf - inf and 0 * inf all come out as in the oracle's fp32 arithmetic."""
+    import warnings
+
+    rng = np.random.default_rng(0)
+    tokens, topk, experts, hidden = 64, 4, 8, 256
+    idx = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int64)
+    lay = olayout.layout(idx, experts)
+    rows = lay["num_rows"]
+    y = torch.from_numpy(rng.normal(size=(rows, hidden)).astype(np.float32)).bfloat16()
+    special = [float("inf"), float("-inf"), float("nan"), -float("nan"), 3.3895e38, -3.3895e38, 0.0, -0.0, 1e-40]
+    for i in range(0, rows, 3):
+        y[i, rng.integers(0, hidden, size=6)] = torch.tensor([special[j] for j in rng.integers(0, len(special), size=6)]).bfloat16()
+    w = rng.random(rows).astype(np.float32)
+    w[::5], w[1::7], w[2::11], w[3::13], w[4::17] = np.inf, 0, np.nan, -1, 3e38
+    route_to_row = torch.from_numpy(lay["route_to_row"]).cuda()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        for weights in (None, w):
+            out, _ = ops.combine(y.cuda(), route_to_row, None if weights is None else torch.from_numpy(weights).cuda())
+            _same_but_for_nan_encoding(bf16_bits(out), ocombine.combine(bf16_bits(y), lay["route_to_row"], weights))
+        codes = rng.integers(0, 256, size=(8, 256), dtype=np.uint8)
+        scales = rng.random((8, 2)).astype(np.float32)
+        scales[0, 0], scales[1, 1], scales[2, 0], scales[3, 1], scales[4, 0], scales[5, 0] = np.inf, np.nan, 0, -1, 3e38, 1e-42
+        got = ops.cast_back(torch.from_numpy(codes).cuda().view(torch.float8_e4m3fn), torch.from_numpy(scales).cuda())
+        _same_but_for_nan_encoding(bf16_bits(got), oquant.cast_back(codes, scales))
