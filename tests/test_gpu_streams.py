@@ -78,3 +78,42 @@ def test_calls_wait_for_their_producers_whatever_the_streams(world, seed):
     finally:
         torch.cuda.synchronize()
         buffer.destroy()
+
+
+def test_mega_moe_calls_on_alternating_streams_share_the_workspace_in_order():
+    """Two forwards of one SymmBuffer queued on different streams, the first behind a sleeping kernel: the second has to
+    wait for the first (they share the workspace), and each has to produce its own inputs' result."""
+    from deepep_amd import megamoe
+    from oracle import megamoe as mm
+    from tests.test_gpu_megamoe import _make_problem, _oracle
+
+    tokens, hidden, inter, experts, topk = 200, 1024, 512, 8, 2
+    problems = [_make_problem(tokens, hidden, inter, experts, 0, experts, topk, seed=s) for s in (21, 22)]
+    l1, l2 = problems[0][2], problems[0][3]  # one set of weights, two batches
+    buf = megamoe.SymmBuffer(None, experts, tokens, topk, hidden, inter)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    try:
+        p1, p2 = megamoe.transform_weights_for_mega_moe(
+            (torch.from_numpy(l1[0]).cuda(), torch.from_numpy(l1[1]).cuda()), (torch.from_numpy(l2[0]).cuda(), torch.from_numpy(l2[1]).cuda()))
+        staged = [(torch.from_numpy(pr[0]).cuda().view(torch.float8_e4m3fn), torch.from_numpy(pr[1]).cuda(), torch.from_numpy(pr[4]).cuda(),
+                   torch.from_numpy(pr[5]).cuda()) for pr in problems]
+        torch.cuda.synchronize()
+        for round_ in range(4):
+            outs = []
+            for which, stream in enumerate(streams if round_ % 2 == 0 else streams[::-1]):
+                codes, scales, ids, wts = staged[which]
+                with torch.cuda.stream(stream):
+                    if which == 0:
+                        torch.cuda._sleep(SLEEP_CYCLES)
+                    y, counts = megamoe.mega_moe((codes, scales), ids, wts, p1, p2, buf)
+                    outs.append((which, y, counts))
+            torch.cuda.synchronize()
+            for which, y, counts in outs:
+                x_codes, x_scales, _, _, idx, weights = problems[which]
+                assert counts.cpu().tolist() == np.bincount(idx.ravel(), minlength=experts).tolist(), (round_, which)
+                want = _oracle(x_codes, x_scales, l1, l2, idx, weights, 0)
+                err = mm.relative_frobenius(y.float().cpu().numpy(), want)
+                assert err <= 2e-2, (round_, which, err)
+    finally:
+        torch.cuda.synchronize()
+        buf.destroy()
