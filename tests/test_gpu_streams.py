@@ -117,3 +117,48 @@ def test_mega_moe_calls_on_alternating_streams_share_the_workspace_in_order():
     finally:
         torch.cuda.synchronize()
         buf.destroy()
+
+
+def test_two_threads_with_buffers_of_their_own():
+    """Two host threads, each with its own ElasticBuffer and stream, dispatching and combining at the same time: the
+    library keeps no state that one thread's calls could take from the other's (the error text is per thread, workspaces
+    are per buffer), so each thread's results are its own inputs' results."""
+    import threading
+
+    import deepep_amd
+
+    tokens, hidden, topk, experts = 300, 1024, 4, 32
+    failures = []
+
+    def work(seed):
+        try:
+            torch.cuda.set_device(0)
+            rng = np.random.default_rng(seed)
+            stream = torch.cuda.Stream()
+            buffer = deepep_amd.ElasticBuffer(None, num_max_tokens_per_rank=tokens, hidden=hidden, num_topk=topk, explicitly_destroy=True)
+            try:
+                with torch.cuda.stream(stream):
+                    for it in range(12):
+                        ids = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int64)
+                        ids[rng.random(ids.shape) < 0.1] = -1
+                        x = torch.from_numpy(rng.normal(size=(tokens, hidden)).astype(np.float32)).bfloat16()
+                        recv, _, _, handle, _ = buffer.dispatch(x.cuda(), topk_idx=torch.from_numpy(ids).cuda(), num_experts=experts)
+                        want = olayout.layout(ids, experts)
+                        np.testing.assert_array_equal(bf16_bits(recv), olayout.expand_rows(bf16_bits(x), want["row_to_route"], topk))
+                        out, _, _ = buffer.combine(recv, handle)
+                        np.testing.assert_array_equal(bf16_bits(out), ocombine.combine(bf16_bits(recv), want["route_to_row"]))
+                        with pytest.raises(ValueError, match="hidden differs"):  # this thread's error, with this thread's text
+                            buffer.dispatch(x[:, :512].contiguous().cuda(), topk_idx=torch.from_numpy(ids).cuda(), num_experts=experts)
+            finally:
+                torch.cuda.synchronize()
+                buffer.destroy()
+        except BaseException as error:  # noqa: BLE001 - reported by the main thread
+            failures.append((seed, repr(error)))
+
+    threads = [threading.Thread(target=work, args=(seed,)) for seed in (1, 2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads)
+    assert not failures, failures
