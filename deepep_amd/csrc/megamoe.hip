@@ -302,12 +302,14 @@ struct GemmParams {
     int column_waves;               // 1: the kernel whose waves split the tile's columns and load their weights straight into registers
 };
 
-// gate / (1 + exp(-gate)) * up with the hardware exponential and reciprocal (about 1 ulp each; the
-// result is rounded to BF16 right after).  The clamp keeps exp finite, like the reference's clip(+-80).
+// gate / (1 + exp(-gate)) * up with the hardware exponential and reciprocal (v_exp_f32, v_rcp_f32: about 1 ulp each; the
+// result is rounded to BF16 right after).  The clamp keeps exp finite, like the reference's clip(+-80).  (The
+// reciprocal is the instruction itself: a correctly rounded 1 / x is a ten-instruction sequence per value, a third of the
+// first GEMM's epilogue, for a last bit that the rounding to BF16 drops.)
 __device__ __forceinline__ float silu_mul(float gate, float up)
 {
     const float clipped = fminf(fmaxf(-gate, -80.0f), 80.0f);
-    return gate * __frcp_rn(1.0f + __expf(clipped)) * up;
+    return gate * __builtin_amdgcn_rcpf(1.0f + __expf(clipped)) * up;
 }
 
 // Asynchronous copy global -> LDS: lane l's bytes land at lds_base + l * size.  lds_base is wave-uniform.
