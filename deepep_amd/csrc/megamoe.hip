@@ -1139,9 +1139,12 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
     u32x2 bscale_now[kCols], bscale_next[kCols];
 
     // The requests of the item under the cursor, which goes to ring position kPos; issued in pieces between MFMAs.
-    auto request_activations = [&](auto pos, auto piece) {
+    auto request_activations_at = [&](auto pos, auto piece, uint32_t offset) {
         constexpr int kPos = decltype(pos)::value, kPiece = decltype(piece)::value;
-        copy16_to_lds_at<kPos * kStageBytes + kPiece * 4096>(p.a_codes + static_cast<size_t>(copy_kt) * kBK, my_offsets[kPiece * kGemmThreads], wave_lds);
+        copy16_to_lds_at<kPos * kStageBytes + kPiece * 4096>(p.a_codes + static_cast<size_t>(copy_kt) * kBK, offset, wave_lds);
+    };
+    auto request_activations = [&](auto pos, auto piece) {
+        request_activations_at(pos, piece, my_offsets[decltype(piece)::value * kGemmThreads]);
     };
     auto request_weights = [&](auto pos, auto step) {
         constexpr int kPos = decltype(pos)::value, kStep = decltype(step)::value;
@@ -1370,10 +1373,13 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
         // is left of the item.
         constexpr int kBarrierAt = kRowTiles + 1;
         constexpr int kSlotsLeft = 2 * kMfmas - kBarrierAt - 1, kCopyEvery = kSlotsLeft / kRowTiles;
+        // (the copies' offsets are read from LDS in one go right behind the barrier: read one by one in front of each copy,
+        // every copy waited for its own read behind whatever fragment reads were queued before it)
+        uint32_t copy_from[kRowTiles];
         auto copies_behind = [&](auto slot) {  // slot = MFMAs issued since the barrier, 1-based
             constexpr int kSlot = decltype(slot)::value;
             if constexpr (kSlot >= 1 && (kSlot - 1) % kCopyEvery == 0 && (kSlot - 1) / kCopyEvery < kRowTiles)
-                request_activations(pos, std::integral_constant<int, (kSlot - 1) / kCopyEvery>{});
+                request_activations_at(pos, std::integral_constant<int, (kSlot - 1) / kCopyEvery>{}, copy_from[(kSlot - 1) / kCopyEvery]);
         };
         static_for<kMfmas>([&](auto n) {
             constexpr int kN = decltype(n)::value;
@@ -1383,6 +1389,8 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
                 // The next item's operands have arrived once each thread has at most the requests of the two items after it
                 // in flight; past the barrier every wave has also read the last fragment of this item's stage.
                 wait_copies_then_barrier<Cfg::kWait>();
+#pragma unroll
+                for (int i = 0; i < kRowTiles; ++i) copy_from[i] = my_offsets[i * kGemmThreads];
                 if (kPos == 0) request_span();
             }
             if constexpr (kN > kBarrierAt) copies_behind(std::integral_constant<int, kN - kBarrierAt>{});
