@@ -3,6 +3,7 @@
 
 from .api import (  # noqa: F401
     LocalGroup,
+    StoreGroup,
     SymmBuffer,
     fp8_fp4_mega_moe,
     mega_moe,
@@ -10,4 +11,4 @@ from .api import (  # noqa: F401
 )
 from .validation import check_routing  # noqa: F401
 
-__all__ = ["LocalGroup", "SymmBuffer", "transform_weights_for_mega_moe", "mega_moe", "fp8_fp4_mega_moe", "check_routing"]
+__all__ = ["LocalGroup", "StoreGroup", "SymmBuffer", "transform_weights_for_mega_moe", "mega_moe", "fp8_fp4_mega_moe", "check_routing"]

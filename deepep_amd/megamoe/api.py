@@ -49,6 +49,33 @@ class LocalGroup:
         return self._rank
 
 
+class StoreGroup(LocalGroup):
+    """The name the reference's examples construct their group with (deep_ep/_store.py:16-60, ``StoreGroup.from_env()``).
+    Here it is the identity alone: rank and size come from the launcher's environment, no store is contacted, and the
+    calls that coordinate processes answer for this process (one process per GPU, no transport between them)."""
+
+    @classmethod
+    def from_env(cls, timeout=300):
+        import os
+
+        _integer("timeout", timeout, 1, 86400)
+        return cls(int(os.environ.get("RANK", "0")), int(os.environ.get("WORLD_SIZE", "1")))
+
+    def barrier(self, stage=""):
+        return None
+
+    def all_gather(self, value, stage):
+        if self._size != 1:
+            raise NotImplementedError("This build has no transport between processes: all_gather needs a single-rank group")
+        return [value]
+
+    def abort(self, error):
+        return None
+
+    def close(self):
+        return None
+
+
 def _pair(value, name):
     if not isinstance(value, tuple) or len(value) != 2:
         raise TypeError(f"{name} must be (quantized_data, E8M0_scales)")

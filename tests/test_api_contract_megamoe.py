@@ -43,7 +43,7 @@ def test_buffer_surface():
 
 def test_exports():
     ours = set(megamoe.__all__)
-    assert ours - {"LocalGroup", "check_routing"} == set(CONTRACT["exports_reference"]) - {"StoreGroup"}
+    assert ours - {"LocalGroup", "check_routing"} == set(CONTRACT["exports_reference"])
 
 
 def test_argument_limits_are_the_reference_ones():

@@ -34,3 +34,24 @@ def test_symm_buffer_argument_gates():
         SymmBuffer(object(), 4, 17, 2, 1024, 512)
     with pytest.raises(ValueError):
         LocalGroup(2, 2)
+
+
+def test_store_group_is_the_launchers_identity(monkeypatch):
+    """StoreGroup.from_env() as the reference's example calls it (README.md:247): rank and size from the launcher's
+    environment, no store behind it; the coordinating calls answer for this process."""
+    from deepep_amd.megamoe import StoreGroup
+
+    monkeypatch.delenv("RANK", raising=False)
+    monkeypatch.delenv("WORLD_SIZE", raising=False)
+    alone = StoreGroup.from_env()
+    assert (alone.rank(), alone.size()) == (0, 1) and isinstance(alone, LocalGroup)
+    assert alone.barrier("before SHMEM teardown") is None and alone.all_gather({"rows": 3}, "sizes") == [{"rows": 3}]
+    assert alone.abort("MegaMoE: RuntimeError: x") is None and alone.close() is None
+    monkeypatch.setenv("RANK", "5")
+    monkeypatch.setenv("WORLD_SIZE", "8")
+    share = StoreGroup.from_env(timeout=30)
+    assert (share.rank(), share.size()) == (5, 8)
+    with pytest.raises(NotImplementedError, match="transport"):
+        share.all_gather(1, "x")
+    with pytest.raises(ValueError):
+        StoreGroup.from_env(timeout=0)
