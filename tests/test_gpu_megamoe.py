@@ -667,3 +667,57 @@ def test_forward_served_only_leaves_unserved_rows_untouched(ops):
         assert (part[~served] == 5.0).all() and not full[~served].any()
     finally:
         ws.destroy()
+
+
+def test_readme_example_runs_as_written(monkeypatch):
+    """The reference README's MegaMoE example (README.md:237-281) with its own imports and call sequence, one shared expert
+    included; only the device name and the sizes differ."""
+    import deepep_amd
+
+    deepep_amd.install_as_deep_ep()
+    from deep_ep_experimental.megamoe import StoreGroup, SymmBuffer, fp8_fp4_mega_moe, transform_weights_for_mega_moe
+
+    monkeypatch.setenv("RANK", "0")
+    monkeypatch.setenv("WORLD_SIZE", "1")
+    monkeypatch.setenv("LOCAL_WORLD_SIZE", "1")
+    tokens, hidden, inter, experts, topk = 40, 1024, 512, 8, 2
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, experts, topk, seed=31)
+    rng = np.random.default_rng(32)
+    sp1, ss1 = mm.quantize_weight_mxfp4((rng.normal(size=(1, 2 * inter, hidden)) * 0.02).astype(np.float32))
+    sp2, ss2 = mm.quantize_weight_mxfp4((rng.normal(size=(1, hidden, inter)) * 0.02).astype(np.float32))
+    as_pair = lambda w, sc: (torch.from_numpy(w).cuda(), torch.from_numpy(sc).cuda())  # noqa: E731
+    l1_weights, l2_weights, shared_l1_weights, shared_l2_weights = as_pair(*l1), as_pair(*l2), as_pair(sp1, ss1), as_pair(sp2, ss2)
+    x_fp8 = torch.from_numpy(x_codes).cuda().view(torch.float8_e4m3fn)
+    x_sf = torch.from_numpy(x_scales).cuda().view(torch.float8_e8m0fnu)
+    topk_idx, topk_weights = torch.from_numpy(idx).cuda(), torch.from_numpy(weights).cuda()
+
+    group = StoreGroup.from_env()
+    try:
+        buffer = SymmBuffer(
+            group, num_experts=experts, num_max_tokens_per_rank=64,
+            num_topk=topk, hidden=hidden, intermediate_hidden=inter,
+            num_shared_experts=1, mma_type="fp8xfp4",
+            ranks_per_node=int(__import__("os").environ["LOCAL_WORLD_SIZE"]),
+        )
+        w1, w2 = transform_weights_for_mega_moe(l1_weights, l2_weights)
+        shared_w1, shared_w2 = transform_weights_for_mega_moe(shared_l1_weights, shared_l2_weights, shared=True)
+        num_tokens = x_fp8.shape[0]
+        buffer.x[:num_tokens].copy_(x_fp8)
+        buffer.x_sf[:num_tokens].copy_(x_sf)
+        buffer.topk_idx[:num_tokens].copy_(topk_idx)
+        buffer.topk_weights[:num_tokens].copy_(topk_weights)
+        buffer.validate_inputs(num_tokens)
+        buffer.prepare(num_tokens)
+        y = torch.empty((num_tokens, hidden), dtype=torch.bfloat16, device="cuda")
+        assert fp8_fp4_mega_moe(y, w1, w2, buffer, shared_l1_weights=shared_w1, shared_l2_weights=shared_w2) is None
+        torch.cuda.synchronize()
+        group.barrier("before SHMEM teardown")
+        buffer.destroy()
+        group.close()
+    except BaseException as error:
+        group.abort(f"MegaMoE: {type(error).__name__}: {error}")
+        raise
+    xq = mm.mx_dequantize(x_codes, x_scales)
+    want = mm.round_bf16(mm.local_reference(xq, idx, weights, mm.unpack_weight(*l1), mm.unpack_weight(*l2), 0,
+                                            mm.unpack_weight(sp1, ss1), mm.unpack_weight(sp2, ss2)))
+    assert mm.relative_frobenius(y.float().cpu().numpy(), want) <= 2e-2
