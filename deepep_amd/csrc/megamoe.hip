@@ -251,16 +251,20 @@ struct GemmCfg : GemmRing<RT> {
     static constexpr int kOffA = 0;                    // kBM rows x 128 B, 16-byte chunks XOR-swizzled
     static constexpr int kOffB = kBM * kBK;            // 8 column tiles x 2 k steps x 1 KiB fragments
     static constexpr int kStageBytes = kOffB + 16384;
-    // Scales travel apart, once per span of four items, into two-slot rings: 16 bytes per row cover
+    // Scales travel apart, once per span of four items, into three-slot rings: 16 bytes per row cover
     // k = 512 of row scales, and one 4 KiB block holds the column scales of the span.  (4-byte copies
     // are several times slower per instruction than 16-byte ones, and a 4-byte copy per row costs a
-    // cache-line lookup per lane.)
+    // cache-line lookup per lane.)  Three slots, not two: a tile whose k is not a multiple of 512 ends with a span of
+    // two items, and in a workgroup that goes on to another tile the copies, up to five items ahead, then reach the
+    // span after next (two items + one: three items on) while the scales of the span before the short one are still
+    // being read; with three slots the span that reuses a slot starts at least seven items behind the last read.
+    static constexpr int kScaleSlots = 3;
     static constexpr int kRowScaleSlot = kBM * 16;
     static constexpr int kColScaleSlot = 4096;
     static constexpr int kOffRowScales = kStages * kStageBytes;
-    static constexpr int kOffColScales = kOffRowScales + 2 * kRowScaleSlot;
+    static constexpr int kOffColScales = kOffRowScales + kScaleSlots * kRowScaleSlot;
     static constexpr int kStagingWave = 32 * kStagingRowStride;  // the epilogue handles one 32-row tile at a time
-    static constexpr int kOffStaging = kOffColScales + 2 * kColScaleSlot;
+    static constexpr int kOffStaging = kOffColScales + kScaleSlots * kColScaleSlot;
     static constexpr int kLdsBytes = kOffStaging + 4 * kStagingWave;
 };
 
@@ -568,9 +572,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     // fetches the gather indices of the workgroup's next tile.  These extra copies only make the counted
     // waits stricter.
     auto issue_span_copies = [&]() {
-        copy_span += (copy_kt & 3) == 0 ? 1 : 0;
+        if ((copy_kt & 3) == 0) copy_span = copy_span + 1 == Cfg::kScaleSlots ? 0 : copy_span + 1;
         const int window = min((copy_kt & ~3) * 4, scale_bytes - 16);
-        const int slot = copy_span & 1;
+        const int slot = copy_span;
         copy16_to_lds_unless(sa_src + window, lds0 + Cfg::kOffRowScales + slot * Cfg::kRowScaleSlot + ((wave * 64) % kBM) * 16,
                              copy_kt & 3);
         copy16_to_lds_unless(sb_src + static_cast<size_t>(copy_kt >> 2) * Cfg::kColScaleSlot,
@@ -778,9 +782,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_kernel(GemmParam
     int read_span = -1, read_kt = 0;
     int row_at = 0, col_at = 0;
     auto next_scale_offsets = [&]() {
-        if ((read_kt & 3) == 0) ++read_span;
+        if ((read_kt & 3) == 0) read_span = read_span + 1 == Cfg::kScaleSlots ? 0 : read_span + 1;
         const int window = min((read_kt & ~3) * 4, scale_bytes - 16);
-        const int ring = read_span & 1;
+        const int ring = read_span;
         row_at = ring * Cfg::kRowScaleSlot + (read_kt * 4 - window);
         col_at = ring * Cfg::kColScaleSlot + (read_kt & 3) * 2;
         read_kt = read_kt + 1 == ktiles ? 0 : read_kt + 1;
@@ -1577,11 +1581,29 @@ struct ScheduleFault {
     int item, what;  // what: 1 = an item's copies, 2 = gather indices
 };
 
+// The rings of scale slots: a span's scales (the scales of item x are read during the body of item x - 1) must all have
+// been read when the copies of a later span go into the same slot; the copies are issued behind the barrier of the body
+// that is running (-1: the prologue, before anything is read).
+struct ScaleSlots {
+    long long last_item[4] = {-1, -1, -1, -1};  // of the span each slot holds
+    int slots, next = 0;
+    explicit ScaleSlots(int n) : slots(n) {}
+    bool take(long long span_last_item, long long body)  // false: the slot's present span is still being read
+    {
+        const long long held = last_item[next];
+        last_item[next] = span_last_item;
+        next = next + 1 == slots ? 0 : next + 1;
+        return held < 0 || held <= body;
+    }
+};
+
 template <int RT>
-bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, bool drain_at_switches, ScheduleFault* fault)
+bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, bool drain_at_switches, int scale_slots, ScheduleFault* fault)
 {
     using Ring = GemmRing<RT>;
     constexpr int kAhead = Ring::kAhead, kCopies = Ring::kCopies;
+    ScaleSlots scales(scale_slots);
+    long long body = -1;
     const long long n_items = static_cast<long long>(my_tiles) * ktiles;
     if (n_items == 0) return true;
     long long issued = 0, done = 0;  // operations [0, done) have certainly completed
@@ -1596,7 +1618,13 @@ bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, bool drain_
     bool ok = true, past_end = false;
     auto issue_copies = [&]() {
         issued += kCopies;
-        if ((copy_kt & 3) == 0) issued += 2;      // row and column scales of the span
+        if ((copy_kt & 3) == 0) {
+            issued += 2;  // row and column scales of the span
+            if (!scales.take(copy_item + (ktiles - 1 - copy_kt < 3 ? ktiles - 1 - copy_kt : 3), body) && ok) {
+                ok = false;
+                *fault = {static_cast<int>(body), 3};
+            }
+        }
         if (copy_kt == 0) index_op = issued++;    // (re-copies past the end sit on the last k tile, never 0)
         if (!past_end) item_last_op[copy_item] = issued - 1;
     };
@@ -1637,6 +1665,7 @@ bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, bool drain_
     for (long long item = 0; item < n_items; ++item) {
         wait(Ring::kWaitPlain);
         check_item(item + 1);  // its first fragments leave LDS during this item's second k step
+        body = item;
         issue_copies();
         advance(false, static_cast<int>(item));
         if (++kt == ktiles) {
@@ -1666,9 +1695,15 @@ bool replay_column_waves(int my_tiles, int ktiles, int epilogue_stores, int slac
     int copy_kt = 0, copy_tile = 0;
     long long copy_item = 0, index_op = -1;
     bool ok = true, past_end = false;
+    ScaleSlots scales(2);
+    long long body = -1;
     auto request_item = [&]() {
         if ((copy_kt & 3) == 0) {
             issued += 2;                            // row and column scales of the span
+            if (!past_end && !scales.take(copy_item + 3, body) && ok) {
+                ok = false;
+                *fault = {static_cast<int>(body), 3};
+            }
             if (copy_kt == 0) index_op = issued++;  // gather indices of the tile after the cursor's
         }
         issued += Ring::kRequests;
@@ -1711,6 +1746,7 @@ bool replay_column_waves(int my_tiles, int ktiles, int epilogue_stores, int slac
     for (long long item = 0; item < n_items; ++item) {
         wait(Ring::kWait + slack);
         check_item(item + 1);  // its first fragments leave LDS during this item's second k step, its weights right after
+        body = item;
         request_item();
         advance(false, static_cast<int>(item));
         if (++kt == ktiles) {
@@ -1765,10 +1801,14 @@ int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktil
     DPEP_REQUIRE(tiles_per_workgroup >= 0 && ktiles >= 2 && ktiles % 2 == 0 && epilogue_stores >= 0,
                  "schedule_check: bad arguments");
     ScheduleFault fault = {0, 0};
-    const bool drain = without_drain == 0;
-    const bool ok = tile_rows == 64    ? replay_workgroup<1>(tiles_per_workgroup, ktiles, epilogue_stores, drain, &fault)
-                    : tile_rows == 128 ? replay_workgroup<2>(tiles_per_workgroup, ktiles, epilogue_stores, drain, &fault)
-                                       : replay_workgroup<3>(tiles_per_workgroup, ktiles, epilogue_stores, drain, &fault);
+    const bool drain = (without_drain & 1) == 0;
+    const int slots = (without_drain & 2) != 0 ? 2 : GemmCfg<1, false>::kScaleSlots;  // (bit 1: the rings as they were, two slots)
+    const bool ok = tile_rows == 64    ? replay_workgroup<1>(tiles_per_workgroup, ktiles, epilogue_stores, drain, slots, &fault)
+                    : tile_rows == 128 ? replay_workgroup<2>(tiles_per_workgroup, ktiles, epilogue_stores, drain, slots, &fault)
+                                       : replay_workgroup<3>(tiles_per_workgroup, ktiles, epilogue_stores, drain, slots, &fault);
+    if (!ok && fault.what == 3)
+        return fail(DPEP_EINVAL, "schedule_check: a span's scales are overwritten while they are still being read (behind item %d)",
+                    fault.item);
     if (!ok)
         return fail(DPEP_EINVAL, "schedule_check: %s read before any wait covers them (item %d)",
                     fault.what == 1 ? "an item's copies are" : "the next tile's gather indices are", fault.item);
@@ -1785,6 +1825,9 @@ int dpep_megamoe_schedule_check_column_waves(int tile_rows, int tiles_per_workgr
     const bool ok = tile_rows == 64    ? replay_column_waves<1>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault)
                     : tile_rows == 128 ? replay_column_waves<2>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault)
                                        : replay_column_waves<3>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault);
+    if (!ok && fault.what == 3)
+        return fail(DPEP_EINVAL, "schedule_check: a span's scales are overwritten while they are still being read (behind item %d)",
+                    fault.item);
     if (!ok)
         return fail(DPEP_EINVAL, "schedule_check: %s read before any wait covers them (item %d)",
                     fault.what == 1 ? "an item's operands are" : "the next tile's gather indices are", fault.item);

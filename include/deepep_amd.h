@@ -199,10 +199,13 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
  * shows, without a GPU, that for a workgroup that walks `tiles_per_workgroup` tiles of `tile_rows` (64, 128 or 192)
  * rows and `ktiles` k tiles of 128 every asynchronous copy is covered by a counted wait before it is read, under
  * in-order completion of vector-memory operations: an item's operands before its MFMAs, the next tile's gather
- * indices before the copy cursor switches tiles).  epilogue_stores = stores a tile end issues (they only make the
- * counted waits stricter).  without_drain != 0 replays the schedule WITHOUT the cursor's wait at tile switches (what a
- * kernel that trusted every index fetch would do): the check then has to fail for tiles shorter than the copies run ahead,
- * which is how the tests know that it can.  Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
+ * indices before the copy cursor switches tiles), and that a ring slot of scale bytes is refilled only when the span of k
+ * tiles it held has been read to the end.  epilogue_stores = stores a tile end issues (they only make the
+ * counted waits stricter).  without_drain: bit 0 replays the schedule WITHOUT the cursor's wait at tile switches (what a
+ * kernel that trusted every index fetch would do): the check then has to fail for tiles shorter than the copies run ahead;
+ * bit 1 replays rings of two scale slots instead of the kernel's three: the check then has to fail where k is no multiple
+ * of 512 and a workgroup has several tiles; that they do fail is how the tests know that the check can.
+ * Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
 int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int without_drain);
 /* The same check for the kernel that runs where K is a multiple of 512 (its waves split the tile's columns and load their
  * weights straight into registers; k tiles come in fours).  slack = operations the replayed wait allows in flight beyond

@@ -65,3 +65,20 @@ def test_column_wave_replay_catches_a_wait_that_is_too_lax(tile_rows, requests):
         assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, 12, requests) == -1, (ktiles, tiles)
         assert b"operands" in lib.dpep_last_error()
         assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, 12, 0) == 0
+
+
+@pytest.mark.parametrize("tile_rows,ahead", [(64, 5), (128, 4), (192, 3)])
+def test_replay_catches_scale_slots_reused_too_early(tile_rows, ahead):
+    """The scales of a span of k tiles sit in a ring of LDS slots; the replay also checks that a slot is refilled only
+    when the span it held has been read to the end.  With the two slots the 2 x 2 kernel used to have, a tile whose k is no
+    multiple of 512 (a last span of two k tiles) breaks that in a workgroup with more than one tile wherever the copies run
+    more than three items ahead (64- and 128-row tiles); with three slots, and with whole spans, it holds everywhere."""
+    lib = _lib.load()
+    two_slots = 2
+    for ktiles, tiles in itertools.product((4, 6, 8, 10, 14, 16, 18), (1, 2, 3, 24)):
+        assert lib.dpep_megamoe_schedule_check(tile_rows, tiles, ktiles, 48, 0) == 0, (ktiles, tiles, lib.dpep_last_error().decode())
+        status = lib.dpep_megamoe_schedule_check(tile_rows, tiles, ktiles, 48, two_slots)
+        must_fail = tiles > 1 and ktiles % 4 == 2 and ahead > 3
+        assert (status != 0) == must_fail, (tile_rows, ktiles, tiles, lib.dpep_last_error().decode())
+        if must_fail:
+            assert b"overwritten" in lib.dpep_last_error()

@@ -208,6 +208,31 @@ def test_both_grouped_gemm_kernels_agree_bit_for_bit(ops, tokens, hidden, inter,
     np.testing.assert_array_equal(new.view(np.uint32), old.view(np.uint32))
 
 
+@pytest.mark.parametrize("tokens,hidden,inter,tile_rows", [
+    (1000, 2304, 1280, 64),   # 320 + 288 tiles of 18 and 10 k tiles on 256 workgroups
+    (1700, 1280, 768, 64),    # 10 and 6 k tiles: the shortest tile that still switches without letting the copies land
+    (2000, 2304, 1280, 128),
+    (3000, 2304, 1280, 192),
+])
+def test_several_tiles_per_workgroup_where_k_is_no_multiple_of_512(ops, tokens, hidden, inter, tile_rows):
+    """K % 512 == 256 takes the 2 x 2 kernel, whose tiles then end with a span of two k tiles instead of four.  A
+    workgroup that goes on to another tile copies up to five items ahead, i.e. into the span after the short one, while
+    the scales of the span before it are still being read: with two scale slots that copy overwrote them (64-row tiles,
+    more tiles than workgroups: wrong rows, differently on every run); the rings have three slots now."""
+    experts = 2
+    row_tiles = 2 * -(-tokens // tile_rows)  # every token goes to both experts
+    assert row_tiles * (2 * inter // 256) > 256 and row_tiles * (hidden // 256) > 256  # more tiles than workgroups, both GEMMs
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, experts, 2, seed=tile_rows)
+    want = _oracle(x_codes, x_scales, l1, l2, idx, weights, 0)
+    for attempt in range(2):
+        got, counts = _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, 0, experts, tile_rows=tile_rows)
+        assert counts.tolist() == [tokens, tokens]
+        err = mm.relative_frobenius(got, want)
+        assert err <= 2e-2, (attempt, err)
+        norms = np.linalg.norm(want, axis=1)
+        assert (np.linalg.norm(got - want, axis=1) / norms).max() <= 6e-2
+
+
 @pytest.mark.parametrize("tokens,hidden,inter,experts,begin,local,topk,shared", [
     (100, 512, 512, 8, 0, 8, 2, 1),     # one shared expert beside 8 routed ones
     (257, 768, 512, 6, 2, 2, 3, 2),     # two shared experts, partial local range, more than one row tile each
