@@ -111,3 +111,60 @@ def test_forward_with_shared_experts_and_switches_at_random_shapes(ops, seed):
     if served.any():
         err = mm.relative_frobenius(got[served], want[served])
         assert err <= 2e-2, (err, case)
+
+
+def _draw_many_tiles(seed):
+    rng = np.random.default_rng(3000 + seed)
+    experts = int(rng.choice([1, 2, 3, 4]))
+    topk = int(rng.integers(1, experts + 1))
+    tokens = int(rng.choice([700, 1000, 2000, 3000]))
+    hidden = int(rng.choice([512, 768, 1024, 1280, 2304]))
+    inter = int(rng.choice([256, 384, 512, 640, 1280]))
+    tile_rows = int(rng.choice([0, 64, 64, 128, 192]))
+    shared = int(rng.choice([0, 0, 1]))
+    return tokens, hidden, inter, experts, topk, tile_rows, shared
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_forward_with_more_tiles_than_workgroups(ops, seed):
+    """Few experts with thousands of rows each: workgroups walk several tiles of a flat stream, through both grouped GEMM
+    kernels (K a multiple of 512 or not), every tile height, with and without a shared expert."""
+    import torch
+
+    tokens, hidden, inter, experts, topk, tile_rows, shared = _draw_many_tiles(seed)
+    case = dict(tokens=tokens, hidden=hidden, inter=inter, experts=experts, topk=topk, tile_rows=tile_rows, shared=shared)
+    print(case, flush=True)
+    rng = np.random.default_rng(seed)
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, 0, experts, topk, seed=seed)
+    sp1, ss1 = mm.quantize_weight_mxfp4((rng.normal(size=(1, 2 * inter, hidden)) * 0.02).astype(np.float32))
+    sp2, ss2 = mm.quantize_weight_mxfp4((rng.normal(size=(1, hidden, inter)) * 0.02).astype(np.float32))
+    dev = "cuda"
+
+    def prepared(packed, scales, count, n, gate_up):
+        return ops.megamoe_prepare_weights(torch.from_numpy(packed).to(dev), torch.from_numpy(scales).reshape(count, n, -1).to(dev), gate_up)
+
+    w1, s1 = prepared(*l1, experts, 2 * inter, True)
+    w2, s2 = prepared(*l2, experts, hidden, False)
+    extra = prepared(sp1, ss1, 1, 2 * inter, True) + prepared(sp2, ss2, 1, hidden, False) if shared else None
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, experts, shared))
+    y = torch.full((tokens, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((experts,), dtype=torch.int32, device=dev)
+    try:
+        ws.tune("gemm_tile_rows", tile_rows)
+        ops.megamoe_forward(ws, torch.from_numpy(x_codes).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(x_scales).to(dev),
+                            torch.from_numpy(idx).to(dev), torch.from_numpy(weights).to(dev), w1, s1, w2, s2, experts, 0, experts, y,
+                            counts, intermediate=inter, shared=extra)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+    finally:
+        ws.destroy()
+    xq = mm.mx_dequantize(x_codes, x_scales)
+    shared_weights = (mm.unpack_weight(sp1, ss1), mm.unpack_weight(sp2, ss2)) if shared else ()
+    want = mm.round_bf16(mm.local_reference(xq, idx, weights, mm.unpack_weight(*l1), mm.unpack_weight(*l2), 0, *shared_weights))
+    np.testing.assert_array_equal(counts.cpu().numpy(), np.bincount(idx.ravel(), minlength=experts), err_msg=str(case))
+    assert np.isfinite(got).all(), case
+    err = mm.relative_frobenius(got, want)
+    assert err <= 2e-2, (err, case)
+    norms = np.linalg.norm(want, axis=1)
+    per_token = np.linalg.norm(got - want, axis=1) / np.maximum(norms, 1e-6 * norms.max() + 1e-30)
+    assert per_token.max() <= 6e-2, (per_token.max(), case)
