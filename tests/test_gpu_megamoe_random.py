@@ -19,6 +19,21 @@ def ops():
     return module
 
 
+def _check_per_token(got, want, case):
+    """No single token may carry the error (a wrong row hides in the norm of a large matrix): 6 % of its own norm.
+
+    One exception is part of the arithmetic.  The first GEMM's result is rounded to BF16, SwiGLU's again, and that value
+    to e4m3; where the fp32 sum sits on a BF16 tie the order of the additions decides the rounding, and the next two
+    roundings can carry that one BF16 step into one e4m3 step, up to an eighth of the activation.  A token whose output
+    one activation dominates then moves by up to that much (the shared expert here is drawn from the same stream as the
+    tokens, so its gate row t repeats token t and every token has such an activation).  Hence: nothing above 13 %, and at
+    most one token in 500 above 6 %."""
+    norms = np.linalg.norm(want, axis=1)
+    per_token = np.linalg.norm(got - want, axis=1) / np.maximum(norms, 1e-6 * norms.max() + 1e-30)
+    assert per_token.max() <= 0.13, (per_token.max(), case)
+    assert (per_token > 6e-2).sum() <= max(1, len(per_token) // 500), (np.sort(per_token)[-5:], case)
+
+
 def _draw(seed):
     rng = np.random.default_rng(1000 + seed)
     experts = int(rng.choice([2, 3, 6, 8, 16, 32, 48]))
@@ -49,10 +64,7 @@ def test_forward_at_random_shapes(ops, seed):
     if served.any():
         err = mm.relative_frobenius(got[served], want[served])
         assert err <= 2e-2, (err, case)
-        # no single token may carry the error either (a wrong row hides in the norm of a large matrix)
-        norms = np.linalg.norm(want[served], axis=1)
-        per_token = np.linalg.norm(got[served] - want[served], axis=1) / np.maximum(norms, 1e-6 * norms.max() + 1e-30)
-        assert per_token.max() <= 6e-2, (per_token.max(), case)
+        _check_per_token(got[served], want[served], case)
     other, _ = _run(ops, x_codes, x_scales, l1, l2, idx, weights, experts, begin, local, tile_rows=tile_rows, column_waves=0)
     np.testing.assert_array_equal(got.view(np.uint32), other.view(np.uint32), err_msg=str(case))
 
@@ -111,6 +123,7 @@ def test_forward_with_shared_experts_and_switches_at_random_shapes(ops, seed):
     if served.any():
         err = mm.relative_frobenius(got[served], want[served])
         assert err <= 2e-2, (err, case)
+        _check_per_token(got[served], want[served], case)
 
 
 def _draw_many_tiles(seed):
@@ -125,10 +138,11 @@ def _draw_many_tiles(seed):
     return tokens, hidden, inter, experts, topk, tile_rows, shared
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", list(range(16)) + [304, 525, 690])
 def test_forward_with_more_tiles_than_workgroups(ops, seed):
     """Few experts with thousands of rows each: workgroups walk several tiles of a flat stream, through both grouped GEMM
-    kernels (K a multiple of 512 or not), every tile height, with and without a shared expert."""
+    kernels (K a multiple of 512 or not), every tile height, with and without a shared expert.  Seeds 304, 525 and 690 each
+    hold one token whose dominant activation lands one e4m3 step from the oracle's (see _check_per_token)."""
     import torch
 
     tokens, hidden, inter, experts, topk, tile_rows, shared = _draw_many_tiles(seed)
@@ -165,6 +179,4 @@ def test_forward_with_more_tiles_than_workgroups(ops, seed):
     assert np.isfinite(got).all(), case
     err = mm.relative_frobenius(got, want)
     assert err <= 2e-2, (err, case)
-    norms = np.linalg.norm(want, axis=1)
-    per_token = np.linalg.norm(got - want, axis=1) / np.maximum(norms, 1e-6 * norms.max() + 1e-30)
-    assert per_token.max() <= 6e-2, (per_token.max(), case)
+    _check_per_token(got, want, case)
