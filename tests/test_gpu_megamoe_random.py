@@ -180,3 +180,88 @@ def test_forward_with_more_tiles_than_workgroups(ops, seed):
     err = mm.relative_frobenius(got, want)
     assert err <= 2e-2, (err, case)
     _check_per_token(got, want, case)
+
+
+def _draw_large(seed):
+    rng = np.random.default_rng(7000 + seed)
+    local = int(rng.choice([1, 2, 3, 5, 8, 16, 32]))
+    spread = int(rng.choice([1, 1, 2, 8]))
+    experts = local * spread
+    begin = int(rng.integers(0, spread)) * local
+    topk = int(rng.integers(1, min(8, experts) + 1))
+    tokens = int(np.exp(rng.uniform(np.log(200), np.log(16384))))
+    hidden = 64 * int(rng.choice([rng.integers(16, 129), 8 * rng.integers(2, 17), 4 * rng.integers(4, 33)]))
+    inter = 128 * int(rng.choice([rng.integers(2, 33), 4 * rng.integers(1, 9), 2 * rng.integers(1, 17)]))
+    while local * 2 * inter * hidden > 3_000_000_000:
+        local = max(1, local // 2)
+        experts = local * spread
+        begin = min(begin, experts - local)
+        topk = min(topk, experts)
+    shared = int(rng.choice([0, 0, 0, 1, 2]))
+    zero_fill = int(rng.integers(0, 2))
+    served_only = int(rng.integers(0, 2)) if shared == 0 else 0
+    return tokens, hidden, inter, experts, begin, local, topk, shared, zero_fill, served_only
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_tile_heights_and_kernels_agree_at_large_random_shapes(ops, seed):
+    """Sizes the oracle cannot follow (up to 16 384 tokens, hidden up to 8192, intermediate up to 4096, 32 local experts,
+    masked routes in a third of the draws): a k sum is taken in the same order whatever the tile height and whichever
+    grouped GEMM kernel runs, so the forward must give the same bits at 64, 128 and 192 rows, through the column-wave
+    kernel and the 2 x 2 kernel, and again on a second run; counts against a bincount, every served token written."""
+    import torch
+
+    tokens, hidden, inter, experts, begin, local, topk, shared, zero_fill, served_only = _draw_large(seed)
+    case = dict(tokens=tokens, hidden=hidden, inter=inter, experts=experts, begin=begin, local=local, topk=topk, shared=shared,
+                zero_fill=zero_fill, served_only=served_only)
+    print(case, flush=True)
+    dev = "cuda"
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    x = torch.randint(0, 256, (tokens, hidden), dtype=torch.int16, device=dev, generator=g)
+    x = torch.where((x & 0x7F) == 0x7F, x - 1, x).to(torch.uint8)  # no NaN codes
+    x_scales = torch.randint(125, 130, (tokens, hidden // 32), dtype=torch.uint8, device=dev, generator=g)
+
+    def weights(count, n, k, gate_up):
+        packed = torch.randint(0, 256, (count, n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+        scales = torch.randint(117, 122, (count, n, k // 32), dtype=torch.uint8, device=dev, generator=g)
+        return ops.megamoe_prepare_weights(packed, scales, gate_up)
+
+    w1, s1 = weights(local, 2 * inter, hidden, True)
+    w2, s2 = weights(local, hidden, inter, False)
+    extra = weights(shared, 2 * inter, hidden, True) + weights(shared, hidden, inter, False) if shared else None
+    idx = torch.rand((tokens, experts), device=dev, generator=g).argsort(dim=1)[:, :topk].to(torch.int32).contiguous()
+    if seed % 3 == 0:
+        idx = torch.where(torch.rand((tokens, topk), device=dev, generator=g) < 0.2, torch.full_like(idx, -1), idx)
+    route_weights = torch.rand((tokens, topk), device=dev, generator=g, dtype=torch.float32)
+    sentinel = 3.0
+    first = None
+    for column_waves, tile_rows in [(1, 0), (1, 64), (1, 128), (1, 192), (0, 64), (0, 128), (0, 192), (1, 0)]:
+        ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local, shared))
+        y = torch.full((tokens, hidden), sentinel, dtype=torch.bfloat16, device=dev)
+        counts = torch.empty((local,), dtype=torch.int32, device=dev)
+        try:
+            ws.tune("gemm_tile_rows", tile_rows)
+            ws.tune("gemm_column_waves", column_waves)
+            ws.tune("gemm_zero_fill", zero_fill)
+            ws.tune("megamoe_served_only", served_only)
+            ops.megamoe_forward(ws, x.view(torch.float8_e4m3fn), x_scales, idx, route_weights, w1, s1, w2, s2, experts, begin, local, y,
+                                counts, intermediate=inter, shared=extra)
+            torch.cuda.synchronize()
+        finally:
+            ws.destroy()
+        bits = y.view(torch.int16)
+        if first is None:
+            first = (bits.clone(), counts.clone())
+            mine = (idx >= begin) & (idx < begin + local)
+            assert torch.equal(counts.long(), torch.bincount(idx[mine].long() - begin, minlength=local)), case
+            assert torch.isfinite(y.float()).all(), case
+            served = mine.any(dim=1) | (shared > 0)
+            written = (y != sentinel).any(dim=1)
+            assert bool((written | ~served).all()), (int((served & ~written).sum()), case)
+            if served_only:
+                assert bool((~written | served).all()), case
+        else:
+            differing = (bits != first[0]).any(dim=1).nonzero().flatten()
+            assert differing.numel() == 0, (column_waves, tile_rows, int(differing.numel()), differing[:8].tolist(), case)
+            assert torch.equal(counts, first[1]), (column_waves, tile_rows, case)
