@@ -209,9 +209,27 @@ def test_tile_heights_and_kernels_agree_at_large_random_shapes(ops, seed):
     masked routes in a third of the draws): a k sum is taken in the same order whatever the tile height and whichever
     grouped GEMM kernel runs, so the forward must give the same bits at 64, 128 and 192 rows, through the column-wave
     kernel and the 2 x 2 kernel, and again on a second run; counts against a bincount, every served token written."""
+    _agreement_case(ops, seed, *_draw_large(seed))
+
+
+@pytest.mark.parametrize(
+    "shape",
+    [
+        (65536, 1024, 512, 8, 0, 8, 8, 0, 1, 0),      # the interface's largest batch: 524 288 rows, 2048 per tile column
+        (65536, 2048, 256, 128, 0, 128, 4, 0, 0, 0),  # the most local experts at the largest batch
+        (40000, 8192, 4096, 2, 0, 2, 2, 0, 1, 0),     # the largest matrices: 20 000 rows per expert
+        (30000, 7168, 2048, 4, 2, 2, 3, 2, 0, 0),     # two shared experts beside two routed ones: 60 000 shared rows
+        (50000, 1088, 384, 16, 8, 8, 8, 0, 0, 1),     # both sizes padded, half the experts local, served-only
+    ],
+    ids=lambda shape: "x".join(str(v) for v in shape),
+)
+def test_tile_heights_and_kernels_agree_at_the_interfaces_largest_sizes(ops, shape):
+    _agreement_case(ops, 12345, *shape)
+
+
+def _agreement_case(ops, seed, tokens, hidden, inter, experts, begin, local, topk, shared, zero_fill, served_only):
     import torch
 
-    tokens, hidden, inter, experts, begin, local, topk, shared, zero_fill, served_only = _draw_large(seed)
     case = dict(tokens=tokens, hidden=hidden, inter=inter, experts=experts, begin=begin, local=local, topk=topk, shared=shared,
                 zero_fill=zero_fill, served_only=served_only)
     print(case, flush=True)
