@@ -283,3 +283,120 @@ def _agreement_case(ops, seed, tokens, hidden, inter, experts, begin, local, top
             differing = (bits != first[0]).any(dim=1).nonzero().flatten()
             assert differing.numel() == 0, (column_waves, tile_rows, int(differing.numel()), differing[:8].tolist(), case)
             assert torch.equal(counts, first[1]), (column_waves, tile_rows, case)
+
+
+def _torch_reference(x_codes, x_scales, idx, route_weights, raw1, raw2, begin, local, shared_raw=None):
+    """The oracle's arithmetic (oracle.megamoe.expert_forward / local_reference) in torch on the device, for sizes NumPy on
+    the host cannot follow: dense fp32 operands expert by expert, fp32 matrix products, the same roundings.  raw1 / raw2:
+    (packed [E,N,K/2] uint8, scales [E,N,K/32] uint8) before preparation."""
+    import torch
+
+    dev = x_codes.device
+    e2m1 = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], device=dev)
+    e2m1 = torch.cat([e2m1, -e2m1])
+
+    def dense(packed, scales):  # one expert: [N, K/2], [N, K/32] -> fp32 [N, K]
+        n, half = packed.shape
+        values = torch.stack((e2m1[(packed & 15).long()], e2m1[(packed >> 4).long()]), dim=-1).reshape(n, half * 2)
+        factor = torch.exp2(scales.float() - 127.0)
+        return (values.view(n, -1, 32) * factor[..., None]).reshape(n, half * 2)
+
+    def quantised(act):  # oracle.megamoe.mx_quantize + mx_dequantize on BF16-representable fp32 [m, I]
+        m, width = act.shape
+        blocks = act.view(m, width // 32, 32)
+        amax = blocks.abs().amax(dim=-1).clamp_min(2.0**-119)
+        byte = ((amax.view(torch.int32) >> 23) - 8).clamp_min(0)
+        shift = 127 - byte  # applied in two steps so that neither factor leaves the fp32 range
+        scaled = blocks * torch.exp2((shift // 2).float())[..., None]
+        scaled = scaled * torch.exp2((shift - shift // 2).float())[..., None]
+        codes = scaled.clamp(-448.0, 448.0).to(torch.float8_e4m3fn).float()
+        return (codes * torch.exp2((byte - 127).float())[..., None]).reshape(m, width)
+
+    def expert(x, w1, w2):
+        inter = w1.shape[0] // 2
+        first = (x @ w1.T).bfloat16().float()
+        gate, up = first[:, :inter], first[:, inter:]
+        act = (gate / (1 + torch.exp((-gate).clamp(-80, 80))) * up).bfloat16().float()
+        return (quantised(act) @ w2.T).bfloat16().float()
+
+    xq = (x_codes.view(torch.float8_e4m3fn).float().view(x_codes.shape[0], -1, 32)
+          * torch.exp2(x_scales.float() - 127.0)[..., None]).reshape(x_codes.shape)
+    result = torch.zeros_like(xq)
+    for e in range(local):
+        token, slot = (idx == begin + e).nonzero(as_tuple=True)
+        if token.numel():
+            out = expert(xq[token], dense(raw1[0][e], raw1[1][e]), dense(raw2[0][e], raw2[1][e]))
+            result.index_put_((token,), out * route_weights[token, slot, None], accumulate=True)
+    if shared_raw is not None:
+        for e in range(shared_raw[0][0].shape[0]):
+            result += expert(xq, dense(shared_raw[0][0][e], shared_raw[0][1][e]), dense(shared_raw[1][0][e], shared_raw[1][1][e]))
+    return result.bfloat16()
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_forward_against_a_device_side_restatement_at_large_random_shapes(ops, seed):
+    """Values, not only agreement between kernels, at the sizes of _draw_large: the forward against the oracle's
+    arithmetic restated in torch on the device (checked against the NumPy oracle itself on a small case below)."""
+    import torch
+
+    tokens, hidden, inter, experts, begin, local, topk, shared, zero_fill, served_only = _draw_large(500 + seed)
+    tokens = min(tokens, 6000)  # dense fp32 weights and activations of one expert at a time stay within a few GB
+    case = dict(tokens=tokens, hidden=hidden, inter=inter, experts=experts, begin=begin, local=local, topk=topk, shared=shared)
+    print(case, flush=True)
+    dev = "cuda"
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    # codes of moderate size (sign, exponent field 4..10, any mantissa) so that no product overflows BF16 on the way
+    x = (torch.randint(0, 2, (tokens, hidden), device=dev, generator=g) << 7 | torch.randint(4, 11, (tokens, hidden), device=dev, generator=g) << 3
+         | torch.randint(0, 8, (tokens, hidden), device=dev, generator=g)).to(torch.uint8)
+    x_scales = torch.randint(125, 130, (tokens, hidden // 32), dtype=torch.uint8, device=dev, generator=g)
+
+    def raw(count, n, k):
+        return (torch.randint(0, 256, (count, n, k // 2), dtype=torch.uint8, device=dev, generator=g),
+                torch.randint(117, 122, (count, n, k // 32), dtype=torch.uint8, device=dev, generator=g))
+
+    raw1, raw2 = raw(local, 2 * inter, hidden), raw(local, hidden, inter)
+    w1, s1 = ops.megamoe_prepare_weights(*raw1, True)
+    w2, s2 = ops.megamoe_prepare_weights(*raw2, False)
+    extra = shared_raw = None
+    if shared:
+        shared_raw = (raw(shared, 2 * inter, hidden), raw(shared, hidden, inter))
+        extra = ops.megamoe_prepare_weights(*shared_raw[0], True) + ops.megamoe_prepare_weights(*shared_raw[1], False)
+    idx = torch.rand((tokens, experts), device=dev, generator=g).argsort(dim=1)[:, :topk].to(torch.int32).contiguous()
+    route_weights = torch.rand((tokens, topk), device=dev, generator=g, dtype=torch.float32)
+    ws = ops.Workspace(ops.megamoe_workspace_bytes(tokens, topk, hidden, inter, local, shared))
+    y = torch.full((tokens, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty((local,), dtype=torch.int32, device=dev)
+    try:
+        ops.megamoe_forward(ws, x.view(torch.float8_e4m3fn), x_scales, idx, route_weights, w1, s1, w2, s2, experts, begin, local, y,
+                            counts, intermediate=inter, shared=extra)
+        torch.cuda.synchronize()
+    finally:
+        ws.destroy()
+    want = _torch_reference(x, x_scales, idx, route_weights, raw1, raw2, begin, local, shared_raw)
+    assert torch.isfinite(y.float()).all() and torch.isfinite(want.float()).all(), case
+    served = ((idx >= begin) & (idx < begin + local)).any(dim=1) | (shared > 0)
+    assert not y[~served].any(), case
+    if served.any():
+        got64, want64 = y[served].double(), want[served].double()
+        err = float((got64 - want64).norm() / want64.norm().clamp_min(1e-30))
+        assert err <= 2e-2, (err, case)
+        _check_per_token(y[served].float().cpu().numpy(), want[served].float().cpu().numpy(), case)
+
+
+def test_device_side_restatement_is_the_numpy_oracle(ops):
+    import torch
+
+    tokens, hidden, inter, experts, begin, local, topk = 130, 512, 384, 6, 1, 4, 3
+    x_codes, x_scales, l1, l2, idx, weights = _make_problem(tokens, hidden, inter, experts, begin, local, topk, seed=11)
+    want = _oracle(x_codes, x_scales, l1, l2, idx, weights, begin)
+    dev = "cuda"
+
+    def on_device(pair, count, n):
+        return torch.from_numpy(pair[0]).to(dev), torch.from_numpy(pair[1]).reshape(count, n, -1).to(dev)
+
+    got = _torch_reference(torch.from_numpy(x_codes).to(dev), torch.from_numpy(x_scales).to(dev), torch.from_numpy(idx).to(dev),
+                           torch.from_numpy(weights).to(dev), on_device(l1, local, 2 * inter), on_device(l2, local, hidden), begin, local)
+    got = got.float().cpu().numpy()
+    # the two differ only where the order of fp32 additions moves a rounding
+    assert mm.relative_frobenius(got, want) <= 2e-3
