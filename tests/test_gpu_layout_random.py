@@ -82,3 +82,30 @@ def test_layout_forms_at_random_shapes(ops, ws, seed):
         assert host_rows == want["num_rows"], case
         _compare(plan, want, case)
         np.testing.assert_array_equal(bf16_bits(out[:host_rows]), olayout.expand_rows(bf16_bits(x), want["row_to_route"], topk), err_msg=str(case))
+
+
+@pytest.mark.parametrize(
+    "experts,begin,local,tokens,topk",
+    [
+        (16384, 16256, 128, 4096, 32),  # the reference's largest expert count, the last rank's range, top-k 32
+        (16384, 0, 1024, 20000, 8),     # the most local experts the layout takes
+        (65536, 65000, 536, 3000, 9),   # expert numbers beyond 16 bits
+        (16384, 8000, 1, 65536, 8),     # a single local expert at the largest batch: one long run of rows
+    ],
+)
+def test_layout_at_the_largest_expert_counts(ops, ws, experts, begin, local, tokens, topk):
+    rng = np.random.default_rng(experts + tokens)
+    ids = rng.integers(-1, experts, size=(tokens, topk)).astype(np.int64)
+    mine = rng.random((tokens, topk)) < 0.4  # (uniform routing alone would leave the local range almost empty)
+    ids[mine] = rng.integers(begin, begin + local, size=int(mine.sum()))
+    want = olayout.layout(ids, experts, begin, local)
+    assert want["num_rows"] > tokens
+    idx = torch.from_numpy(ids).cuda()
+    case = dict(experts=experts, begin=begin, local=local, tokens=tokens, topk=topk)
+    try:
+        for one_launch in (1, 0):
+            ws.tune("layout_one_launch", one_launch)
+            _compare(ops.layout(ws, idx, experts, begin, local), want, case)
+    finally:
+        ws.tune("layout_one_launch", 1)
+    _compare(_layout_static(_lib.load(), idx, experts, begin, local), want, case)
