@@ -28,17 +28,12 @@ struct GemmRing {
 // its item loop, the asynchronous requests per thread and item (activation copies + four weight loads; a span's first item
 // adds two scale copies, a tile's first item the fetch of the next tile's gather indices), and what may still be in flight at
 // an item's wait such that the NEXT item's operands have arrived: the requests of the two items after it.
-// The epilogue's stores count in the same counter as the loads and are acknowledged late, so a wait right behind them would
-// make the loads drain as well (the counter cannot tell them apart).  Hence the wait at a tile's end, in front of the
-// stores: everything but the last item's requests has arrived (kTileEndWait), i.e. the operands of the next tile's first
-// THREE items, and the first kNoWaitItems items of every tile wait for nothing but the barrier.  The prologue ends the same way.
 template <int RT>
 struct ColumnRing {
     static constexpr int kStages = 4;
     static constexpr int kRequests = 2 * RT + 4;
     static constexpr int kWait = 2 * kRequests;
-    static constexpr int kTileEndWait = kRequests;
-    static constexpr int kNoWaitItems = 2;
+    static constexpr int kPrologueWait = (kStages - 1) * kRequests;  // behind the prologue's four items: item 0 has arrived
 };
 
 // When the copy cursor may trust the next tile's gather indices.  They are fetched (asynchronously, into LDS)

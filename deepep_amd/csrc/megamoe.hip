@@ -401,24 +401,6 @@ __device__ __forceinline__ void wait_copies_then_barrier()
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
-// The same where an earlier, stronger wait may already have covered the operands: with first_group_kt == 0 (the item belongs
-// to a tile's first four) only the wave's own LDS reads and the barrier remain.  The branch sits inside the statement, so
-// the compiler sees straight-line code (see mfma_fp8_fp4 on branches around MFMA statements).
-template <int kOutstanding>
-__device__ __forceinline__ void wait_copies_unless_covered_then_barrier(int first_group_kt)
-{
-    asm volatile("s_cmp_eq_u32 %1, 0\n\ts_cbranch_scc1 .Lcovered_%=\n\ts_waitcnt vmcnt(%0)\n.Lcovered_%=:\n\t"
-                 "s_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding),
-                 "s"(__builtin_amdgcn_readfirstlane(first_group_kt))
-                 : "memory", "scc");
-}
-// The wait alone: the barrier of the item that follows makes it the workgroup's.
-template <int kOutstanding>
-__device__ __forceinline__ void wait_copies()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kOutstanding) : "memory");
-}
-
 // One scaled MFMA (FP8 A, FP4 B) as a volatile asm statement: volatile statements keep their source order,
 // which is what lets the copies and the barrier be placed between individual MFMAs (builtin MFMAs are pure
 // and the compiler gathers them into bursts).  kSecond selects scale bytes 2|3 of A and byte 1 of B.
@@ -1350,7 +1332,7 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
     request_item(std::integral_constant<int, 1>{});
     request_item(std::integral_constant<int, 2>{});
     request_item(std::integral_constant<int, 3>{});
-    wait_copies_then_barrier<Cfg::kTileEndWait>();  // items 0..2 and the span have arrived (as at every tile's end)
+    wait_copies_then_barrier<Cfg::kPrologueWait>();  // item 0 and its span have arrived
     int read_span = 0;
     read_col_scales();
 #pragma unroll
@@ -1410,10 +1392,7 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
             if constexpr (kN == kBarrierAt) {
                 // The next item's operands have arrived once each thread has at most the requests of the two items after it
                 // in flight; past the barrier every wave has also read the last fragment of this item's stage.
-                // (kt is the k tile of the group's first item: 0 in a tile's first group, whose first items the wait at the
-                // previous tile's end has covered)
-                if constexpr (kPos < Cfg::kNoWaitItems) wait_copies_unless_covered_then_barrier<Cfg::kWait>(kt);
-                else wait_copies_then_barrier<Cfg::kWait>();
+                wait_copies_then_barrier<Cfg::kWait>();
 #pragma unroll
                 for (int i = 0; i < kRowTiles; ++i) copy_from[i] = my_offsets[i * kGemmThreads];
                 if (kPos == 0) request_span();
@@ -1451,7 +1430,6 @@ __global__ __launch_bounds__(kGemmThreads, ColCfg<RT>::kWorkgroupsPerCu) void gr
         kt += 4;
         if (__builtin_expect(kt == ktiles, 0)) {
             settle_accumulators();
-            wait_copies<Cfg::kTileEndWait>();  // in front of the epilogue's stores (see ColumnRing)
 #pragma unroll
             for (int i = 0; i < kRowTiles; ++i)
 #pragma unroll
@@ -1700,12 +1678,10 @@ bool replay_workgroup(int my_tiles, int ktiles, int epilogue_stores, bool drain_
 
 // The same replay for the column-wave kernel: the prologue requests items 0..3 (each: its span's scales and the next tile's
 // gather indices where it opens a span / a tile, its activation copies, its weight loads), then waits; every item's body
-// waits (kWait + slack in flight; not the first kNoWaitItems of a tile), then requests the item four ahead in the same order;
-// tiles end behind every ktiles-th item with the tile-end wait (kTileEndWait + slack) and then the epilogue's stores.
-// slack > 0 replays a kernel whose waits are laxer than the real ones, more_no_wait_items > 0 one whose tiles start with
-// more items that do not wait than the wait at a tile's end covers.
+// waits (kWait + slack in flight), then requests the item four ahead in the same order; tiles end behind every ktiles-th
+// item with the epilogue's stores.  slack > 0 replays a kernel whose wait is laxer than the real one.
 template <int RT>
-bool replay_column_waves(int my_tiles, int ktiles, int epilogue_stores, int slack, int more_no_wait_items, ScheduleFault* fault)
+bool replay_column_waves(int my_tiles, int ktiles, int epilogue_stores, int slack, ScheduleFault* fault)
 {
     using Ring = ColumnRing<RT>;
     const long long n_items = static_cast<long long>(my_tiles) * ktiles;
@@ -1764,17 +1740,16 @@ bool replay_column_waves(int my_tiles, int ktiles, int epilogue_stores, int slac
         request_item();
         advance(true, -1);
     }
-    wait(Ring::kTileEndWait + slack);
+    wait(Ring::kPrologueWait);
     check_item(0);
     int kt = 0;
     for (long long item = 0; item < n_items; ++item) {
-        if (kt >= Ring::kNoWaitItems + more_no_wait_items) wait(Ring::kWait + slack);  // (a tile's first items rely on the wait at the previous tile's end)
+        wait(Ring::kWait + slack);
         check_item(item + 1);  // its first fragments leave LDS during this item's second k step, its weights right after
         body = item;
         request_item();
         advance(false, static_cast<int>(item));
         if (++kt == ktiles) {
-            wait(Ring::kTileEndWait + slack);
             issued += epilogue_stores;
             kt = 0;
         }
@@ -1847,11 +1822,9 @@ int dpep_megamoe_schedule_check_column_waves(int tile_rows, int tiles_per_workgr
     DPEP_REQUIRE(tiles_per_workgroup >= 0 && ktiles >= 4 && ktiles % 4 == 0 && epilogue_stores >= 0 && slack >= 0,
                  "schedule_check: bad arguments (the column-wave kernel takes k tiles in fours)");
     ScheduleFault fault = {0, 0};
-    const int more = slack >> 16;
-    slack &= 0xffff;
-    const bool ok = tile_rows == 64    ? replay_column_waves<1>(tiles_per_workgroup, ktiles, epilogue_stores, slack, more, &fault)
-                    : tile_rows == 128 ? replay_column_waves<2>(tiles_per_workgroup, ktiles, epilogue_stores, slack, more, &fault)
-                                       : replay_column_waves<3>(tiles_per_workgroup, ktiles, epilogue_stores, slack, more, &fault);
+    const bool ok = tile_rows == 64    ? replay_column_waves<1>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault)
+                    : tile_rows == 128 ? replay_column_waves<2>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault)
+                                       : replay_column_waves<3>(tiles_per_workgroup, ktiles, epilogue_stores, slack, &fault);
     if (!ok && fault.what == 3)
         return fail(DPEP_EINVAL, "schedule_check: a span's scales are overwritten while they are still being read (behind item %d)",
                     fault.item);

@@ -208,10 +208,8 @@ int dpep_mx_quant(const void* x, int rows, int hidden, void* codes, uint8_t* sca
  * Returns 0, or DPEP_EINVAL with the first violation in dpep_last_error(). */
 int dpep_megamoe_schedule_check(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int without_drain);
 /* The same check for the kernel that runs where K is a multiple of 512 (its waves split the tile's columns and load their
- * weights straight into registers; k tiles come in fours; a wait at every tile's end, in front of the epilogue's stores,
- * covers the next tile's first items, which do not wait themselves).  slack: bits 0..15 = operations the replayed waits
- * allow in flight beyond the kernel's own counts, bits 16.. = items at a tile's start that do not wait, beyond the kernel's
- * two: with either above zero the check has to fail, which is how the tests know that it can. */
+ * weights straight into registers; k tiles come in fours).  slack = operations the replayed wait allows in flight beyond
+ * the kernel's own count: with slack > 0 the check has to fail, which is how the tests know that it can. */
 int dpep_megamoe_schedule_check_column_waves(int tile_rows, int tiles_per_workgroup, int ktiles, int epilogue_stores, int slack);
 
 /* Bytes of workspace dpep_megamoe_forward needs (buffer_size(), experiments/megamoe/csrc/forward.cpp:480).

@@ -67,17 +67,6 @@ def test_column_wave_replay_catches_a_wait_that_is_too_lax(tile_rows, requests):
         assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, 12, 0) == 0
 
 
-@pytest.mark.parametrize("tile_rows", [64, 128, 192])
-def test_column_wave_replay_catches_a_tile_start_that_waits_too_late(tile_rows):
-    """The wait at a tile's end (in front of the epilogue's stores) covers the operands of the next tile's first three items,
-    so its first two items need no wait of their own; a third would read operands that nothing covers."""
-    lib = _lib.load()
-    for ktiles, tiles in itertools.product((4, 8, 16, 56), (1, 2, 24)):
-        assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, 24, 1 << 16) == -1, (ktiles, tiles)
-        assert b"operands" in lib.dpep_last_error()
-        assert lib.dpep_megamoe_schedule_check_column_waves(tile_rows, tiles, ktiles, 24, 0) == 0
-
-
 @pytest.mark.parametrize("tile_rows,ahead", [(64, 5), (128, 4), (192, 3)])
 def test_replay_catches_scale_slots_reused_too_early(tile_rows, ahead):
     """The scales of a span of k tiles sit in a ring of LDS slots; the replay also checks that a slot is refilled only
